@@ -1,0 +1,100 @@
+/* C ABI of libbf16n_hip.so — the drop-in boundary of the BF16N hot path on MI355X (gfx950).
+ *
+ * Plain pointers and sizes only.  Every function returns a status: BF16N_OK, BF16N_EINVAL (the reference throws
+ * std::invalid_argument with the same message) or BF16N_ERUNTIME (std::runtime_error: HIP errors, encoder invariants);
+ * bf16n_last_error() gives the message of the calling thread's last failure.  `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  Launchers only enqueue kernels: no allocation, no host synchronisation, no
+ * environment reads, so they can be captured into HIP graphs after bf16n_init().  All device pointers are the caller's.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the reference repository root).
+ * The C++ API of the reference (namespace bf16n, core/include/bf16n/{encode,policy,launch}.h) is provided on top of
+ * this file by the headers under include/bf16n/ with the same names, argument meaning and exceptions.
+ */
+#ifndef BF16N_C_H
+#define BF16N_C_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { BF16N_OK = 0, BF16N_EINVAL = 1, BF16N_ERUNTIME = 2 };
+enum { BF16N_FMT_NIBBLE = 1, BF16N_FMT_HUFFMAN = 2, BF16N_FMT_HUFPAIR = 3 };
+enum { BF16N_FLAG_CHUNK_MAJOR = 1, BF16N_FLAG_FRAG_ORDER = 2, BF16N_FLAG_WAVE64 = 4 };
+enum { BF16N_ENGINE_LLAMA = 0, BF16N_ENGINE_VLLM = 1, BF16N_ENGINE_MI355X = 2 };
+enum { BF16N_MODE_HYBRID = 0, BF16N_MODE_HUFFMAN = 1, BF16N_MODE_NIBBLE = 2 };
+
+const char * bf16n_last_error(void);
+
+/* ---- host encoder: bf16n::encode, core/include/bf16n/encode.h:12-26, core/src/encode.cpp:443-526 ----------------- */
+typedef struct bf16n_encoded bf16n_encoded; /* owns plane + aux (struct encoded, encode.h:12-17) */
+/* w: rows x K BF16 bit patterns, row-major (host).  flags: BF16N_FLAG_* layout bits (chunk_major / frag_order arguments
+ * of the reference; FRAG_ORDER is rejected with EINVAL, WAVE64 is this build's wave64 stream layout). */
+int bf16n_encode(const uint16_t * w, int64_t rows, int64_t K, int format, int R, uint32_t flags, bf16n_encoded ** out);
+const uint8_t * bf16n_encoded_plane(const bf16n_encoded * e, uint64_t * bytes);
+const uint8_t * bf16n_encoded_aux(const bf16n_encoded * e, uint64_t * bytes);
+int  bf16n_encoded_format(const bf16n_encoded * e); /* format actually produced (HUFPAIR may fall back to HUFFMAN) */
+int  bf16n_encoded_R(const bf16n_encoded * e);      /* rows per unit, 0 for NIBBLE */
+void bf16n_encoded_free(bf16n_encoded * e);
+/* worker threads of the encoder (the reference fixes min(12, cores), encode.cpp:27); 0 = default min(16, cores) */
+void bf16n_set_encode_threads(int n);
+
+/* ---- shape policy: bf16n::choose, core/include/bf16n/policy.h:12-38, core/src/policy.cpp:45-69 -------------------- */
+/* out[5] = {format, R, chunk_major, frag_order, wave64}.  Returns 1 if a choice was made, 0 if the shape stays BF16
+ * (std::nullopt).  Never fails.  engine MI355X: the reference's llama rules with unit sizes chosen for 256 CUs of
+ * wave64 and the wave64 stream layout where the shape allows it. */
+int bf16n_choose(int64_t rows, int64_t K, int64_t n_matrices, int engine, int mode, int64_t dense_min, int expert,
+                 int dense_frag_order, int * out);
+
+/* ---- device view of one encoded matrix: struct weight, core/include/bf16n/launch.h:15-25 --------------------------- */
+typedef struct bf16n_weight {
+    const uint8_t * plane; /* device, 16-byte aligned */
+    const uint8_t * aux;   /* device, 16-byte aligned */
+    int32_t  format, R;
+    int64_t  K, rows;
+    uint32_t flags;        /* BF16N_FLAG_* from the aux header (cm / fo booleans of the reference) */
+    uint32_t pad_;
+    uint64_t off_a, off_b, off_c, off_d;
+} bf16n_weight;
+
+/* struct mmv_args, core/include/bf16n/launch.h:27-44: same fields and meaning (signed strides in bytes) */
+typedef struct bf16n_mmv_args {
+    const void * x; void * y; const void * ids;
+    int64_t x_tok, y_tok, ids_s0, ids_s1, x_slot, y_slot;
+    int64_t rows_per_matrix, row0, nrows;
+    int32_t ncols, n_used, x_per_slot;
+    uint8_t x_bf16, y_bf16, pad_[2];
+} bf16n_mmv_args;
+
+/* ---- launchers: core/include/bf16n/launch.h:46-83, core/src/launch.cu ------------------------------------------------ */
+int bf16n_init(void);                 /* init(), launch.h:47, launch.cu:270-306: once per process, before graph capture */
+int bf16n_cu_count(int * out);        /* sm_count(), launch.h:48 */
+int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, int multi_col); /* mmv, launch.h:52, launch.cu:313-325 */
+int bf16n_mmv_glu(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream);            /* mmv_glu merged [gate;up], launch.h:55, launch.cu:327-339 */
+int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf16n_mmv_args * a, void * stream); /* mmv_glu(gate, up), launch.h:61, launch.cu:341-365 */
+int bf16n_dequant(const bf16n_weight * w, int64_t row0, int64_t nrows, uint16_t * out, void * stream); /* dequant, launch.h:63, launch.cu:367-402 */
+int bf16n_get_rows(const bf16n_weight * w, const void * ids, int64_t ids_s0, int64_t n, void * dst, int dst_bf16,
+                   int64_t dst_s1, void * stream, int64_t row0);                                /* get_rows, launch.h:68-69, launch.cu:404-443 */
+int bf16n_mm_ids_supported(const bf16n_weight * w, const bf16n_weight * up);                    /* launch.h:74, launch.cu:446-456; 1/0 */
+int bf16n_mm_ids_route(const void * ids, int ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst,
+                       int32_t * bounds, int n_experts, int n_tok, int n_used, int nchannels_y, int sis1, void * stream); /* launch.h:75-76, launch.cu:458-471, mmid_helper.cu */
+int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row,
+                 const int32_t * ids_src1, const int32_t * ids_dst, const int32_t * bounds, void * dst, int dst_bf16,
+                 int64_t dst_col, int n_experts, int n_tok, int n_used, void * stream);          /* launch.h:77-79, launch.cu:473-535 */
+int bf16n_moe_combine(const float * ys, const void * w, int w_bf16, void * y, int y_bf16, int n_tok, int n_used,
+                      int64_t n, void * stream);                                                /* launch.h:82-83, launch.cu:562-572 */
+int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * stream);       /* launch.h:85, launch.cu:574-582 */
+
+/* Router softmax + top-k on the device, so that a whole MoE decode step can be captured into one HIP graph.  The
+ * reference leaves this to the engines (vllm_bf16n/moe.py:62-67 receives topk_weights/topk_ids); it has no core
+ * counterpart.  logits: n_tok x n_experts FP32 (row stride in elements); ids: n_tok x k int32; weights: n_tok x k FP32,
+ * softmax probabilities of the k largest logits (ties: lower index), renormalised to sum 1 when renorm != 0. */
+int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
+                      int32_t * ids, float * weights, void * stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

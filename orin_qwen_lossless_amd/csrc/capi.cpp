@@ -1,0 +1,336 @@
+// C ABI of libbf16n_hip.so (include/bf16n_c.h): argument checks, dispatch and error reporting.  Contract checks and
+// messages follow the reference launchers (core/src/launch.cu:261-582) so that callers and tests written against the
+// reference see the same failures.  This file and the .hip files are the only places that call HIP.
+#include "bf16n_c.h"
+
+#include "encode_impl.h"
+#include "launchers.h"
+
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+
+using namespace bf16n;
+
+struct bf16n_encoded {
+    impl::encoded_buffers b;
+};
+
+namespace {
+
+thread_local std::string g_error;
+
+int g_cus = 0;
+int g_lds_max = 0;
+std::once_flag g_once;
+
+void require(bool cond, const char * msg) {
+    if (!cond) {
+        throw std::invalid_argument(std::string("bf16n: ") + msg);
+    }
+}
+
+void hip_check(hipError_t e, const char * what) {
+    if (e != hipSuccess) {
+        throw std::runtime_error(std::string("bf16n: HIP error ") + hipGetErrorString(e) + " in " + what);
+    }
+}
+
+void ensure_init() {
+    std::call_once(g_once, [] {
+        int dev = 0;
+        hip_check(hipGetDevice(&dev), "hipGetDevice");
+        hip_check(hipDeviceGetAttribute(&g_cus, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute");
+        hip_check(hipDeviceGetAttribute(&g_lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev), "hipDeviceGetAttribute");
+        dev::w64_init();
+    });
+}
+
+template <typename F>
+int guarded(F && f) {
+    try {
+        f();
+        return BF16N_OK;
+    } catch (const std::invalid_argument & e) {
+        g_error = e.what();
+        return BF16N_EINVAL;
+    } catch (const std::exception & e) {
+        g_error = e.what();
+        return BF16N_ERUNTIME;
+    }
+}
+
+// launch.cu:261-268
+void check_weight(const bf16n_weight & w) {
+    require(w.K % 512 == 0 && w.K >= 512 && w.K <= K_MAX, "K must be a multiple of 512 in [512, 4096]");
+    require(w.format == FMT_NIBBLE || w.format == FMT_HUFFMAN || w.format == FMT_HUFPAIR, "unknown format");
+    require(w.format == FMT_NIBBLE || (w.R > 0 && w.rows % w.R == 0), "rows must be a multiple of R");
+    require(!(w.flags & FLAG_CHUNK_MAJOR) || w.format == FMT_HUFPAIR, "chunk-major units exist only for HUFPAIR");
+    require(!(w.flags & FLAG_FRAG_ORDER), "fragment-order weights are not supported by the MI355X build");
+    require(!(w.flags & FLAG_WAVE64) || (w.format == FMT_HUFPAIR && !(w.flags & FLAG_CHUNK_MAJOR)),
+            "the wave64 layout exists only for row-major HUFPAIR");
+    require(!(w.flags & ~(FLAG_CHUNK_MAJOR | FLAG_FRAG_ORDER | FLAG_WAVE64)), "unknown layout flags");
+}
+
+bool is_w64(const bf16n_weight & w) { return (w.flags & FLAG_WAVE64) != 0; }
+
+dev::cols make_cols(const bf16n_mmv_args & a) { // launch.cu:69-84
+    dev::cols p = {};
+    p.x = (const char *) a.x;
+    p.y = (char *) a.y;
+    p.x_tok = a.x_tok; p.y_tok = a.y_tok;
+    p.ids = (const char *) a.ids;
+    p.ids_s0 = a.ids_s0; p.ids_s1 = a.ids_s1;
+    p.n_used = a.ids ? a.n_used : 1;
+    p.x_per_slot = a.x_per_slot > 0 ? a.x_per_slot : 1;
+    p.x_slot = a.x_slot; p.y_slot = a.y_slot;
+    p.rows_per_matrix = a.rows_per_matrix;
+    p.row0 = a.row0;
+    p.nrows = a.nrows;
+    p.y_bf16 = a.y_bf16 != 0;
+    return p;
+}
+
+void launch_check(const char * what) { hip_check(hipGetLastError(), what); }
+
+} // namespace
+
+extern "C" {
+
+const char * bf16n_last_error(void) { return g_error.c_str(); }
+
+// ---------------------------------------------------------------- encoder / policy
+
+int bf16n_encode(const uint16_t * w, int64_t rows, int64_t K, int format, int R, uint32_t flags, bf16n_encoded ** out) {
+    return guarded([&] {
+        require(out != nullptr, "encode: null output");
+        *out = nullptr;
+        auto * e = new bf16n_encoded;
+        try {
+            e->b = impl::encode(w, rows, K, format, R, flags);
+        } catch (...) {
+            delete e;
+            throw;
+        }
+        *out = e;
+    });
+}
+
+const uint8_t * bf16n_encoded_plane(const bf16n_encoded * e, uint64_t * bytes) {
+    if (bytes) {
+        *bytes = e->b.plane.size();
+    }
+    return e->b.plane.data();
+}
+const uint8_t * bf16n_encoded_aux(const bf16n_encoded * e, uint64_t * bytes) {
+    if (bytes) {
+        *bytes = e->b.aux.size();
+    }
+    return e->b.aux.data();
+}
+int bf16n_encoded_format(const bf16n_encoded * e) { return e->b.format; }
+int bf16n_encoded_R(const bf16n_encoded * e) { return e->b.R; }
+void bf16n_encoded_free(bf16n_encoded * e) { delete e; }
+void bf16n_set_encode_threads(int n) { impl::set_threads(n); }
+
+int bf16n_choose(int64_t rows, int64_t K, int64_t n_matrices, int engine, int mode, int64_t dense_min, int expert,
+                 int dense_frag_order, int * out) {
+    impl::choice c;
+    if (!impl::choose(rows, K, n_matrices, engine, mode, dense_min, expert != 0, dense_frag_order != 0, c)) {
+        return 0;
+    }
+    out[0] = c.format; out[1] = c.R; out[2] = c.chunk_major; out[3] = c.frag_order; out[4] = c.wave64;
+    return 1;
+}
+
+// ---------------------------------------------------------------- launchers
+
+int bf16n_init(void) {
+    return guarded([] { ensure_init(); });
+}
+
+int bf16n_cu_count(int * out) {
+    return guarded([&] {
+        ensure_init();
+        *out = g_cus;
+    });
+}
+
+// launch.cu:313-325
+int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, int multi_col) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(a->ncols > 0 && a->ncols <= 65535, "ncols out of range");
+        require(w->format == FMT_NIBBLE || (a->nrows % w->R == 0 && a->row0 % w->R == 0 && a->rows_per_matrix % w->R == 0),
+                "rows of a product must be whole units");
+        if (a->nrows == 0) {
+            return;
+        }
+        const dev::cols p = make_cols(*a);
+        if (is_w64(*w)) {
+            require(dev::w64_mmv_supported(*w, a->x_bf16 != 0), "no wave64 GEMV kernel for this K / R (K in {512, 1024, 2048, 4096})");
+            dev::launch_w64_mmv(*w, p, a->ncols, a->x_bf16 != 0, multi_col != 0, g_cus, (hipStream_t) stream);
+        } else {
+            dev::launch_compat_mmv(*w, nullptr, 0, p, a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
+        }
+        launch_check("mmv");
+    });
+}
+
+// launch.cu:327-339
+int bf16n_mmv_glu(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(w->format == FMT_NIBBLE, "mmv_glu supports NIBBLE matrices only");
+        require(a->rows_per_matrix == 2 * a->nrows, "mmv_glu: rows per matrix must be [gate; up] of nrows each");
+        require(a->ncols > 0 && a->ncols <= 65535, "ncols out of range");
+        if (a->nrows == 0) {
+            return;
+        }
+        dev::launch_compat_mmv(*w, nullptr, 1, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
+        launch_check("mmv_glu");
+    });
+}
+
+// launch.cu:341-365
+int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf16n_mmv_args * a, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*gate);
+        check_weight(*up);
+        require(gate->format == up->format && gate->K == up->K, "mmv_glu: gate/up format and K must match");
+        require(gate->rows == up->rows, "mmv_glu: gate/up row counts must match");
+        require(a->row0 >= 0 && a->nrows >= 0 && a->row0 <= gate->rows && a->nrows <= gate->rows - a->row0,
+                "mmv_glu: product rows out of range");
+        require(!(gate->flags & FLAG_CHUNK_MAJOR) && !(up->flags & FLAG_CHUNK_MAJOR),
+                "mmv_glu: chunk-major weights require separate mmv launches");
+        require(!is_w64(*gate) && !is_w64(*up), "mmv_glu: wave64 weights require separate mmv launches");
+        require(gate->format == FMT_NIBBLE || gate->R == up->R, "mmv_glu: gate/up R must match");
+        require(a->ncols > 0 && a->ncols <= 65535, "ncols out of range");
+        require(gate->format == FMT_NIBBLE || (a->nrows % gate->R == 0 && a->row0 % gate->R == 0 && a->rows_per_matrix % gate->R == 0),
+                "rows of a product must be whole units");
+        if (a->nrows == 0) {
+            return;
+        }
+        dev::launch_compat_mmv(*gate, up, 2, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
+        launch_check("mmv_glu");
+    });
+}
+
+// launch.cu:367-402
+int bf16n_dequant(const bf16n_weight * w, int64_t row0, int64_t nrows, uint16_t * out, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(row0 >= 0 && nrows >= 0 && row0 + nrows <= w->rows, "dequant rows out of range");
+        if (nrows == 0) {
+            return;
+        }
+        if (w->format != FMT_NIBBLE) {
+            require(nrows % w->R == 0 && row0 % w->R == 0, "dequant rows must be whole units");
+        }
+        if (is_w64(*w)) {
+            dev::launch_w64_dequant(*w, row0, nrows, out, g_cus, (hipStream_t) stream);
+        } else {
+            dev::launch_compat_dequant(*w, row0, nrows, out, g_cus, (hipStream_t) stream);
+        }
+        launch_check("dequant");
+    });
+}
+
+// launch.cu:404-443
+int bf16n_get_rows(const bf16n_weight * w, const void * ids, int64_t ids_s0, int64_t n, void * dst, int dst_bf16,
+                   int64_t dst_s1, void * stream, int64_t row0) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(n >= 0, "get_rows: n must be nonnegative");
+        require(row0 >= 0 && (n == 0 ? row0 <= w->rows : row0 < w->rows), "get_rows: row0 out of range");
+        require(!(w->flags & FLAG_CHUNK_MAJOR), "get_rows of a chunk-major (expert) matrix");
+        require(w->format != FMT_HUFFMAN, "get_rows is not implemented for the single-symbol Huffman format");
+        if (n == 0) {
+            return;
+        }
+        if (is_w64(*w)) {
+            dev::launch_w64_get_rows(*w, ids, ids_s0, n, dst, dst_bf16 != 0, dst_s1, row0, (hipStream_t) stream);
+        } else {
+            dev::launch_compat_get_rows(*w, ids, ids_s0, n, dst, dst_bf16 != 0, dst_s1, row0, (hipStream_t) stream);
+        }
+        launch_check("get_rows");
+    });
+}
+
+int bf16n_mm_ids_supported(const bf16n_weight * w, const bf16n_weight * up) { return dev::mm_ids_shape_ok(*w, up) ? 1 : 0; }
+
+// launch.cu:458-471
+int bf16n_mm_ids_route(const void * ids, int ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst,
+                       int32_t * bounds, int n_experts, int n_tok, int n_used, int nchannels_y, int sis1, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        require(n_tok > 0 && n_tok < (1 << 22) && n_used > 0 && n_used < (1 << 10), "routing sizes out of range");
+        require(n_experts > 0, "routing sizes out of range");
+        require((int64_t) n_tok * ids_row_stride < INT32_MAX, "routing ids too large for 32-bit indexing");
+        dev::launch_route(ids, ids_i64 != 0, ids_row_stride, ids_src1, ids_dst, bounds, n_experts, n_tok, n_used, nchannels_y, sis1,
+                          (hipStream_t) stream);
+        launch_check("mm_ids_route");
+    });
+}
+
+// launch.cu:473-535
+int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row,
+                 const int32_t * ids_src1, const int32_t * ids_dst, const int32_t * bounds, void * dst, int dst_bf16,
+                 int64_t dst_col, int n_experts, int n_tok, int n_used, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(dev::mm_ids_shape_ok(*w, up), "no batched kernel for this matrix");
+        require(n_experts > 0 && w->rows % n_experts == 0, "rows must split evenly into experts");
+        dev::launch_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, n_tok, n_used,
+                           g_cus, (hipStream_t) stream);
+        launch_check("mm_ids");
+    });
+}
+
+// launch.cu:562-572
+int bf16n_moe_combine(const float * ys, const void * w, int w_bf16, void * y, int y_bf16, int n_tok, int n_used, int64_t n,
+                      void * stream) {
+    return guarded([&] {
+        ensure_init();
+        if (n_tok == 0 || n == 0) {
+            return;
+        }
+        require(n_tok <= 65535, "moe_combine: too many tokens for one launch");
+        dev::launch_moe_combine(ys, w, w_bf16 != 0, y, y_bf16 != 0, n_tok, n_used, n, (hipStream_t) stream);
+        launch_check("moe_combine");
+    });
+}
+
+// launch.cu:574-582
+int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        if (n == 0) {
+            return;
+        }
+        dev::launch_swiglu(g, u, y, n, g_cus, (hipStream_t) stream);
+        launch_check("swiglu");
+    });
+}
+
+int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
+                      int32_t * ids, float * weights, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        require(n_tok > 0 && n_experts > 0 && k > 0 && k <= n_experts && k <= 64, "router_topk: need 0 < k <= min(n_experts, 64)");
+        require(n_experts <= 8192, "router_topk: too many experts");
+        dev::launch_router_topk(logits, logits_stride, n_tok, n_experts, k, renorm != 0, ids, weights, (hipStream_t) stream);
+        launch_check("router_topk");
+    });
+}
+
+} // extern "C"

@@ -1,0 +1,448 @@
+// Kernels for the reference's 32-lane layouts: HUFPAIR row-/chunk-major, HUFFMAN and NIBBLE (GEMV, GLU-GEMV, exact
+// dequant, row gather).  Buffers made by the reference encoder decode here unchanged.
+//
+// A wave64 carries two units (HUFPAIR / HUFFMAN) or two rows (NIBBLE): lanes 0..31 the even one, lanes 32..63 the odd
+// one; each half reads its 512-byte plane chunk with one 16-byte load per lane.  Lane streams are per-lane sequential
+// reads through the vector cache.  These kernels favour generality (any K, R, layout, expert ids, FP32 or BF16
+// activations) over speed; the wave64 layout (kernels_w64.hip) is the fast path.
+#include "dev_common.h"
+#include "launchers.h"
+
+namespace bf16n {
+namespace dev {
+
+namespace {
+
+constexpr int NT = 256;          // threads per block
+constexpr int HALVES = NT / 32;  // units (rows) per block
+
+struct hp_ptrs { const uint8_t * plane; const uint32_t * lut; const uint32_t * ubase; const uint16_t * lrel; const uint32_t * stream; };
+struct huf_ptrs { const uint8_t * plane; const uint32_t * lut; const uint32_t * lane_off; const uint32_t * stream; };
+struct nib_ptrs { const uint8_t * plane; const uint8_t * codes; const uint8_t * table; const uint32_t * esc_off; const uint32_t * esc; };
+
+__device__ __forceinline__ hp_ptrs hpp(const bf16n_weight & w) {
+    return {w.plane, (const uint32_t *) (w.aux + w.off_a), (const uint32_t *) (w.aux + w.off_b),
+            (const uint16_t *) (w.aux + w.off_c), (const uint32_t *) (w.aux + w.off_d)};
+}
+__device__ __forceinline__ huf_ptrs hufp(const bf16n_weight & w) {
+    return {w.plane, (const uint32_t *) (w.aux + w.off_a), (const uint32_t *) (w.aux + w.off_b),
+            (const uint32_t *) (w.aux + w.off_c)};
+}
+__device__ __forceinline__ nib_ptrs nibp(const bf16n_weight & w, int64_t shift_rows) {
+    // the up half of a merged [gate; up] matrix: every per-row array shifted by shift_rows (escape offsets are absolute)
+    return {w.plane + shift_rows * w.K, w.aux + w.off_a + shift_rows * (w.K / 2), w.aux + w.off_b + shift_rows * 16,
+            (const uint32_t *) (w.aux + w.off_c) + shift_rows, (const uint32_t *) (w.aux + w.off_d)};
+}
+
+// MSB-first bit buffer over one lane stream: `v` valid bits at the top of `buf`, one word of lookahead in `nxt`.
+// Two table lookups (<= 24 bits) are always covered because v > 32 after every refill.  The stream buffers end with
+// padding words, so the lookahead never leaves the allocation.
+struct lane_bits {
+    const uint32_t * sp;
+    uint64_t buf;
+    uint32_t nxt;
+    int v;
+    __device__ __forceinline__ void begin(const uint32_t * p) {
+        sp = p;
+        buf = ((uint64_t) sp[0] << 32) | sp[1];
+        nxt = sp[2];
+        sp += 3;
+        v = 64;
+    }
+    template <int BITS>
+    __device__ __forceinline__ uint32_t take(const uint32_t * lut) {
+        const uint32_t ent = lut[(uint32_t) (buf >> (64 - BITS))];
+        const int len = (int) (ent & 31u);
+        buf <<= len;
+        v -= len;
+        return ent;
+    }
+    __device__ __forceinline__ void refill() {
+        if (v <= 32) {
+            buf |= (uint64_t) nxt << (32 - v);
+            v += 32;
+            nxt = *sp++;
+        }
+    }
+};
+
+// the 16 weights of one lane in one chunk as 8 BF16 pairs: wp[2j], wp[2j+1] = columns 128j + 4l + {0,1}, {2,3}
+template <int FORMAT>
+__device__ __forceinline__ void decode_chunk(lane_bits & bits, const uint32_t * lut, const uint4 sm, uint32_t (&wp)[8]) {
+    const uint32_t smw[4] = {sm.x, sm.y, sm.z, sm.w};
+    if (FORMAT == FMT_HUFPAIR) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t e0 = bits.take<HP_LP>(lut);
+            const uint32_t e1 = bits.take<HP_LP>(lut);
+            bits.refill();
+            wp[2 * j] = merge(spread_lo(smw[j]), e0);
+            wp[2 * j + 1] = merge(spread_hi(smw[j]), e1);
+        }
+    } else { // single exponents, entry = len | exponent << 7
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t a = bits.take<HUF_LMAX>(lut), b = bits.take<HUF_LMAX>(lut);
+            bits.refill();
+            const uint32_t c = bits.take<HUF_LMAX>(lut), d = bits.take<HUF_LMAX>(lut);
+            bits.refill();
+            wp[2 * j] = merge(spread_lo(smw[j]), (a & 0x7F80u) | ((b & 0x7F80u) << 16));
+            wp[2 * j + 1] = merge(spread_hi(smw[j]), (c & 0x7F80u) | ((d & 0x7F80u) << 16));
+        }
+    }
+}
+
+template <typename TX>
+__device__ __forceinline__ float x_at(const char * x, int i);
+template <> __device__ __forceinline__ float x_at<float>(const char * x, int i) { return ((const float *) x)[i]; }
+template <> __device__ __forceinline__ float x_at<bf16_t>(const char * x, int i) { return bf16_bits_to_f32(((const uint16_t *) x)[i]); }
+
+__device__ __forceinline__ float dot_chunk(const uint32_t (&wp)[8], const float * xs, int l32) {
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float4 xv = *(const float4 *) (xs + 128 * j + 4 * l32);
+        a0 = fmaf(bf16_bits_to_f32(wp[2 * j] & 0xFFFFu), xv.x, a0);
+        a1 = fmaf(__uint_as_float(wp[2 * j] & 0xFFFF0000u), xv.y, a1);
+        a2 = fmaf(bf16_bits_to_f32(wp[2 * j + 1] & 0xFFFFu), xv.z, a2);
+        a3 = fmaf(__uint_as_float(wp[2 * j + 1] & 0xFFFF0000u), xv.w, a3);
+    }
+    return (a0 + a1) + (a2 + a3);
+}
+
+// One unit of R rows: y[rr] (rr < R) ends up in lane rr of the half-wave.  Row-major streams finish a row every C
+// chunks; chunk-major streams add one partial sum per (chunk, row).
+template <int FORMAT>
+__device__ __forceinline__ float unit_dot(const uint8_t * plane, const uint32_t * lut, const uint32_t * sp, int64_t gu, int R,
+                                          int C, bool cm, const float * xs, int l32) {
+    lane_bits bits;
+    bits.begin(sp);
+    const uint8_t * up = plane + gu * R * (int64_t) C * CHUNK;
+    float mine = 0.f;
+    if (cm) {
+        for (int c = 0; c < C; c++) {
+            for (int rr = 0; rr < R; rr++) {
+                uint32_t wp[8];
+                decode_chunk<FORMAT>(bits, lut, *((const uint4 *) (up + ((int64_t) c * R + rr) * CHUNK) + l32), wp);
+                const float s = half_wave_sum(dot_chunk(wp, xs + c * CHUNK, l32));
+                mine += l32 == rr ? s : 0.f;
+            }
+        }
+    } else {
+        for (int rr = 0; rr < R; rr++) {
+            float acc = 0.f;
+            for (int c = 0; c < C; c++) {
+                uint32_t wp[8];
+                decode_chunk<FORMAT>(bits, lut, *((const uint4 *) (up + ((int64_t) rr * C + c) * CHUNK) + l32), wp);
+                acc += dot_chunk(wp, xs + c * CHUNK, l32);
+            }
+            const float s = half_wave_sum(acc);
+            mine = l32 == rr ? s : mine;
+        }
+    }
+    return mine;
+}
+
+template <int FORMAT>
+__device__ __forceinline__ const uint32_t * lane_stream(const bf16n_weight & w, int64_t gu, int l32) {
+    if (FORMAT == FMT_HUFPAIR) {
+        const hp_ptrs p = hpp(w);
+        return p.stream + p.ubase[gu] + p.lrel[gu * 32 + l32];
+    }
+    const huf_ptrs p = hufp(w);
+    return p.stream + p.lane_off[gu * 32 + l32];
+}
+
+// y = W x (GLU: y = silu(gate x) * up x) for HUFPAIR / HUFFMAN in the 32-lane layouts; one half-wave per unit,
+// blockIdx.y = column.  Shared memory: x as FP32 [K], then one table per matrix.
+template <int FORMAT, typename TX, bool GLU>
+__global__ void __launch_bounds__(NT) k_huf_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p) {
+    constexpr int LUT_N = FORMAT == FMT_HUFPAIR ? (1 << HP_LP) : (1 << HUF_LMAX);
+    extern __shared__ __align__(16) unsigned char shm_raw[];
+    const int K = (int) w.K, C = K / CHUNK, R = w.R;
+    float * xs = (float *) shm_raw;
+    uint32_t * lut = (uint32_t *) (xs + K);
+    uint32_t * lut_up = lut + LUT_N;
+    const col_view cv = col_setup(p, blockIdx.y);
+    for (int i = threadIdx.x; i < K; i += NT) {
+        xs[i] = x_at<TX>(cv.x, i);
+    }
+    const uint32_t * lut_g = (const uint32_t *) (w.aux + w.off_a);
+    for (int i = threadIdx.x; i < LUT_N; i += NT) {
+        lut[i] = lut_g[i];
+    }
+    if (GLU) {
+        const uint32_t * lut_ug = (const uint32_t *) (w_up.aux + w_up.off_a);
+        for (int i = threadIdx.x; i < LUT_N; i += NT) {
+            lut_up[i] = lut_ug[i];
+        }
+    }
+    __syncthreads();
+    const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
+    const bool cm = (w.flags & FLAG_CHUNK_MAJOR) != 0;
+    const int64_t units = p.nrows / R;
+    for (int64_t u = (int64_t) blockIdx.x * HALVES + half; u < units; u += (int64_t) gridDim.x * HALVES) {
+        const int64_t gu = cv.rbase / R + u;
+        float v = unit_dot<FORMAT>(w.plane, lut, lane_stream<FORMAT>(w, gu, l32), gu, R, C, cm, xs, l32);
+        if (GLU) {
+            const float uv = unit_dot<FORMAT>(w_up.plane, lut_up, lane_stream<FORMAT>(w_up, gu, l32), gu, R, C, false, xs, l32);
+            v = uv * silu(v);
+        }
+        if (l32 < R) {
+            store_y(cv.y, p.y_bf16, u * R + l32, v);
+        }
+    }
+}
+
+// exact BF16 bits of rows [row0, row0 + nrows) (whole units), row-major; one half-wave per unit
+template <int FORMAT>
+__global__ void __launch_bounds__(NT) k_huf_dequant(const bf16n_weight w, int64_t row0, int64_t nrows, uint16_t * __restrict__ out) {
+    constexpr int LUT_N = FORMAT == FMT_HUFPAIR ? (1 << HP_LP) : (1 << HUF_LMAX);
+    __shared__ uint32_t lut[LUT_N];
+    const uint32_t * lut_g = (const uint32_t *) (w.aux + w.off_a);
+    for (int i = threadIdx.x; i < LUT_N; i += NT) {
+        lut[i] = lut_g[i];
+    }
+    __syncthreads();
+    const int K = (int) w.K, C = K / CHUNK, R = w.R;
+    const bool cm = (w.flags & FLAG_CHUNK_MAJOR) != 0;
+    const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
+    for (int64_t u = (int64_t) blockIdx.x * HALVES + half; u < nrows / R; u += (int64_t) gridDim.x * HALVES) {
+        const int64_t gu = row0 / R + u;
+        lane_bits bits;
+        bits.begin(lane_stream<FORMAT>(w, gu, l32));
+        const uint8_t * up = w.plane + gu * R * (int64_t) K;
+        for (int o = 0; o < R * C; o++) {
+            const int rr = cm ? o % R : o / C, c = cm ? o / R : o % C;
+            uint32_t wp[8];
+            decode_chunk<FORMAT>(bits, lut, *((const uint4 *) (up + (int64_t) o * CHUNK) + l32), wp);
+            uint16_t * dst = out + (u * R + rr) * K + c * CHUNK;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                *(uint2 *) (dst + 128 * j + 4 * l32) = make_uint2(wp[2 * j], wp[2 * j + 1]);
+            }
+        }
+    }
+}
+
+// dst[i] = row (row0 + ids[i]) as FP32 or BF16: the half-wave decodes the row's unit from its start and stores only
+// the requested row (reference kernels.cuh:840-891)
+template <bool BF>
+__global__ void __launch_bounds__(NT) k_hp_get_rows(const bf16n_weight w, const char * __restrict__ ids, int64_t ids_s0, int64_t n,
+                                                    int64_t row0, char * __restrict__ dst, int64_t dst_s1) {
+    __shared__ uint32_t lut[1 << HP_LP];
+    const uint32_t * lut_g = (const uint32_t *) (w.aux + w.off_a);
+    for (int i = threadIdx.x; i < (1 << HP_LP); i += NT) {
+        lut[i] = lut_g[i];
+    }
+    __syncthreads();
+    const int K = (int) w.K, C = K / CHUNK, R = w.R;
+    const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
+    const int64_t i = (int64_t) blockIdx.x * HALVES + half;
+    if (i >= n) {
+        return;
+    }
+    const int64_t gr = row0 + *(const int32_t *) (ids + i * ids_s0);
+    const int64_t gu = gr / R;
+    lane_bits bits;
+    bits.begin(lane_stream<FMT_HUFPAIR>(w, gu, l32));
+    char * o = dst + i * dst_s1;
+    for (int64_t r = gu * R; r <= gr; r++) {
+        for (int c = 0; c < C; c++) {
+            uint32_t wp[8];
+            decode_chunk<FMT_HUFPAIR>(bits, lut, *((const uint4 *) (w.plane + r * K + c * CHUNK) + l32), wp);
+            if (r == gr) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int col = c * CHUNK + 128 * j + 4 * l32;
+                    if (BF) {
+                        *(uint2 *) (o + 2 * col) = make_uint2(wp[2 * j], wp[2 * j + 1]);
+                    } else {
+                        *(float4 *) (o + 4 * col) = make_float4(bf16_bits_to_f32(wp[2 * j] & 0xFFFFu), __uint_as_float(wp[2 * j] & 0xFFFF0000u),
+                                                                bf16_bits_to_f32(wp[2 * j + 1] & 0xFFFFu), __uint_as_float(wp[2 * j + 1] & 0xFFFF0000u));
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- NIBBLE
+
+// 4 exponents of 4 adjacent columns from 4 nibble codes (16 bits) and the row's 16-byte table, as bytes e0..e3
+__device__ __forceinline__ uint32_t nib_lookup4(const uint4 T, uint32_t codes16) {
+    uint32_t s = (codes16 | (codes16 << 8)) & 0x00FF00FFu;
+    s = (s | (s << 4)) & 0x0F0F0F0Fu; // one code per byte
+    const uint32_t lo = __builtin_amdgcn_perm(T.y, T.x, s & 0x07070707u);
+    const uint32_t hi = __builtin_amdgcn_perm(T.w, T.z, s & 0x07070707u);
+    const uint32_t pick_hi = ((s >> 3) & 0x01010101u) * 0xFFu;
+    return (hi & pick_hi) | (lo & ~pick_hi);
+}
+
+// the 16 weights of one lane in one NIBBLE chunk
+__device__ __forceinline__ void nib_chunk(const uint4 sm, const uint2 cd, const uint4 T, uint32_t (&wp)[8]) {
+    const uint32_t smw[4] = {sm.x, sm.y, sm.z, sm.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t c16 = ((j & 2) ? cd.y : cd.x) >> ((j & 1) * 16) & 0xFFFFu;
+        const uint32_t e4 = nib_lookup4(T, c16);
+        wp[2 * j] = merge(spread_lo(smw[j]), __builtin_amdgcn_perm(0, e4, 0x0c010c00u) << 7);
+        wp[2 * j + 1] = merge(spread_hi(smw[j]), __builtin_amdgcn_perm(0, e4, 0x0c030c02u) << 7);
+    }
+}
+
+__device__ __forceinline__ uint32_t esc_bits(uint32_t rec) { // BF16 bits of an escape record col | sm << 12 | exponent << 20
+    const uint32_t smb = (rec >> 12) & 0xFFu, ex = rec >> 20;
+    return ((smb & 0x80u) << 8) | (ex << 7) | (smb & 0x7Fu);
+}
+
+// dot(row gr, x); escaped weights read as +0 in the dense part and add their exact product afterwards; result in
+// every lane of the half-wave
+__device__ __forceinline__ float nib_row_dot(const nib_ptrs & w, int64_t gr, int C, const float * xs, int l32) {
+    const int64_t K = (int64_t) C * CHUNK;
+    const uint4 T = *(const uint4 *) (w.table + gr * 16);
+    float acc = 0.f;
+    for (int c = 0; c < C; c++) {
+        const uint4 sm = *((const uint4 *) (w.plane + gr * K + c * CHUNK) + l32);
+        const uint2 cd = *((const uint2 *) (w.codes + gr * (K / 2) + c * 256) + l32);
+        uint32_t wp[8];
+        nib_chunk(sm, cd, T, wp);
+        acc += dot_chunk(wp, xs + c * CHUNK, l32);
+    }
+    const uint32_t e0 = w.esc_off[gr], e1 = w.esc_off[gr + 1];
+    for (uint32_t i = e0 + l32; i < e1; i += 32) {
+        const uint32_t rec = w.esc[i];
+        acc = fmaf(bf16_bits_to_f32(esc_bits(rec)), xs[rec & 0xFFFu], acc);
+    }
+    return half_wave_sum(acc);
+}
+
+// NIBBLE GEMV; GLU 1: rows_per_matrix = [gate (nrows); up (nrows)] of one matrix; GLU 2: separate gate / up matrices
+template <typename TX, int GLU>
+__global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p) {
+    extern __shared__ __align__(16) unsigned char shm_raw[];
+    float * xs = (float *) shm_raw;
+    const int K = (int) w.K, C = K / CHUNK;
+    const col_view cv = col_setup(p, blockIdx.y);
+    for (int i = threadIdx.x; i < K; i += NT) {
+        xs[i] = x_at<TX>(cv.x, i);
+    }
+    __syncthreads();
+    const nib_ptrs g = nibp(w, 0);
+    const nib_ptrs u = GLU == 1 ? nibp(w, p.nrows) : nibp(w_up, 0);
+    const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
+    for (int64_t r = (int64_t) blockIdx.x * HALVES + half; r < p.nrows; r += (int64_t) gridDim.x * HALVES) {
+        float v = nib_row_dot(g, cv.rbase + r, C, xs, l32);
+        if (GLU) {
+            v = nib_row_dot(u, cv.rbase + r, C, xs, l32) * silu(v);
+        }
+        if (l32 == 0) {
+            store_y(cv.y, p.y_bf16, r, v);
+        }
+    }
+}
+
+// exact rows of a NIBBLE matrix: FP32 or BF16, to out + i * stride (bytes); row index from ids (gather) or row0 + i
+template <bool BF>
+__global__ void __launch_bounds__(NT) k_nib_rows(const bf16n_weight w, const char * __restrict__ ids, int64_t ids_s0, int64_t n,
+                                                 int64_t row0, char * __restrict__ dst, int64_t dst_s1) {
+    const nib_ptrs q = nibp(w, 0);
+    const int K = (int) w.K, C = K / CHUNK;
+    const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
+    for (int64_t i = (int64_t) blockIdx.x * HALVES + half; i < n; i += (int64_t) gridDim.x * HALVES) {
+        const int64_t gr = row0 + (ids ? (int64_t) * (const int32_t *) (ids + i * ids_s0) : i);
+        char * o = dst + i * dst_s1;
+        const uint4 T = *(const uint4 *) (q.table + gr * 16);
+        for (int c = 0; c < C; c++) {
+            const uint4 sm = *((const uint4 *) (q.plane + gr * K + c * CHUNK) + l32);
+            const uint2 cd = *((const uint2 *) (q.codes + gr * (K / 2) + c * 256) + l32);
+            uint32_t wp[8];
+            nib_chunk(sm, cd, T, wp);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int col = c * CHUNK + 128 * j + 4 * l32;
+                if (BF) {
+                    *(uint2 *) (o + 2 * col) = make_uint2(wp[2 * j], wp[2 * j + 1]);
+                } else {
+                    *(float4 *) (o + 4 * col) = make_float4(bf16_bits_to_f32(wp[2 * j] & 0xFFFFu), __uint_as_float(wp[2 * j] & 0xFFFF0000u),
+                                                            bf16_bits_to_f32(wp[2 * j + 1] & 0xFFFFu), __uint_as_float(wp[2 * j + 1] & 0xFFFF0000u));
+                }
+            }
+        }
+        // the dense stores of this half-wave must land before its escape stores to the same row
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t e = q.esc_off[gr] + l32; e < q.esc_off[gr + 1]; e += 32) {
+            const uint32_t rec = q.esc[e];
+            if (BF) {
+                ((uint16_t *) o)[rec & 0xFFFu] = (uint16_t) esc_bits(rec);
+            } else {
+                ((float *) o)[rec & 0xFFFu] = bf16_bits_to_f32(esc_bits(rec));
+            }
+        }
+    }
+}
+
+// blocks of HALVES units (rows) each, capped so that a launch of several columns stays within a few blocks per CU
+int grid_for(int64_t work, int ncols, int cus) {
+    const int64_t blocks = (work + HALVES - 1) / HALVES;
+    const int64_t cap = (int64_t) cus * 8 / (ncols < 1 ? 1 : ncols > 4 ? 4 : ncols);
+    return (int) (blocks < 1 ? 1 : blocks > cap ? cap : blocks);
+}
+
+} // namespace
+
+void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,
+                       int cus, hipStream_t stream) {
+    const bf16n_weight & wu = up ? *up : w;
+    const int64_t work = w.format == FMT_NIBBLE ? p.nrows : p.nrows / w.R;
+    const dim3 grid(grid_for(work, ncols, cus), ncols);
+    if (w.format == FMT_NIBBLE) {
+        const size_t shm = (size_t) w.K * 4;
+#define NIB(TX, G) hipLaunchKernelGGL((k_nib_mmv<TX, G>), grid, dim3(NT), shm, stream, w, wu, p)
+        if (x_bf16) { if (glu == 0) NIB(bf16_t, 0); else if (glu == 1) NIB(bf16_t, 1); else NIB(bf16_t, 2); }
+        else        { if (glu == 0) NIB(float, 0);  else if (glu == 1) NIB(float, 1);  else NIB(float, 2); }
+#undef NIB
+        return;
+    }
+    const bool hp = w.format == FMT_HUFPAIR;
+    const size_t shm = (size_t) w.K * 4 + (size_t) (glu ? 2 : 1) * (hp ? (4u << HP_LP) : (4u << HUF_LMAX));
+#define HUF(F, TX, G) hipLaunchKernelGGL((k_huf_mmv<F, TX, G>), grid, dim3(NT), shm, stream, w, wu, p)
+    if (hp) {
+        if (x_bf16) { if (glu) HUF(FMT_HUFPAIR, bf16_t, true); else HUF(FMT_HUFPAIR, bf16_t, false); }
+        else        { if (glu) HUF(FMT_HUFPAIR, float, true);  else HUF(FMT_HUFPAIR, float, false); }
+    } else {
+        if (x_bf16) { if (glu) HUF(FMT_HUFFMAN, bf16_t, true); else HUF(FMT_HUFFMAN, bf16_t, false); }
+        else        { if (glu) HUF(FMT_HUFFMAN, float, true);  else HUF(FMT_HUFFMAN, float, false); }
+    }
+#undef HUF
+}
+
+void launch_compat_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream) {
+    const int64_t work = w.format == FMT_NIBBLE ? nrows : nrows / w.R;
+    const int64_t blocks = (work + HALVES - 1) / HALVES;
+    const dim3 grid((unsigned) (blocks < (int64_t) cus * 16 ? blocks : (int64_t) cus * 16));
+    if (w.format == FMT_NIBBLE) {
+        hipLaunchKernelGGL((k_nib_rows<true>), grid, dim3(NT), 0, stream, w, (const char *) nullptr, (int64_t) 0, nrows, row0,
+                           (char *) out, (int64_t) w.K * 2);
+    } else if (w.format == FMT_HUFPAIR) {
+        hipLaunchKernelGGL((k_huf_dequant<FMT_HUFPAIR>), grid, dim3(NT), 0, stream, w, row0, nrows, out);
+    } else {
+        hipLaunchKernelGGL((k_huf_dequant<FMT_HUFFMAN>), grid, dim3(NT), 0, stream, w, row0, nrows, out);
+    }
+}
+
+void launch_compat_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
+                            int64_t dst_s1, int64_t row0, hipStream_t stream) {
+    const dim3 grid((unsigned) ((n + HALVES - 1) / HALVES));
+    if (w.format == FMT_NIBBLE) {
+        if (dst_bf16) hipLaunchKernelGGL((k_nib_rows<true>), grid, dim3(NT), 0, stream, w, (const char *) ids, ids_s0, n, row0, (char *) dst, dst_s1);
+        else          hipLaunchKernelGGL((k_nib_rows<false>), grid, dim3(NT), 0, stream, w, (const char *) ids, ids_s0, n, row0, (char *) dst, dst_s1);
+    } else {
+        if (dst_bf16) hipLaunchKernelGGL((k_hp_get_rows<true>), grid, dim3(NT), 0, stream, w, (const char *) ids, ids_s0, n, row0, (char *) dst, dst_s1);
+        else          hipLaunchKernelGGL((k_hp_get_rows<false>), grid, dim3(NT), 0, stream, w, (const char *) ids, ids_s0, n, row0, (char *) dst, dst_s1);
+    }
+}
+
+} // namespace dev
+} // namespace bf16n

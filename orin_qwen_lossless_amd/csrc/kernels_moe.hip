@@ -1,0 +1,180 @@
+// MoE glue around the expert GEMVs: SiLU gating, weighted combine, expert-sorted routing lists for the batched kernel,
+// and the router's softmax + top-k (on the device so that a decode step has no host round trip and can be captured
+// into a HIP graph).  All reductions run in a fixed order: results are bitwise reproducible.
+#include "dev_common.h"
+#include "launchers.h"
+
+namespace bf16n {
+namespace dev {
+
+namespace {
+
+// y = silu(g) * u (reference launch.cu:554-558)
+__global__ void __launch_bounds__(256) k_swiglu(const float * __restrict__ g, const float * __restrict__ u, float * __restrict__ y, int64_t n) {
+    for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) {
+        y[i] = silu(g[i]) * u[i];
+    }
+}
+
+// y[t, i] = sum_k w[t, k] * ys[t, k, i], slots in order, one fmaf each (reference launch.cu:539-552)
+__global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ ys, const char * __restrict__ w, bool w_bf16,
+                                                     char * __restrict__ y, bool y_bf16, int n_used, int64_t n) {
+    const int t = blockIdx.y;
+    for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) {
+        float acc = 0.f;
+        for (int k = 0; k < n_used; k++) {
+            const int64_t s = (int64_t) t * n_used + k;
+            const float wk = w_bf16 ? bf16_bits_to_f32(((const uint16_t *) w)[s]) : ((const float *) w)[s];
+            acc = fmaf(wk, ys[s * n + i], acc);
+        }
+        store_y(y + (int64_t) t * n * (y_bf16 ? 2 : 4), y_bf16, i, acc);
+    }
+}
+
+// Routing lists (reference mmid_helper.cu:48-136): block e lists the (token, slot) pairs of expert e in token order at
+// positions bounds[e].., where bounds[e] = number of pairs of experts < e.  ids element i of token t at byte
+// ids + (t * stride + i) * elem (low 32 bits are read).
+__global__ void __launch_bounds__(256) k_route(const char * __restrict__ ids, int elem, int64_t stride, int32_t * __restrict__ ids_src1,
+                                               int32_t * __restrict__ ids_dst, int32_t * __restrict__ bounds, int n_tok, int n_used,
+                                               int nchannels_y, int sis1) {
+    __shared__ int wave_hits[4], wave_lower[4];
+    __shared__ int s_lower_total;
+    const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // pass 1: pairs of lower experts (the start of this expert's range)
+    int lower = 0;
+    for (int64_t i = tid; i < (int64_t) n_tok * n_used; i += 256) {
+        const int64_t t = i / n_used, k = i % n_used;
+        lower += *(const int32_t *) (ids + (t * stride + k) * elem) < e;
+    }
+    for (int o = 32; o; o >>= 1) {
+        lower += __shfl_xor(lower, o, 64);
+    }
+    if (lane == 0) {
+        wave_lower[wave] = lower;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        s_lower_total = wave_lower[0] + wave_lower[1] + wave_lower[2] + wave_lower[3];
+    }
+    __syncthreads();
+    const int base = s_lower_total;
+    // pass 2: compact the tokens that use expert e, 256 tokens per round, in token order
+    int run = 0;
+    for (int t0 = 0; t0 < n_tok; t0 += 256) {
+        const int t = t0 + tid;
+        int slot = -1;
+        if (t < n_tok) {
+            for (int k = 0; k < n_used; k++) {
+                if (*(const int32_t *) (ids + ((int64_t) t * stride + k) * elem) == e) {
+                    slot = k;
+                }
+            }
+        }
+        const uint64_t m = __ballot(slot >= 0);
+        const int before = (int) __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
+        if (lane == 0) {
+            wave_hits[wave] = (int) __builtin_popcountll(m);
+        }
+        __syncthreads();
+        int off = run;
+        for (int w2 = 0; w2 < wave; w2++) {
+            off += wave_hits[w2];
+        }
+        if (slot >= 0) {
+            const int j = base + off + before;
+            ids_dst[j] = t * n_used + slot;
+            ids_src1[j] = t * sis1 + slot % nchannels_y;
+        }
+        run += wave_hits[0] + wave_hits[1] + wave_hits[2] + wave_hits[3];
+        __syncthreads();
+    }
+    if (tid == 0) {
+        bounds[e] = base;
+        if (e == (int) gridDim.x - 1) {
+            bounds[gridDim.x] = base + run;
+        }
+    }
+}
+
+// softmax over the experts, k largest (ties: lower index), weights renormalised to sum 1 if asked; one wave per token
+__global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ logits, int64_t stride, int n_experts, int k, bool renorm,
+                                                    int32_t * __restrict__ ids, float * __restrict__ weights) {
+    extern __shared__ float val[]; // logits of this token; taken ones become -inf
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float * lg = logits + (int64_t) t * stride;
+    float mx = -INFINITY;
+    for (int i = lane; i < n_experts; i += 64) {
+        val[i] = lg[i];
+        mx = fmaxf(mx, lg[i]);
+    }
+    for (int o = 32; o; o >>= 1) {
+        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    }
+    float sum = 0.f;
+    for (int i = lane; i < n_experts; i += 64) {
+        sum += expf(val[i] - mx);
+    }
+    sum = wave_sum(sum);
+    float top = 0.f, mine = 0.f; // lane j keeps the j-th weight
+    for (int j = 0; j < k; j++) {
+        float bv = -INFINITY;
+        int bi = 0x7FFFFFFF;
+        for (int i = lane; i < n_experts; i += 64) {
+            const float v = val[i];
+            if (v > bv) { // ascending i within a lane: the first maximum wins
+                bv = v;
+                bi = i;
+            }
+        }
+        for (int o = 32; o; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        const float pj = expf(bv - mx) / sum;
+        top += pj;
+        if (lane == (j & 63)) {
+            mine = pj; // k <= 64
+            ids[(int64_t) t * k + j] = bi;
+        }
+        if (lane == (bi & 63)) {
+            val[bi] = -INFINITY;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (lane < k) {
+        weights[(int64_t) t * k + lane] = renorm ? mine / top : mine;
+    }
+}
+
+} // namespace
+
+void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int cus, hipStream_t stream) {
+    const int64_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(k_swiglu, dim3((unsigned) (blocks < (int64_t) cus * 8 ? blocks : (int64_t) cus * 8)), dim3(256), 0, stream, g, u, y, n);
+}
+
+void launch_moe_combine(const float * ys, const void * w, bool w_bf16, void * y, bool y_bf16, int n_tok, int n_used, int64_t n,
+                        hipStream_t stream) {
+    const int64_t bx = (n + 255) / 256;
+    hipLaunchKernelGGL(k_moe_combine, dim3((unsigned) (bx < 64 ? bx : 64), (unsigned) n_tok), dim3(256), 0, stream, ys, (const char *) w,
+                       w_bf16, (char *) y, y_bf16, n_used, n);
+}
+
+void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds,
+                  int n_experts, int n_tok, int n_used, int nchannels_y, int sis1, hipStream_t stream) {
+    hipLaunchKernelGGL(k_route, dim3(n_experts), dim3(256), 0, stream, (const char *) ids, ids_i64 ? 8 : 4, ids_row_stride, ids_src1,
+                       ids_dst, bounds, n_tok, n_used, nchannels_y, sis1);
+}
+
+void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
+                        float * weights, hipStream_t stream) {
+    hipLaunchKernelGGL(k_router_topk, dim3(n_tok), dim3(64), (size_t) n_experts * 4, stream, logits, stride, n_experts, k, renorm, ids,
+                       weights);
+}
+
+} // namespace dev
+} // namespace bf16n

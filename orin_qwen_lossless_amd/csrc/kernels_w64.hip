@@ -1,0 +1,481 @@
+// Kernels for the wave64 HUFPAIR layout (FLAG_WAVE64): fused decode + GEMV, exact dequant, row gather.
+//
+// One 64-lane wavefront decodes one unit at a time and owns a contiguous range of units, so everything it reads is
+// sequential in memory:
+//   * the sign|mantissa plane: 1024 contiguous bytes per step, one 16-byte load per lane (lanes 0..31 the even,
+//     lanes 32..63 the odd 512-column chunk of the step);
+//   * the unit streams: one word stream per unit, consumed front to back.  The wave copies it in 1 KiB blocks into a
+//     private ring in LDS (coalesced 16-byte loads, one block in flight in registers) and every lane that needs a new
+//     word after a pair of codes reads ring[consumed + rank among the refilling lanes] — consecutive addresses, no bank
+//     conflicts, no per-lane pointers;
+//   * the 4096-entry pair table sits in LDS once per block; an entry already holds both exponents in BF16 position, so
+//     one v_perm + one v_bfi turn two plane bytes and an entry into two BF16 weights.
+// Activations stay in registers for the whole kernel (a lane always meets the same columns), products are accumulated in
+// FP32 (v_dot2_f32_bf16 for BF16 activations, v_fma_f32 for FP32 ones) and reduced across the wave once per row.
+#include "dev_common.h"
+#include "launchers.h"
+
+namespace bf16n {
+namespace dev {
+
+namespace {
+
+constexpr int RING = 1024;    // ring words per wave (4 KiB)
+constexpr int RING_PAD = 128; // copy of the first ring words behind the end: reads never wrap
+constexpr int BLK = 256;      // words per refill block: one uint4 per lane
+constexpr int AHEAD = 640;    // words kept ahead of the consumer: a unit start (128) + a step (4 x 64) and one block
+constexpr int LUT_WORDS = 1 << HP_LP;
+
+struct w64_ptrs { const uint8_t * plane; const uint32_t * lut; const uint32_t * ubase; const uint32_t * stream; };
+__device__ __forceinline__ w64_ptrs w64p(const bf16n_weight & w) {
+    return {w.plane, (const uint32_t *) (w.aux + w.off_a), (const uint32_t *) (w.aux + w.off_b), (const uint32_t *) (w.aux + w.off_d)};
+}
+
+__device__ __forceinline__ uint32_t lds_entry(const uint32_t * lut, uint32_t byte_off) {
+    return *(const uint32_t *) ((const char *) lut + byte_off);
+}
+
+// Decoder state of one wave.  cons / filled / limit are the same in every lane (kept in scalar registers).
+struct w64_dec {
+    uint32_t w0, w1, P; // per lane: two stream words and the bit position in w0 (< 32)
+    uint32_t cons;      // words consumed, relative to src
+    uint32_t filled;    // words copied into the ring, relative to src (multiple of BLK)
+    uint32_t limit;     // end of this wave's streams, relative to src
+    uint32_t * ring;
+    const uint32_t * src; // 16-byte aligned
+    uint4 pend;           // block filled / BLK, in flight
+    int lane;
+
+    __device__ __forceinline__ uint4 load_block(uint32_t first_word) const {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (first_word < limit) { // a block that starts inside the range may run past it: the stream is padded
+            v = *((const uint4 *) (src + first_word) + lane);
+        }
+        return v;
+    }
+    __device__ __forceinline__ void store_block(uint32_t first_word, const uint4 v) {
+        const uint32_t off = first_word & (RING - 1);
+        *((uint4 *) (ring + off) + lane) = v;
+        if (off == 0 && lane < RING_PAD / 4) {
+            *((uint4 *) (ring + RING) + lane) = v;
+        }
+    }
+    // stream words [first, end) of the aux stream belong to this wave
+    __device__ __forceinline__ void start(uint32_t * ring_, const uint32_t * stream, uint32_t first, uint32_t end, int lane_) {
+        ring = ring_;
+        lane = lane_;
+        const uint32_t a = first & ~3u;
+        src = stream + a;
+        cons = first - a;
+        limit = end - a;
+        const uint4 b0 = load_block(0), b1 = load_block(BLK), b2 = load_block(2 * BLK);
+        pend = load_block(3 * BLK);
+        store_block(0, b0);
+        store_block(BLK, b1);
+        store_block(2 * BLK, b2);
+        filled = 3 * BLK;
+    }
+    __device__ __forceinline__ void keep_ahead() {
+        while (filled - cons < AHEAD) {
+            store_block(filled, pend);
+            filled += BLK;
+            pend = load_block(filled);
+        }
+    }
+    __device__ __forceinline__ void begin_unit() {
+        const uint32_t * p = ring + (cons & (RING - 1)) + 2 * lane;
+        w0 = p[0];
+        w1 = p[1];
+        P = 0;
+        cons += 128;
+    }
+    // two pair codes; afterwards lanes whose position passed a word boundary take the next stream words in lane order
+    __device__ __forceinline__ void two(const uint32_t * lut, uint32_t & e0, uint32_t & e1) {
+        const uint32_t W = __builtin_amdgcn_alignbit(w1, w0, P);
+        e0 = lds_entry(lut, W & 0x3FFCu);
+        const uint32_t W2 = W >> (e0 & 31u);
+        e1 = lds_entry(lut, W2 & 0x3FFCu);
+        P += (e0 + e1) & 63u;
+        const bool need = P >= 32u;
+        const uint64_t m = __ballot(need);
+        const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
+        const uint32_t nw = ring[(cons & (RING - 1)) + rank];
+        w0 = need ? w1 : w0;
+        w1 = need ? nw : w1;
+        P &= 31u;
+        cons += (uint32_t) __builtin_popcountll(m);
+    }
+    // the 16 weights of this lane in one step as 8 BF16 pairs: wp[2j], wp[2j+1] = columns 128j + 4(lane%32) + {0,1}, {2,3}
+    __device__ __forceinline__ void step(const uint32_t * lut, const uint4 sm, uint32_t (&wp)[8]) {
+        const uint32_t smw[4] = {sm.x, sm.y, sm.z, sm.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t e0, e1;
+            two(lut, e0, e1);
+            wp[2 * j] = merge(spread_lo(smw[j]), e0);
+            wp[2 * j + 1] = merge(spread_hi(smw[j]), e1);
+        }
+    }
+};
+
+__device__ __forceinline__ void stage_lut(uint32_t * lut, const uint32_t * lut_g) {
+    for (int i = threadIdx.x; i < LUT_WORDS / 4; i += blockDim.x) {
+        ((uint4 *) lut)[i] = ((const uint4 *) lut_g)[i];
+    }
+}
+
+// ---------------------------------------------------------------- activations in registers
+
+// the 16 activations one lane meets in one 512-column chunk, as the GEMV consumes them
+template <typename TX> struct xchunk;
+template <> struct xchunk<bf16_t> { // 8 BF16 pairs
+    uint32_t v[8];
+    __device__ __forceinline__ void load(const char * x, int col0) { // col0 = chunk * 512 + 4 * (lane % 32)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint2 t = *(const uint2 *) (x + 2 * (col0 + 128 * j));
+            v[2 * j] = t.x;
+            v[2 * j + 1] = t.y;
+        }
+    }
+    __device__ __forceinline__ float dot(const uint32_t (&wp)[8], float acc) const {
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            acc = dot2_bf16(wp[q], v[q], acc);
+        }
+        return acc;
+    }
+};
+template <> struct xchunk<float> {
+    float v[16];
+    __device__ __forceinline__ void load(const char * x, int col0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float4 t = *(const float4 *) (x + 4 * (col0 + 128 * j));
+            v[4 * j] = t.x; v[4 * j + 1] = t.y; v[4 * j + 2] = t.z; v[4 * j + 3] = t.w;
+        }
+    }
+    __device__ __forceinline__ float dot(const uint32_t (&wp)[8], float acc) const {
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            acc = fmaf(__uint_as_float(wp[q] << 16), v[2 * q], acc);
+            acc = fmaf(__uint_as_float(wp[q] & 0xFFFF0000u), v[2 * q + 1], acc);
+        }
+        return acc;
+    }
+};
+
+// ---------------------------------------------------------------- GEMV
+//
+// C = K / 512 in {1, 2, 4, 8}.  The loop body covers NB steps (2, or 4 for C = 8) so that the plane registers of a step
+// are reloaded for the same step of the next body as soon as they are consumed.  A body is 4 rows (C = 1: a step
+// holds two rows, one per half-wave), 2 rows (C = 2) or 1 row (C = 4, 8); a unit must hold whole bodies.
+template <int C> struct geom {
+    static constexpr int NB = C == 8 ? 4 : 2;           // steps per body
+    static constexpr int XS = C >= 2 ? C / 2 : 1;       // activation chunk sets per lane
+    static constexpr int ROWS = C == 1 ? 4 : C == 2 ? 2 : 1; // rows per body
+};
+
+template <typename TX, int C, int NC>
+__global__ void __launch_bounds__(1024) k_w64_mmv(const bf16n_weight w, const cols p, int units_per_wave) {
+    using G = geom<C>;
+    constexpr int K = C * CHUNK;
+    extern __shared__ __align__(16) uint32_t shm[];
+    uint32_t * lut = shm;
+    const w64_ptrs q = w64p(w);
+    stage_lut(lut, q.lut);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int R = w.R;
+    const col_view cv = col_setup(p, blockIdx.y * NC);
+    // activations: chunk 2i + half of the row for i < XS (C = 1: chunk 0 for both halves)
+    xchunk<TX> xr[NC][G::XS];
+#pragma unroll
+    for (int n = 0; n < NC; n++) {
+#pragma unroll
+        for (int i = 0; i < G::XS; i++) {
+            xr[n][i].load(cv.x + n * p.x_tok, (C == 1 ? 0 : (2 * i + half) * CHUNK) + 4 * l32);
+        }
+    }
+    __syncthreads();
+    const int64_t units = p.nrows / R;
+    const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
+    if (u_begin >= units) {
+        return;
+    }
+    const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
+    const int64_t gu0 = cv.rbase / R + u_begin;
+    w64_dec dec;
+    dec.start(shm + LUT_WORDS + wave * (RING + RING_PAD), q.stream, q.ubase[gu0], q.ubase[gu0 + (u_end - u_begin)], lane);
+    const uint4 * pp = (const uint4 *) (q.plane + gu0 * R * K) + lane; // + 64 per step
+    const int64_t steps_total = (u_end - u_begin) * R * C / 2;
+    int64_t steps_loaded = G::NB;
+    uint4 sm[G::NB];
+#pragma unroll
+    for (int s = 0; s < G::NB; s++) {
+        sm[s] = pp[64 * s];
+    }
+    pp += 64 * G::NB;
+    const int bodies_per_unit = R * C / 2 / G::NB;
+    int64_t row = u_begin * R; // output row of the body's first row, relative to the product
+    for (int64_t u = u_begin; u < u_end; u++) {
+        dec.keep_ahead();
+        dec.begin_unit();
+        for (int b = 0; b < bodies_per_unit; b++, row += G::ROWS) {
+            float acc[NC][G::NB];
+#pragma unroll
+            for (int s = 0; s < G::NB; s++) {
+                dec.keep_ahead();
+                uint32_t wp[8];
+                dec.step(lut, sm[s], wp);
+                if (steps_loaded < steps_total) { // the same step of the next body
+                    sm[s] = pp[0];
+                }
+                pp += 64;
+                steps_loaded++;
+#pragma unroll
+                for (int n = 0; n < NC; n++) {
+                    const int xi = C >= 4 ? s : 0;
+                    if (C >= 4) {
+                        acc[n][0] = xr[n][xi].dot(wp, s == 0 ? 0.f : acc[n][0]);
+                    } else {
+                        acc[n][s] = xr[n][xi].dot(wp, 0.f);
+                    }
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < NC; n++) {
+                char * y = cv.y + n * p.y_tok;
+                if (C >= 4) {
+                    const float v = wave_sum(acc[n][0]);
+                    if (lane == 0) {
+                        store_y(y, p.y_bf16, row, v);
+                    }
+                } else if (C == 2) {
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+                        const float v = wave_sum(acc[n][s]);
+                        if (lane == 0) {
+                            store_y(y, p.y_bf16, row + s, v);
+                        }
+                    }
+                } else { // a step = rows 2s (lanes 0..31) and 2s + 1 (lanes 32..63)
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+                        const float v = half_wave_sum(acc[n][s]);
+                        if (l32 == 0) {
+                            store_y(y, p.y_bf16, row + 2 * s + half, v);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- dequant / row gather
+
+// exact BF16 bits of rows [row0, row0 + nrows) (whole units) into out (row-major); one wave per range of units.
+// only_row >= 0: store just that row (relative to row0) — the row gather decodes its unit from the start.
+__device__ __forceinline__ void w64_unit_rows(w64_dec & dec, const uint32_t * lut, const uint8_t * unit_plane, int R, int C,
+                                              int lane, int64_t only_row, char * out, int64_t out_row_bytes, bool f32) {
+    const int l32 = lane & 31, half = lane >> 5;
+    const uint4 * pp = (const uint4 *) unit_plane + lane;
+    for (int st = 0; st < R * C / 2; st++) {
+        dec.keep_ahead();
+        uint32_t wp[8];
+        dec.step(lut, pp[64 * st], wp);
+        const int o = 2 * st + half, rr = o / C, c = o % C;
+        if (only_row >= 0 && (2 * st) / C > only_row) { // same decision in both half-waves
+            break;
+        }
+        if (only_row >= 0 && rr != only_row) {
+            continue;
+        }
+        char * dst = out + (only_row >= 0 ? 0 : rr) * out_row_bytes;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int col = c * CHUNK + 128 * j + 4 * l32;
+            if (f32) {
+                *(float4 *) (dst + 4 * col) = make_float4(__uint_as_float(wp[2 * j] << 16), __uint_as_float(wp[2 * j] & 0xFFFF0000u),
+                                                          __uint_as_float(wp[2 * j + 1] << 16), __uint_as_float(wp[2 * j + 1] & 0xFFFF0000u));
+            } else {
+                *(uint2 *) (dst + 2 * col) = make_uint2(wp[2 * j], wp[2 * j + 1]);
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) k_w64_dequant(const bf16n_weight w, int64_t row0, int64_t nrows, uint16_t * __restrict__ out,
+                                                     int units_per_wave) {
+    extern __shared__ __align__(16) uint32_t shm[];
+    uint32_t * lut = shm;
+    const w64_ptrs q = w64p(w);
+    stage_lut(lut, q.lut);
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int R = w.R, K = (int) w.K, C = K / CHUNK;
+    const int64_t units = nrows / R;
+    const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
+    if (u_begin >= units) {
+        return;
+    }
+    const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
+    const int64_t gu0 = row0 / R + u_begin;
+    w64_dec dec;
+    dec.start(shm + LUT_WORDS + wave * (RING + RING_PAD), q.stream, q.ubase[gu0], q.ubase[gu0 + (u_end - u_begin)], lane);
+    for (int64_t u = u_begin; u < u_end; u++) {
+        dec.keep_ahead();
+        dec.begin_unit();
+        w64_unit_rows(dec, lut, q.plane + (row0 / R + u) * R * (int64_t) K, R, C, lane, -1, (char *) (out + u * R * (int64_t) K),
+                      (int64_t) K * 2, false);
+    }
+}
+
+__global__ void __launch_bounds__(256) k_w64_get_rows(const bf16n_weight w, const char * __restrict__ ids, int64_t ids_s0, int64_t n,
+                                                      int64_t row0, char * __restrict__ dst, int64_t dst_s1, bool f32) {
+    extern __shared__ __align__(16) uint32_t shm[];
+    uint32_t * lut = shm;
+    const w64_ptrs q = w64p(w);
+    stage_lut(lut, q.lut);
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int R = w.R, K = (int) w.K, C = K / CHUNK;
+    const int64_t i = (int64_t) blockIdx.x * nwaves + wave;
+    if (i >= n) {
+        return;
+    }
+    const int64_t gr = row0 + *(const int32_t *) (ids + i * ids_s0);
+    const int64_t gu = gr / R;
+    w64_dec dec;
+    dec.start(shm + LUT_WORDS + wave * (RING + RING_PAD), q.stream, q.ubase[gu], q.ubase[gu + 1], lane);
+    dec.keep_ahead();
+    dec.begin_unit();
+    w64_unit_rows(dec, lut, q.plane + gu * R * (int64_t) K, R, C, lane, gr - gu * R, dst + i * dst_s1, 0, f32);
+}
+
+size_t w64_shm(int waves) { return (size_t) (LUT_WORDS + waves * (RING + RING_PAD)) * 4; }
+
+// waves per block and units per wave for `units` units per column: every wave gets the same number of units (but the
+// last), and a launch fills the device once when it can
+void w64_dims(int64_t units, int ncols, int cus, int & waves_per_block, int & blocks, int & units_per_wave) {
+    int64_t max_waves = (int64_t) cus * 16 / (ncols < 1 ? 1 : ncols);
+    max_waves = max_waves < 16 ? 16 : max_waves;
+    const int64_t upw = (units + max_waves - 1) / max_waves;
+    const int64_t waves = (units + upw - 1) / upw;
+    waves_per_block = waves >= 16 * (int64_t) cus ? 16 : waves >= 8 * (int64_t) cus ? 8 : 4;
+    if (waves < waves_per_block) {
+        waves_per_block = (int) waves;
+    }
+    blocks = (int) ((waves + waves_per_block - 1) / waves_per_block);
+    units_per_wave = (int) upw;
+}
+
+// columns that share one decode: as many (up to 4) as keep the activations within 64 registers per lane
+template <typename TX, int C>
+constexpr int max_group() {
+    constexpr int per_col = geom<C>::XS * (sizeof(TX) == 2 ? 8 : 16);
+    return 64 / per_col < 1 ? 1 : 64 / per_col > 4 ? 4 : 64 / per_col;
+}
+
+template <typename TX, int C>
+void mmv_nc(int nc, dim3 grid, int nt, size_t shm, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
+    constexpr int G = max_group<TX, C>();
+    if (nc == 1) {
+        hipLaunchKernelGGL((k_w64_mmv<TX, C, 1>), grid, dim3(nt), shm, stream, w, p, upw);
+    } else if (nc == 2) {
+        if constexpr (G >= 2) hipLaunchKernelGGL((k_w64_mmv<TX, C, 2>), grid, dim3(nt), shm, stream, w, p, upw);
+    } else if (nc == 3) {
+        if constexpr (G >= 3) hipLaunchKernelGGL((k_w64_mmv<TX, C, 3>), grid, dim3(nt), shm, stream, w, p, upw);
+    } else {
+        if constexpr (G >= 4) hipLaunchKernelGGL((k_w64_mmv<TX, C, 4>), grid, dim3(nt), shm, stream, w, p, upw);
+    }
+}
+
+template <typename TX>
+void mmv_c(int C, int nc, dim3 grid, int nt, size_t shm, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
+    switch (C) {
+        case 1: mmv_nc<TX, 1>(nc, grid, nt, shm, stream, w, p, upw); break;
+        case 2: mmv_nc<TX, 2>(nc, grid, nt, shm, stream, w, p, upw); break;
+        case 4: mmv_nc<TX, 4>(nc, grid, nt, shm, stream, w, p, upw); break;
+        default: mmv_nc<TX, 8>(nc, grid, nt, shm, stream, w, p, upw); break;
+    }
+}
+
+template <typename TX>
+int group_for(int C) {
+    return C == 1 ? max_group<TX, 1>() : C == 2 ? max_group<TX, 2>() : C == 4 ? max_group<TX, 4>() : max_group<TX, 8>();
+}
+
+template <typename TX, int C, int NC>
+void set_attr() {
+    if constexpr (NC <= max_group<TX, C>()) {
+        (void) hipFuncSetAttribute((const void *) k_w64_mmv<TX, C, NC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(16));
+    }
+}
+template <typename TX, int C>
+void set_attr_nc() { set_attr<TX, C, 1>(); set_attr<TX, C, 2>(); set_attr<TX, C, 3>(); set_attr<TX, C, 4>(); }
+template <typename TX>
+void set_attr_c() { set_attr_nc<TX, 1>(); set_attr_nc<TX, 2>(); set_attr_nc<TX, 4>(); set_attr_nc<TX, 8>(); }
+
+} // namespace
+
+void w64_init() {
+    set_attr_c<bf16_t>();
+    set_attr_c<float>();
+}
+
+// shapes with a fused wave64 GEMV: K in {512, 1024, 2048, 4096} and units that hold whole loop bodies
+bool w64_mmv_supported(const bf16n_weight & w, bool) {
+    const int64_t C = w.K / CHUNK;
+    if (C != 1 && C != 2 && C != 4 && C != 8) {
+        return false;
+    }
+    const int nb = C == 8 ? 4 : 2;
+    return (w.R * C / 2) % nb == 0;
+}
+
+void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf16, bool multi_col, int cus, hipStream_t stream) {
+    const int C = (int) (w.K / CHUNK);
+    const int64_t units = p.nrows / w.R;
+    // dense batches: groups of up to 4 columns share one decode (reference launch.cu:174-193), fewer where the
+    // activations of 4 columns would not fit in 64 registers per lane
+    const int group_max = !multi_col || p.ids ? 1 : x_bf16 ? group_for<bf16_t>(C) : group_for<float>(C);
+    for (int c0 = 0; c0 < (group_max == 1 ? 1 : ncols); c0 += group_max) {
+        const int nc = group_max == 1 ? 1 : (ncols - c0 < group_max ? ncols - c0 : group_max);
+        const int ny = group_max == 1 ? ncols : 1;
+        cols q = p;
+        if (group_max > 1) {
+            q.x += c0 * p.x_tok;
+            q.y += c0 * p.y_tok;
+        }
+        int wpb, blocks, upw;
+        w64_dims(units, ny, cus, wpb, blocks, upw);
+        const dim3 grid(blocks, ny);
+        if (x_bf16) {
+            mmv_c<bf16_t>(C, nc, grid, wpb * 64, w64_shm(wpb), stream, w, q, upw);
+        } else {
+            mmv_c<float>(C, nc, grid, wpb * 64, w64_shm(wpb), stream, w, q, upw);
+        }
+    }
+}
+
+void launch_w64_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream) {
+    const int64_t units = nrows / w.R;
+    const int64_t max_waves = (int64_t) cus * 16;
+    const int64_t upw = (units + max_waves - 1) / max_waves;
+    const int64_t waves = (units + upw - 1) / upw;
+    const int wpb = 4;
+    hipLaunchKernelGGL(k_w64_dequant, dim3((unsigned) ((waves + wpb - 1) / wpb)), dim3(wpb * 64), w64_shm(wpb), stream, w, row0, nrows,
+                       out, (int) upw);
+}
+
+void launch_w64_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
+                         int64_t dst_s1, int64_t row0, hipStream_t stream) {
+    const int wpb = 4;
+    hipLaunchKernelGGL(k_w64_get_rows, dim3((unsigned) ((n + wpb - 1) / wpb)), dim3(wpb * 64), w64_shm(wpb), stream, w, (const char *) ids,
+                       ids_s0, n, row0, (char *) dst, dst_s1, !dst_bf16);
+}
+
+} // namespace dev
+} // namespace bf16n

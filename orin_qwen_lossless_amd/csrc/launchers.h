@@ -1,0 +1,45 @@
+// Kernel launchers (defined in the .hip files), called by the C ABI after argument checks.  They only enqueue work.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "bf16n_c.h"
+#include "dev_common.h"
+
+namespace bf16n {
+namespace dev {
+
+// 32-lane layouts (kernels_compat.hip). glu: 0 plain, 1 merged [gate; up] NIBBLE matrix, 2 separate gate / up matrices
+void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,
+                       int cus, hipStream_t stream);
+void launch_compat_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream);
+void launch_compat_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
+                            int64_t dst_s1, int64_t row0, hipStream_t stream);
+
+// wave64 layout (kernels_w64.hip)
+void w64_init();
+bool w64_mmv_supported(const bf16n_weight & w, bool x_bf16);
+void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf16, bool multi_col, int cus, hipStream_t stream);
+void launch_w64_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream);
+void launch_w64_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
+                         int64_t dst_s1, int64_t row0, hipStream_t stream);
+
+// MoE glue (kernels_moe.hip)
+void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int cus, hipStream_t stream);
+void launch_moe_combine(const float * ys, const void * w, bool w_bf16, void * y, bool y_bf16, int n_tok, int n_used, int64_t n,
+                        hipStream_t stream);
+void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds,
+                  int n_experts, int n_tok, int n_used, int nchannels_y, int sis1, hipStream_t stream);
+void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
+                        float * weights, hipStream_t stream);
+
+// batched MoE prefill (kernels_mm_ids.hip)
+bool mm_ids_shape_ok(const bf16n_weight & w, const bf16n_weight * up);
+void launch_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
+                   const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
+                   int n_tok, int n_used, int cus, hipStream_t stream);
+
+} // namespace dev
+} // namespace bf16n

@@ -1,0 +1,107 @@
+// Shape policy: which format, unit size and layout a weight matrix gets (reference core/src/policy.cpp:9-69).
+// The llama and vllm engines reproduce the reference's decisions; mi355x is this build's tuning for 256 CUs of wave64.
+#include "encode_impl.h"
+
+namespace bf16n {
+namespace impl {
+
+namespace {
+
+// dense matrices: rows per unit.  llama: the largest R in {16, 8, 4, 2} that divides rows and leaves >= 512 units.
+// vllm: start from that R and move to a smaller one whenever its cost — waves of 512 units times R — is at least 5 %
+// lower (policy.cpp:9-31; the 0.95 comparison is done in double precision there as well).
+int dense_unit_rows(int64_t rows, int engine) noexcept {
+    int chosen = 1;
+    int64_t chosen_cost = 0;
+    const int candidates[] = {16, 8, 4, 2};
+    for (int r : candidates) {
+        if (rows % r != 0 || rows / r < 512) {
+            continue;
+        }
+        const int64_t units = rows / r;
+        const int64_t waves = units / 512 + (units % 512 != 0);
+        const int64_t cost = waves * r;
+        if (chosen == 1) {
+            chosen = r;
+            chosen_cost = cost;
+            if (engine == 0) {
+                return chosen;
+            }
+        } else if ((double) cost <= 0.95 * (double) chosen_cost) {
+            chosen = r;
+            chosen_cost = cost;
+        }
+    }
+    return chosen;
+}
+
+// rows * K * n >= threshold without forming the product (policy.cpp:34-41)
+bool reaches(int64_t rows, int64_t K, int64_t n, int64_t threshold) noexcept {
+    if (threshold <= 0) {
+        return true;
+    }
+    const int64_t per_matrix = threshold / n + (threshold % n != 0);
+    const int64_t rows_needed = per_matrix / K + (per_matrix % K != 0);
+    return rows >= rows_needed;
+}
+
+// mi355x dense: one wave64 decodes one unit and a launch wants several thousand units in flight (256 CUs x 8-16
+// waves), so take the largest R in {16, 8, 4, 2} that still leaves at least 4096 units, else the largest that leaves
+// 1024, else 2 (the wave64 layout needs an even number of chunks per unit; R = 1 only when rows is odd).
+int mi355x_dense_unit_rows(int64_t rows, int64_t K) noexcept {
+    const int candidates[] = {16, 8, 4, 2};
+    for (int64_t floor_units : {(int64_t) 4096, (int64_t) 1024, (int64_t) 1}) {
+        for (int r : candidates) {
+            if (rows % r == 0 && rows / r >= floor_units) {
+                return r;
+            }
+        }
+    }
+    (void) K;
+    return 1;
+}
+
+} // namespace
+
+bool choose(int64_t rows, int64_t K, int64_t n, int engine, int mode, int64_t dense_min, bool expert_flag,
+            bool dense_frag_order, choice & out) noexcept {
+    if (rows <= 0 || n <= 0 || K <= 0 || K % CHUNK != 0 || K > K_MAX) {
+        return false;
+    }
+    const bool vllm = engine == 1, mi355x = engine == 2;
+    const bool expert = vllm ? n > 1 : expert_flag; // llama (and mi355x) classify by the caller's flag (policy.cpp:49)
+    if (mode == 2 || (mode == 0 && !expert && !reaches(rows, K, n, dense_min))) {
+        out = {FMT_NIBBLE, 0, false, false, false};
+        return true;
+    }
+    const int64_t C = K / CHUNK;
+    if (mi355x) {
+        int R;
+        if (n > 1) { // experts: the reference's rule (policy.cpp:59-61)
+            R = rows % 16 == 0 && rows >= 2048 ? 16 : rows % 8 == 0 ? 8 : rows % 4 == 0 ? 4 : 1;
+        } else {
+            R = mi355x_dense_unit_rows(rows, K);
+        }
+        // the wave64 layout where the fused GEMV has an instance (K in {512, 1024, 2048, 4096}, units of whole loop
+        // bodies); it is row-major: the batched kernel decodes whole rows per step and needs no chunk-major order.
+        // Other shapes keep the reference layout and its rules.
+        const bool w64 = (C == 1 && R % 4 == 0) || (C == 2 && R % 2 == 0) || C == 4 || C == 8;
+        const bool cm = !w64 && n > 1 && K > CHUNK && (R == 4 || R == 8 || R == 16);
+        out = {FMT_HUFPAIR, R, cm, false, w64};
+        return true;
+    }
+    const bool fo_dense = vllm && dense_frag_order && n == 1 && rows % 16 == 0;
+    const bool fo_gate_up = vllm && n > 1 && K == 4 * CHUNK && rows % 16 == 0;
+    int R;
+    if (n > 1) {
+        R = fo_gate_up || (rows % 16 == 0 && rows >= 2048) ? 16 : rows % 8 == 0 ? 8 : rows % 4 == 0 ? 4 : 1;
+    } else {
+        R = fo_dense ? 16 : dense_unit_rows(rows, engine);
+    }
+    const bool fo_experts = fo_gate_up || (vllm && n > 1 && K == CHUNK && R == 16);
+    out = {FMT_HUFPAIR, R, n > 1 && K > CHUNK && !fo_experts, fo_experts || fo_dense, false};
+    return true;
+}
+
+} // namespace impl
+} // namespace bf16n

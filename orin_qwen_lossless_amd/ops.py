@@ -1,0 +1,509 @@
+"""Host-side operator layer over the C ABI, with the names, argument meaning and error behaviour of the reference's
+Python operator module (engines/vllm/vllm_bf16n/ops.py) so that code and tests written against it carry over:
+encode / upload / dequant / roundtrip_equal / mmv / mmv_glu / linear / get_rows / embedding / moe_mm_ids /
+moe_combine / swiglu / moe_experts, plus router_topk and choose.
+
+torch is used for device memory and streams only; every product runs in libbf16n_hip.so.  Weights are passed
+explicitly as plane + aux uint8 tensors with metadata parsed once from the aux header on the host."""
+from __future__ import annotations
+
+import ctypes as C
+import struct
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import _lib
+
+FMT_NIBBLE, FMT_HUFFMAN, FMT_HUFPAIR = 1, 2, 3
+FORMAT_NAMES = {FMT_NIBBLE: "nibble", FMT_HUFFMAN: "huffman", FMT_HUFPAIR: "hufpair"}
+MAGIC = 0x4E363142
+HEADER = struct.Struct("<IIIIQQQQQQQII")  # include/bf16n/format.h aux_header
+FLAG_CHUNK_MAJOR, FLAG_FRAG_ORDER, FLAG_WAVE64 = 1, 2, 4
+
+# up to 8 tokens through the GEMV kernels, more through the batched MoE kernel / dequant + GEMM
+# (engines/vllm/vllm_bf16n/ops.py:25-27, core/torch/torch_bindings.cpp:195)
+GEMV_MAX_TOKENS = 8
+DEQUANT_CHUNK_BYTES = 64 << 20
+
+ENGINES = {"llama": 0, "vllm": 1, "mi355x": 2}
+MODES = {"hybrid": 0, "huffman": 1, "nibble": 2}
+
+
+@dataclass(frozen=True)
+class Meta:
+    """Host-side metadata of one encoded matrix, parsed once from its aux header."""
+
+    format: int
+    K: int
+    rows: int
+    R: int
+    chunk_major: bool
+    frag_order: bool
+    off_a: int
+    off_b: int
+    off_c: int
+    off_d: int
+    wave64: bool = False
+
+    @property
+    def flags(self) -> int:
+        return ((FLAG_CHUNK_MAJOR if self.chunk_major else 0) | (FLAG_FRAG_ORDER if self.frag_order else 0)
+                | (FLAG_WAVE64 if self.wave64 else 0))
+
+    def as_list(self) -> list[int]:
+        return [self.format, self.K, self.rows, self.R, self.flags, self.off_a, self.off_b, self.off_c, self.off_d]
+
+
+def parse_header(aux: torch.Tensor) -> Meta:
+    """Metadata from the first 256 bytes of a CPU aux tensor; raises on a malformed header."""
+    if aux.device.type != "cpu" or aux.dtype != torch.uint8 or aux.numel() < 256:
+        raise ValueError("bf16n: aux must be a CPU uint8 tensor of at least 256 bytes")
+    (magic, fmt, K, R, rows, a, b, c, d, _na, _nb, flags, _pad) = HEADER.unpack(bytes(aux[: HEADER.size].tolist()))
+    if magic != MAGIC or fmt not in FORMAT_NAMES:
+        raise ValueError(f"bf16n: bad aux header (magic {magic:#x}, format {fmt})")
+    if flags & ~(FLAG_CHUNK_MAJOR | FLAG_FRAG_ORDER | FLAG_WAVE64):
+        raise ValueError(f"bf16n: unknown layout flags {flags:#x}")
+    return Meta(fmt, K, rows, R, bool(flags & FLAG_CHUNK_MAJOR), bool(flags & FLAG_FRAG_ORDER), a, b, c, d,
+                bool(flags & FLAG_WAVE64))
+
+
+@dataclass
+class Weight:
+    """One encoded matrix on the device: plane (rows x K sign|mantissa bytes) + aux, and its metadata."""
+
+    plane: torch.Tensor
+    aux: torch.Tensor
+    meta: Meta
+
+    @property
+    def m(self) -> list[int]:
+        return self.meta.as_list()
+
+    @property
+    def nbytes(self) -> int:
+        return self.plane.numel() + self.aux.numel()
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _cweight(w: Weight) -> _lib.Weight:
+    m = w.meta
+    if not (w.plane.is_cuda and w.aux.is_cuda):
+        raise ValueError("bf16n: plane and aux must be device tensors")
+    if w.plane.dtype != torch.uint8 or w.aux.dtype != torch.uint8:
+        raise ValueError("bf16n: plane and aux must be uint8")
+    if not (w.plane.is_contiguous() and w.aux.is_contiguous()):
+        raise ValueError("bf16n: plane and aux must be contiguous")
+    if w.plane.numel() != m.rows * m.K:
+        raise ValueError(f"bf16n: plane has {w.plane.numel()} bytes, meta says {m.rows} x {m.K}")
+    if max(m.off_a, m.off_b, m.off_c, m.off_d) >= w.aux.numel():
+        raise ValueError(f"bf16n: aux ({w.aux.numel()} bytes) shorter than its offsets")
+    if w.plane.data_ptr() % 16 or w.aux.data_ptr() % 16:
+        raise ValueError("bf16n: plane/aux must be 16-byte aligned")
+    return _lib.Weight(w.plane.data_ptr(), w.aux.data_ptr(), m.format, m.R, m.K, m.rows, m.flags, 0, m.off_a, m.off_b,
+                       m.off_c, m.off_d)
+
+
+def _check_x(x: torch.Tensor, K: int, what: str) -> None:
+    if not x.is_cuda:
+        raise ValueError(f"bf16n: {what} must be a device tensor")
+    if x.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"bf16n: {what} must be bf16 or f32")
+    if x.shape[-1] != K or x.stride(-1) != 1:
+        raise ValueError(f"bf16n: {what} last dim must be K = {K} and contiguous")
+    if x.data_ptr() % 16:
+        raise ValueError(f"bf16n: {what} must be 16-byte aligned")
+    for d in range(x.dim() - 1):
+        if (x.stride(d) * x.element_size()) % 16:
+            raise ValueError(f"bf16n: {what} row strides must be multiples of 16 bytes")
+
+
+def _check_ids(ids: torch.Tensor) -> None:
+    if not ids.is_cuda or ids.dim() != 2:
+        raise ValueError("bf16n: ids must be a 2-D device tensor [tokens, n_used]")
+    if ids.dtype not in (torch.int32, torch.int64):
+        raise ValueError("bf16n: ids must be int32 or int64")
+    if ids.stride(1) != 1:
+        raise ValueError("bf16n: ids must be contiguous along the slot dimension")
+
+
+def init() -> None:
+    """Device attributes and kernel shared-memory limits; once per process, before any launch / graph capture."""
+    _lib.check(_lib.lib().bf16n_init())
+
+
+def cu_count() -> int:
+    n = C.c_int()
+    _lib.check(_lib.lib().bf16n_cu_count(C.byref(n)))
+    return n.value
+
+
+def set_encode_threads(n: int) -> None:
+    _lib.lib().bf16n_set_encode_threads(int(n))
+
+
+def choose(rows: int, K: int, n_matrices: int = 1, engine: str = "mi355x", mode: str = "hybrid",
+           dense_min: int = 8 << 20, expert: bool = False, dense_frag_order: bool = False):
+    """Shape policy (core/src/policy.cpp). Returns None (stay BF16) or (format, R, chunk_major, frag_order, wave64)."""
+    out = (C.c_int * 5)()
+    ok = _lib.lib().bf16n_choose(rows, K, n_matrices, ENGINES[engine], MODES[mode], dense_min, int(expert),
+                                 int(dense_frag_order), out)
+    return None if not ok else (out[0], out[1], bool(out[2]), bool(out[3]), bool(out[4]))
+
+
+def encode_bits(w_bits: np.ndarray, fmt: int, R: int, chunk_major: bool = False, frag_order: bool = False,
+                wave64: bool = False) -> tuple[np.ndarray, np.ndarray, int, int]:
+    """Encode rows x K BF16 bit patterns (numpy uint16). Returns (plane, aux, format produced, R)."""
+    w_bits = np.ascontiguousarray(w_bits, dtype=np.uint16)
+    if w_bits.ndim < 2:
+        raise ValueError("bf16n.encode: weight must be at least 2-D (rows x K)")
+    K = w_bits.shape[-1]
+    rows = w_bits.size // max(K, 1)
+    flags = (FLAG_CHUNK_MAJOR if chunk_major else 0) | (FLAG_FRAG_ORDER if frag_order else 0) | (FLAG_WAVE64 if wave64 else 0)
+    L = _lib.lib()
+    h = C.c_void_p()
+    _lib.check(L.bf16n_encode(w_bits.ctypes.data, rows, K, fmt, R, flags, C.byref(h)))
+    try:
+        n = C.c_uint64()
+        p = L.bf16n_encoded_plane(h, C.byref(n))
+        plane = np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(n.value,)).copy().reshape(rows, K)
+        p = L.bf16n_encoded_aux(h, C.byref(n))
+        aux = np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(n.value,)).copy()
+        return plane, aux, L.bf16n_encoded_format(h), L.bf16n_encoded_R(h)
+    finally:
+        L.bf16n_encoded_free(h)
+
+
+def encode(w: torch.Tensor, fmt: int, R: int, chunk_major: bool, frag_order: bool = False, wave64: bool = False
+           ) -> tuple[torch.Tensor, torch.Tensor, Meta]:
+    """Encode a BF16 CPU tensor (..., K) on the host cores. FMT_HUFPAIR falls back to FMT_HUFFMAN when the tensor has
+    more than 4096 distinct exponent pairs; the returned Meta holds the format and layout actually produced."""
+    if w.device.type != "cpu":
+        raise ValueError("bf16n.encode: weight must be on the CPU")
+    if w.dtype != torch.bfloat16:
+        raise ValueError("bf16n.encode: weight must be bfloat16")
+    if w.dim() < 2:
+        raise ValueError("bf16n.encode: weight must be at least 2-D (rows x K)")
+    bits = w.contiguous().view(torch.int16).numpy().view(np.uint16)
+    plane, aux, _, _ = encode_bits(bits, fmt, R, chunk_major, frag_order, wave64)
+    tp, ta = torch.from_numpy(plane), torch.from_numpy(aux)
+    return tp, ta, parse_header(ta)
+
+
+def upload(plane: torch.Tensor, aux: torch.Tensor, meta: Meta, device: torch.device | str) -> Weight:
+    return Weight(plane.to(device), aux.to(device), meta)
+
+
+def dequant(w: Weight, row0: int = 0, nrows: int | None = None) -> torch.Tensor:
+    nrows = w.meta.rows - row0 if nrows is None else nrows
+    cw = _cweight(w)
+    if row0 < 0 or nrows < 0 or row0 + nrows > w.meta.rows:
+        raise ValueError("bf16n.dequant: rows out of range")
+    out = torch.empty((nrows, w.meta.K), dtype=torch.bfloat16, device=w.plane.device)
+    with torch.cuda.device(w.plane.device):
+        _lib.check(_lib.lib().bf16n_dequant(C.byref(cw), row0, nrows, out.data_ptr(), _stream()))
+    return out
+
+
+def roundtrip_equal(w: Weight, src: torch.Tensor, chunk_bytes: int = 64 << 20) -> bool:
+    """Bitwise check of the GPU decode against the BF16 source (any device), in row chunks of whole units."""
+    K, rows = w.meta.K, w.meta.rows
+    unit = max(w.meta.R, 1)
+    src2 = src.reshape(rows, K)
+    step = max(chunk_bytes // (2 * K) // unit * unit, unit)
+    for r0 in range(0, rows, step):
+        nr = min(step, rows - r0)
+        got = dequant(w, r0, nr).view(torch.int16)
+        ref = src2[r0: r0 + nr].to(got.device).view(torch.int16)
+        if not torch.equal(got, ref):
+            return False
+    return True
+
+
+def _mmv_common(x: torch.Tensor, w: Weight, ids: torch.Tensor | None, rows_per_matrix: int, out_bf16: bool, glu: bool,
+                multi_col: bool = True) -> torch.Tensor:
+    cw = _cweight(w)
+    K, rows = w.meta.K, w.meta.rows
+    _check_x(x, K, "x")
+    a = _lib.MmvArgs()
+    a.x = x.data_ptr()
+    a.x_bf16 = int(x.dtype == torch.bfloat16)
+    a.y_bf16 = int(out_bf16)
+    odt = torch.bfloat16 if out_bf16 else torch.float32
+    osz = 2 if out_bf16 else 4
+    a.n_used, a.x_per_slot = 1, 1
+    if ids is None:
+        if x.dim() != 2:
+            raise ValueError("bf16n.mmv: dense x must be [tokens, K]")
+        rpm = rows_per_matrix if rows_per_matrix > 0 else rows
+        if rpm != rows:
+            raise ValueError("bf16n.mmv: a dense product uses the whole matrix")
+        if glu and rpm % 2:
+            raise ValueError("bf16n.mmv_glu: odd row count")
+        n_out = rpm // 2 if glu else rpm
+        T = x.shape[0]
+        y = torch.empty((T, n_out), dtype=odt, device=x.device)
+        if T == 0:
+            return y
+        a.y = y.data_ptr()
+        a.ncols = T
+        a.x_tok = x.stride(0) * x.element_size()
+        a.y_tok = n_out * osz
+        a.rows_per_matrix = rpm
+        a.nrows = n_out
+    else:
+        _check_ids(ids)
+        if ids.device != w.plane.device:
+            raise ValueError("bf16n.mmv: ids on another device")
+        T, n_used = ids.shape
+        if rows_per_matrix <= 0 or rows % rows_per_matrix:
+            raise ValueError("bf16n.mmv: rows_per_matrix must divide the rows")
+        if glu and rows_per_matrix % 2:
+            raise ValueError("bf16n.mmv_glu: odd rows per matrix")
+        n_out = rows_per_matrix // 2 if glu else rows_per_matrix
+        if not ((x.dim() == 2 and x.shape[0] == T) or (x.dim() == 3 and x.shape[0] == T and x.shape[1] == n_used)):
+            raise ValueError("bf16n.mmv: x must be [tokens, K] or [tokens, n_used, K]")
+        y = torch.empty((T, n_used, n_out), dtype=odt, device=x.device)
+        if T == 0 or n_used == 0:
+            return y
+        a.y = y.data_ptr()
+        a.ncols = T * n_used
+        a.ids = ids.data_ptr()
+        a.ids_s0 = ids.element_size()
+        a.ids_s1 = ids.stride(0) * ids.element_size()
+        a.n_used = n_used
+        a.x_tok = x.stride(0) * x.element_size()
+        a.x_per_slot = n_used if x.dim() == 3 else 1
+        a.x_slot = x.stride(1) * x.element_size() if x.dim() == 3 else 0
+        a.y_tok = n_used * n_out * osz
+        a.y_slot = n_out * osz
+        a.rows_per_matrix = rows_per_matrix
+        a.nrows = n_out
+    L = _lib.lib()
+    with torch.cuda.device(x.device):
+        if glu:
+            _lib.check(L.bf16n_mmv_glu(C.byref(cw), C.byref(a), _stream()))
+        else:
+            _lib.check(L.bf16n_mmv(C.byref(cw), C.byref(a), _stream(), int(multi_col)))
+    return y
+
+
+def mmv(x: torch.Tensor, w: Weight, ids: torch.Tensor | None = None, rows_per_matrix: int = 0,
+        out_dtype: torch.dtype = torch.float32, multi_col: bool = True) -> torch.Tensor:
+    return _mmv_common(x, w, ids, rows_per_matrix, out_dtype == torch.bfloat16, False, multi_col)
+
+
+def mmv_glu(x: torch.Tensor, w: Weight, ids: torch.Tensor | None = None, rows_per_matrix: int = 0,
+            out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """silu(gate x) * (up x) for a NIBBLE matrix whose rows per matrix are [gate; up]."""
+    return _mmv_common(x, w, ids, rows_per_matrix or w.meta.rows, out_dtype == torch.bfloat16, True)
+
+
+def mmv_glu2(x: torch.Tensor, gate: Weight, up: Weight, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """silu(gate x) * (up x) for separate dense gate / up matrices (bf16n::mmv_glu(gate, up), core launch.h:61)."""
+    cg, cu = _cweight(gate), _cweight(up)
+    _check_x(x, gate.meta.K, "x")
+    if x.dim() != 2:
+        raise ValueError("bf16n.mmv_glu: dense x must be [tokens, K]")
+    out_bf16 = out_dtype == torch.bfloat16
+    T, n_out = x.shape[0], gate.meta.rows
+    y = torch.empty((T, n_out), dtype=out_dtype, device=x.device)
+    if T == 0:
+        return y
+    a = _lib.MmvArgs()
+    a.x, a.y = x.data_ptr(), y.data_ptr()
+    a.x_bf16, a.y_bf16 = int(x.dtype == torch.bfloat16), int(out_bf16)
+    a.ncols, a.n_used, a.x_per_slot = T, 1, 1
+    a.x_tok = x.stride(0) * x.element_size()
+    a.y_tok = n_out * (2 if out_bf16 else 4)
+    a.rows_per_matrix, a.nrows = n_out, n_out
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().bf16n_mmv_glu2(C.byref(cg), C.byref(cu), C.byref(a), _stream()))
+    return y
+
+
+def linear(x: torch.Tensor, w: Weight, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """y = x W^T (+ bias) in BF16: up to GEMV_MAX_TOKENS tokens through the decode GEMV (FP32 accumulation, the bias
+    added in FP32 before the one rounding to BF16), more through exact dequant in row chunks + a stock BF16 GEMM
+    (core/torch/torch_bindings.cpp:198-239)."""
+    if x.dtype != torch.bfloat16:
+        raise ValueError("bf16n.linear: x must be bf16")
+    K, rows = w.meta.K, w.meta.rows
+    if x.shape[-1] != K:
+        raise ValueError(f"bf16n.linear: x last dim must be K = {K}")
+    oshape = list(x.shape[:-1]) + [rows]
+    x2 = x.reshape(-1, K)
+    T = x2.shape[0]
+    if T <= GEMV_MAX_TOKENS:
+        ok = x2.stride(1) == 1 and (x2.stride(0) * 2) % 16 == 0 and x2.data_ptr() % 16 == 0
+        xc = x2 if ok else x2.contiguous()
+        if bias is not None:
+            y = _mmv_common(xc, w, None, 0, False, False).add_(bias).to(torch.bfloat16)
+        else:
+            y = _mmv_common(xc, w, None, 0, True, False)
+    else:
+        y = torch.empty((T, rows), dtype=x.dtype, device=x.device)
+        unit = 1 if w.meta.format == FMT_NIBBLE else w.meta.R
+        chunk = min(max(DEQUANT_CHUNK_BYTES // (K * 2) // unit * unit, unit), rows)
+        for r0 in range(0, rows, chunk):
+            nr = min(chunk, rows - r0)
+            wc = dequant(w, r0, nr)
+            ys = y.narrow(1, r0, nr)
+            torch.mm(x2, wc.t(), out=ys) if nr != rows else ys.copy_(torch.mm(x2, wc.t()))
+            if bias is not None:
+                ys.add_(bias.narrow(0, r0, nr))
+    return y.view(oshape)
+
+
+def get_rows(ids: torch.Tensor, w: Weight, out_dtype: torch.dtype = torch.bfloat16, row0: int = 0) -> torch.Tensor:
+    cw = _cweight(w)
+    if not ids.is_cuda or ids.dim() != 1:
+        raise ValueError("bf16n.get_rows: ids must be a 1-D device tensor")
+    if ids.dtype not in (torch.int32, torch.int64):
+        raise ValueError("bf16n.get_rows: ids must be int32 or int64")
+    n = ids.shape[0]
+    out = torch.empty((n, w.meta.K), dtype=out_dtype, device=w.plane.device)
+    with torch.cuda.device(w.plane.device):
+        _lib.check(_lib.lib().bf16n_get_rows(C.byref(cw), ids.data_ptr(), ids.stride(0) * ids.element_size(), n,
+                                             out.data_ptr(), int(out_dtype == torch.bfloat16),
+                                             w.meta.K * out.element_size(), _stream(), row0))
+    return out
+
+
+def embedding(ids: torch.Tensor, w: Weight) -> torch.Tensor:
+    flat = ids.reshape(-1)
+    return get_rows(flat, w).view(*ids.shape, w.meta.K)
+
+
+def mm_ids_supported(w: Weight, up: Weight | None = None) -> bool:
+    """Shapes with a batched (prefill) MoE kernel (bf16n::mm_ids_supported, core/src/launch.cu:446-456)."""
+    cw = _cweight(w)
+    cu = _cweight(up) if up is not None else None
+    return bool(_lib.lib().bf16n_mm_ids_supported(C.byref(cw), C.byref(cu) if cu is not None else None))
+
+
+def mm_ids_route(topk_ids: torch.Tensor, n_experts: int, per_slot: bool):
+    """Expert-sorted routing lists on the device (bf16n::mm_ids_route): (ids_src1, ids_dst, bounds) int32."""
+    _check_ids(topk_ids)
+    T, n_used = topk_ids.shape
+    dev = topk_ids.device
+    src1 = torch.empty(T * n_used, dtype=torch.int32, device=dev)
+    dst = torch.empty(T * n_used, dtype=torch.int32, device=dev)
+    bounds = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    nch = n_used if per_slot else 1
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().bf16n_mm_ids_route(topk_ids.data_ptr(), int(topk_ids.dtype == torch.int64), topk_ids.stride(0),
+                                                 src1.data_ptr(), dst.data_ptr(), bounds.data_ptr(), n_experts, T, n_used,
+                                                 nch, nch, _stream()))
+    return src1, dst, bounds
+
+
+def moe_mm_ids(x: torch.Tensor, topk_ids: torch.Tensor, w: Weight, n_experts: int, up: Weight | None = None,
+               out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Batched MUL_MAT_ID over routed tokens (core/torch/torch_bindings.cpp:307-345): x [T, K] (gate / up) or
+    [T, n_used, K] (down), BF16; out [T, n_used, N]; up given: fused gate/up + SwiGLU."""
+    cw = _cweight(w)
+    cu = _cweight(up) if up is not None else None
+    _check_ids(topk_ids)
+    _check_x(x, w.meta.K, "x")
+    if x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError("bf16n.moe_mm_ids: x must be contiguous bf16 (BF16 activations)")
+    if n_experts <= 0 or w.meta.rows % n_experts:
+        raise ValueError("bf16n.moe_mm_ids: rows must split into n_experts")
+    T, n_used = topk_ids.shape
+    N = w.meta.rows // n_experts
+    per_slot = x.dim() == 3
+    if not ((x.dim() == 2 and x.shape[0] == T) or (per_slot and x.shape[0] == T and x.shape[1] == n_used)):
+        raise ValueError("bf16n.moe_mm_ids: x must be [tokens, K] or [tokens, n_used, K]")
+    y = torch.empty((T, n_used, N), dtype=out_dtype, device=x.device)
+    if T == 0:
+        return y
+    L = _lib.lib()
+    if not L.bf16n_mm_ids_supported(C.byref(cw), C.byref(cu) if cu is not None else None):
+        raise ValueError("bf16n.moe_mm_ids: no batched kernel for this matrix (format/K/R/layout)")
+    src1, dst, bounds = mm_ids_route(topk_ids, n_experts, per_slot)
+    with torch.cuda.device(x.device):
+        _lib.check(L.bf16n_mm_ids(C.byref(cw), C.byref(cu) if cu is not None else None, x.data_ptr(), w.meta.K,
+                                  src1.data_ptr(), dst.data_ptr(), bounds.data_ptr(), y.data_ptr(),
+                                  int(out_dtype == torch.bfloat16), N, n_experts, T, n_used, _stream()))
+    return y
+
+
+def moe_combine(ys: torch.Tensor, topk_weights: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    if not (ys.is_cuda and ys.dim() == 3 and ys.dtype == torch.float32 and ys.is_contiguous()):
+        raise ValueError("bf16n.moe_combine: ys must be contiguous f32 [tokens, n_used, N]")
+    if not (topk_weights.is_cuda and topk_weights.dim() == 2 and topk_weights.is_contiguous()
+            and topk_weights.dtype in (torch.float32, torch.bfloat16)):
+        raise ValueError("bf16n.moe_combine: topk_weights must be contiguous f32/bf16 [tokens, n_used]")
+    T, n_used, N = ys.shape
+    if tuple(topk_weights.shape) != (T, n_used):
+        raise ValueError("bf16n.moe_combine: shape mismatch")
+    y = torch.empty((T, N), dtype=out_dtype, device=ys.device)
+    with torch.cuda.device(ys.device):
+        _lib.check(_lib.lib().bf16n_moe_combine(ys.data_ptr(), topk_weights.data_ptr(), int(topk_weights.dtype == torch.bfloat16),
+                                                y.data_ptr(), int(out_dtype == torch.bfloat16), T, n_used, N, _stream()))
+    return y
+
+
+def swiglu(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    if not (g.is_cuda and g.dtype == torch.float32 and g.is_contiguous() and u.shape == g.shape
+            and u.dtype == torch.float32 and u.is_contiguous()):
+        raise ValueError("bf16n.swiglu: g and u must be contiguous f32 of one shape")
+    y = torch.empty_like(g)
+    with torch.cuda.device(g.device):
+        _lib.check(_lib.lib().bf16n_swiglu(g.data_ptr(), u.data_ptr(), y.data_ptr(), g.numel(), _stream()))
+    return y
+
+
+def router_topk(logits: torch.Tensor, k: int, renorm: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+    """Softmax over experts + k largest on the device: (topk_weights f32 [T, k], topk_ids int32 [T, k])."""
+    if not (logits.is_cuda and logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1):
+        raise ValueError("bf16n.router_topk: logits must be f32 [tokens, n_experts], contiguous along experts")
+    T, E = logits.shape
+    ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    wts = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    with torch.cuda.device(logits.device):
+        _lib.check(_lib.lib().bf16n_router_topk(logits.data_ptr(), logits.stride(0), T, E, k, int(renorm), ids.data_ptr(),
+                                                wts.data_ptr(), _stream()))
+    return wts, ids
+
+
+def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_weights: torch.Tensor,
+                topk_ids: torch.Tensor, n_experts: int) -> torch.Tensor:
+    """Routed experts of one MoE layer: sum_k w_k * down(silu(gate x) * up x) over the top-k experts, BF16 out.
+    Up to GEMV_MAX_TOKENS tokens (or shapes without a batched kernel): expert GEMVs with FP32 activations between
+    them; more: the batched kernels (fused gate/up + SwiGLU written as BF16, then down)
+    (engines/vllm/vllm_bf16n/ops.py:251-271)."""
+    T = x.shape[0]
+    N = gate.meta.rows // n_experts
+    H = down.meta.rows // n_experts
+    x = x.contiguous()
+    if T > GEMV_MAX_TOKENS and mm_ids_supported(gate, up) and mm_ids_supported(down):
+        a = moe_mm_ids(x, topk_ids, gate, n_experts, up=up, out_dtype=torch.bfloat16)
+        ys = moe_mm_ids(a, topk_ids, down, n_experts, out_dtype=torch.float32)
+    else:
+        g = mmv(x, gate, topk_ids, N)
+        u = mmv(x, up, topk_ids, N)
+        ys = mmv(swiglu(g, u), down, topk_ids, H)
+    return moe_combine(ys, topk_weights, torch.bfloat16)
+
+
+def moe_experts_reference(x, gate, up, down, topk_weights, topk_ids, n_experts):
+    """Exact-weight reference in FP32 (dequant per used expert): slow, for tests
+    (engines/vllm/vllm_bf16n/ops.py:274-287)."""
+    N = gate.meta.rows // n_experts
+    H = down.meta.rows // n_experts
+    xf = x.float()
+    out = torch.zeros(x.shape[0], H, dtype=torch.float32, device=x.device)
+    for e in torch.unique(topk_ids).tolist():
+        tok, slot = (topk_ids == e).nonzero(as_tuple=True)
+        g = dequant(gate, e * N, N).float()
+        u = dequant(up, e * N, N).float()
+        d = dequant(down, e * H, H).float()
+        a = torch.nn.functional.silu(xf[tok] @ g.t()) * (xf[tok] @ u.t())
+        out.index_add_(0, tok, (a @ d.t()) * topk_weights[tok, slot].float()[:, None])
+    return out.to(torch.bfloat16)
