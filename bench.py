@@ -1,0 +1,164 @@
+"""Benchmark of the BF16N hot path on one MI355X.
+
+A step is one fused decode+GEMV over the output projection (248320 x 2048 BF16 weights N(0, 0.02), HUFPAIR, one BF16
+activation vector N(0, 1), FP32 accumulation, FP32 output) with the encoded weights resident in HBM.  Two copies of the
+weights at different addresses are used in turn so that the 256 MB last-level cache does not serve the stream.
+Reported: compressed bytes per second (metric), the roofline of the GEMV kernel on algorithmic bytes, the BF16 GEMV of
+the stock BLAS on the uncompressed tensor, and the CPU restatement (oracle) of decode+GEMV on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--rows R] [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def gen_weights(rows: int, K: int, seed: int):
+    """N(0, 0.02) -> BF16 (RNE) on the GPU, returned as a CPU bf16 tensor and kept on the device for the BLAS baseline."""
+    import torch
+
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    w = torch.empty((rows, K), dtype=torch.bfloat16, device="cuda")
+    step = 1 << 15
+    for r0 in range(0, rows, step):
+        n = min(step, rows - r0)
+        w[r0: r0 + n] = (torch.randn((n, K), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    return w
+
+
+def time_kernel(fn, steps: int, warmup: int):
+    """Per-launch durations (ms) from HIP events recorded on the launch stream, and the wall time of the timed region."""
+    import torch
+
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev[i][0].record()
+        fn(i)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return [a.elapsed_time(b) for a, b in ev], wall
+
+
+def cpu_baseline(wbits, K: int, xf, sample_rows: int):
+    """The oracle's decode+GEMV (reference layout, R = 16) on the first sample_rows rows, all host threads available
+    to this process (capped at 16)."""
+    import numpy as np
+
+    from oracle import pyoracle as O
+    from orin_qwen_lossless_amd import ops
+
+    threads = max(1, min(16, len(os.sched_getaffinity(0))))
+    sub = np.ascontiguousarray(wbits[:sample_rows])
+    plane, aux, _, _ = ops.encode_bits(sub, 3, 16, False)
+    nbytes = plane.size + aux.size
+    O.decode_gemv(plane, aux, xf, 0, sample_rows, threads)  # warm-up
+    reps, t_total, best = 0, 0.0, None
+    while t_total < 12.0 and reps < 200:
+        t0 = time.perf_counter()
+        O.decode_gemv(plane, aux, xf, 0, sample_rows, threads)
+        dt = time.perf_counter() - t0
+        t_total += dt
+        reps += 1
+        best = dt if best is None else min(best, dt)
+    med = t_total / reps
+    return {"value": round(nbytes / med / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"first {sample_rows} of the workload's rows ({sample_rows}x{K}, HUFPAIR R=16 reference layout, "
+                      f"{nbytes} compressed bytes), mean of {reps} runs ({med * 1e3:.1f} ms each, best {best * 1e3:.1f} ms)"}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--rows", type=int, default=248320)
+    ap.add_argument("--K", type=int, default=2048)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=16384)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU (the path has no collective); run with --gpus 1")
+
+    import numpy as np
+    import torch
+
+    from orin_qwen_lossless_amd import ops
+
+    torch.cuda.set_device(0)
+    ops.init()
+    rows, K = args.rows, args.K
+    t0 = time.perf_counter()
+    w_dev = gen_weights(rows, K, seed=1)
+    w_cpu = w_dev.cpu()
+    wbits = w_cpu.view(torch.int16).numpy().view(np.uint16)
+    fmt, R, cm, _, w64 = ops.choose(rows, K, engine="mi355x")
+    t1 = time.perf_counter()
+    plane, aux, fmt_out, _ = ops.encode_bits(wbits, fmt, R, cm, wave64=w64)
+    t_enc = time.perf_counter() - t1
+    ta = torch.from_numpy(aux)
+    meta = ops.parse_header(ta)
+    copies = [ops.upload(torch.from_numpy(plane), ta, meta, "cuda") for _ in range(2)]
+    assert ops.roundtrip_equal(copies[0], w_dev), "GPU decode is not bit-exact"  # the load-time verify, before timing
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn((1, K), generator=g, device="cuda").to(torch.bfloat16)
+    y = ops.mmv(x, copies[0])
+    ref = (w_dev.float() @ x[0].float())
+    err = float(((y[0] - ref).abs() / (w_dev.float().abs() @ x[0].float().abs())).max())
+    assert err < 1e-5, f"GEMV error {err}"
+
+    comp_bytes = plane.size + aux.size
+    algo_bytes = comp_bytes + K * 2 + rows * 4  # weights (plane + aux incl. table, unit bases, padding) + x + y
+    durs, wall = time_kernel(lambda i: ops.mmv(x, copies[i & 1]), args.steps, args.warmup)
+    ms = wall * 1e3 / args.steps
+    kern_ms = float(np.mean(durs))
+    # stock BF16 GEMV on the uncompressed tensor (the "vs BF16" column), same timing loop
+    w2 = [w_dev, w_dev.clone()]
+    xt = x[0].contiguous()
+    bd, _ = time_kernel(lambda i: torch.mv(w2[i & 1], xt), min(args.steps, 100), 10)
+    blas_us = float(np.median(bd)) * 1e3
+
+    out = {
+        "metric": "fused decode+GEMV HBM GB/s (% peak, compressed bytes); us/decode step vs BF16",
+        "value": round(comp_bytes / (ms * 1e-3) / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"output projection {rows}x{K} BF16 N(0,0.02), {ops.FORMAT_NAMES[fmt_out]} R={R} "
+                               f"{'wave64' if w64 else 'reference'} layout, fused decode+GEMV, batch 1 BF16 activations "
+                               "N(0,1), FP32 accumulate/out; 2 weight copies alternated",
+                   "rows": rows, "K": K, "batch": 1, "compressed_bytes": comp_bytes, "bits_per_weight": round(8 * comp_bytes / (rows * K), 4),
+                   "ratio_of_bf16": round(comp_bytes / (2 * rows * K), 4)},
+        "roofline": {"bound": "hbm", "achieved": round(algo_bytes / (kern_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_w64_mmv<bf16,4,1>", "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 2),
+                     "median_launch_us": round(float(np.median(durs)) * 1e3, 2)},
+        "extra": {"pct_of_hbm_peak_compressed": round(100 * comp_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+                  "us_per_matrix": round(ms * 1e3, 2), "blas_bf16_gemv_us": round(blas_us, 2),
+                  "speedup_vs_blas_bf16": round(blas_us / (ms * 1e3), 3), "tokens_per_s_lm_head_only": round(1e3 / ms, 1),
+                  "host_encode_s": round(t_enc, 2), "max_err_over_sum_abs": err, "setup_s": round(time.perf_counter() - t0, 1)},
+    }
+    if not args.no_cpu:
+        xf = x[0].float().cpu().numpy()
+        out["cpu_baseline"] = cpu_baseline(wbits, K, xf, min(args.cpu_rows, rows // 16 * 16))
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
