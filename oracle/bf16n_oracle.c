@@ -443,10 +443,10 @@ int orc_decode(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, uin
  * 32..63 chunk 2i+1 of step i, each with the reference (lane, slot) ownership, so the plane is the reference plane.
  * Every lane has a bit sequence: 2 zero bits, then its pair codes, each code written first-bit-lowest; 32-bit word k of
  * the lane holds sequence bits [32k, 32k+32) with bit j of the word = sequence bit 32k+j.  The LUT at off_a is indexed
- * by the next 12 sequence bits (first bit = index bit 0).  A lane holds two words (w0, w1) and a position P into w0;
- * after every second pair it adds the two code lengths to P and, if P >= 32, takes the unit stream's next word
- * (lanes in ascending order) as its new w1, moves the old w1 to w0 and subtracts 32.  The unit stream is: the lanes'
- * first two words (lane 0 word 0, lane 0 word 1, lane 1 word 0, ...), then the refill words in the order taken.
+ * by the next 12 sequence bits (first bit = index bit 0).  A lane holds three words (w0, w1, w2) and a position P into
+ * w0; after every second pair it adds the two code lengths to P and, if P >= 32, takes the unit stream's next word
+ * (lanes in ascending order) as its new w2, moves w2 to w1 and w1 to w0 and subtracts 32.  The unit stream is: the
+ * lanes' first three words (lane 0 words 0, 1, 2, lane 1 words 0, 1, 2, ...), then the refill words in the order taken.
  * off_b: u32 unit_base[units + 1] (word index of each unit's stream), off_d: words. */
 int orc_decode_w64(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, uint16_t *out) {
     orc_header h;
@@ -458,8 +458,11 @@ int orc_decode_w64(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes,
     if ((R * C) % 2) return -1;
     for (uint64_t u = 0; u < h.n_a; u++) {
         uint64_t next = h.off_d + 4ull * rd32(aux, h.off_b + 4 * u);
-        uint32_t w0[64], w1[64], P[64];
-        for (int l = 0; l < 64; l++) { w0[l] = rd32(aux, next); w1[l] = rd32(aux, next + 4); next += 8; P[l] = 0; }
+        uint32_t w0[64], w1[64], w2[64], P[64];
+        for (int l = 0; l < 64; l++) {
+            w0[l] = rd32(aux, next); w1[l] = rd32(aux, next + 4); w2[l] = rd32(aux, next + 8);
+            next += 12; P[l] = 0;
+        }
         for (int64_t step = 0; step < R * C / 2; step++) {
             for (int q = 0; q < 8; q += 2) {
                 for (int l = 0; l < 64; l++) {
@@ -481,7 +484,7 @@ int orc_decode_w64(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes,
                 for (int l = 0; l < 64; l++)
                     if (P[l] >= 32) {
                         if (next + 4 > aux_bytes) return -1;
-                        w0[l] = w1[l]; w1[l] = rd32(aux, next); next += 4; P[l] -= 32;
+                        w0[l] = w1[l]; w1[l] = w2[l]; w2[l] = rd32(aux, next); next += 4; P[l] -= 32;
                     }
             }
         }

@@ -543,14 +543,15 @@ std::vector<uint8_t> encode_hufpair(const uint16_t * w, int64_t rows, int64_t K,
 //
 // Every lane has a bit sequence: 2 zero bits, then its pair codes in order, each written with its first (most
 // significant) code bit lowest.  Word k of the lane holds sequence bits [32k, 32k + 32), sequence bit 32k + j in bit
-// j.  The decoder keeps two words per lane (w0, w1) and a position P < 32 into w0; the next code's table index is
-// bits [P + 2, P + 14) of w1:w0.  After every second pair it adds the two code lengths to P; every lane with P >= 32
-// then takes the next word of the unit's stream (lanes in ascending order) as its new w1, the old w1 becomes w0 and P
-// drops by 32.  The unit's stream is therefore: words 0 and 1 of lane 0, of lane 1, ... of lane 63, then the refill
-// words in exactly the order the decoder takes them — a wave reads it front to back with coalesced loads, and the lane
-// of a refill word is its rank among the refilling lanes.  The table at off_a is indexed by those 12 bits as they
-// sit in the word (first code bit = index bit 0), i.e. the canonical table with bit-reversed index.
-// unit_base has units + 1 entries (word index of each unit's first word and the end).
+// j.  The decoder keeps three words per lane (w0, w1, w2) and a position P < 32 into w0; the next code's table index
+// is bits [P + 2, P + 14) of w1:w0.  After every second pair it adds the two code lengths to P; every lane with
+// P >= 32 then takes the next word of the unit's stream (lanes in ascending order) as its new w2, the old w2 becomes
+// w1, the old w1 becomes w0, and P drops by 32 (the word taken is not needed before the next such check, so its read
+// overlaps the table lookups in between).  The unit's stream is therefore: words 0, 1, 2 of lane 0, of lane 1, ... of
+// lane 63, then the refill words in exactly the order the decoder takes them — a wave reads it front to back with
+// coalesced loads, and the lane of a refill word is its rank among the refilling lanes.  The table at off_a is
+// indexed by those 12 bits as they sit in the word (first code bit = index bit 0), i.e. the canonical table with
+// bit-reversed index.  unit_base has units + 1 entries (word index of each unit's first word and the end).
 std::vector<uint8_t> encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, bool cm) {
     pair_code pc;
     if (!build_pair_code(w, rows, K, pc)) {
@@ -566,7 +567,7 @@ std::vector<uint8_t> encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_
         s0 = sym_at(base + pos_of(l & 31, 4 * t));
         s1 = sym_at(base + pos_of(l & 31, 4 * t + 2));
     };
-    // pass 1: words per unit = 128 + number of refills
+    // pass 1: words per unit = 192 + number of refills
     std::vector<uint64_t> ubase(units + 1, 0);
     parallel_blocks(units, 8, [&](int64_t u0, int64_t u1) {
         for (int64_t u = u0; u < u1; u++) {
@@ -585,7 +586,7 @@ std::vector<uint8_t> encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_
                     }
                 }
             }
-            ubase[u + 1] = 128 + refills;
+            ubase[u + 1] = 192 + refills;
         }
     });
     for (int64_t u = 0; u < units; u++) {
@@ -655,10 +656,11 @@ std::vector<uint8_t> encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_
             uint32_t * out = stream + ubase[u];
             for (int l = 0; l < 64; l++) {
                 lane_bits[l].push_back((uint32_t) acc[l]); // partial last word, zero-filled
-                lane_bits[l].resize(lane_bits[l].size() + 3, 0);
+                lane_bits[l].resize(lane_bits[l].size() + 4, 0);
                 *out++ = lane_bits[l][0];
                 *out++ = lane_bits[l][1];
-                taken[l] = 2;
+                *out++ = lane_bits[l][2];
+                taken[l] = 3;
             }
             for (uint8_t l : order) {
                 *out++ = lane_bits[l][taken[l]++];

@@ -7,7 +7,8 @@
 //   * the unit streams: one word stream per unit, consumed front to back.  The wave copies it in 1 KiB blocks into a
 //     private ring in LDS (coalesced 16-byte loads, one block in flight in registers) and every lane that needs a new
 //     word after a pair of codes reads ring[consumed + rank among the refilling lanes] — consecutive addresses, no bank
-//     conflicts, no per-lane pointers;
+//     conflicts, no per-lane pointers.  A lane buffers three words, so a requested word is not needed before the next
+//     check and its LDS read overlaps the table lookups in between;
 //   * the 4096-entry pair table sits in LDS once per block; an entry already holds both exponents in BF16 position, so
 //     one v_perm + one v_bfi turn two plane bytes and an entry into two BF16 weights.
 // Activations stay in registers for the whole kernel (a lane always meets the same columns), products are accumulated in
@@ -20,11 +21,12 @@ namespace dev {
 
 namespace {
 
-constexpr int RING = 1024;    // ring words per wave (4 KiB)
-constexpr int RING_PAD = 128; // copy of the first ring words behind the end: reads never wrap
+constexpr int RING = 512;     // ring words per wave (2 KiB)
+constexpr int RING_PAD = 256; // copy of the first ring words behind the end: reads never wrap
 constexpr int BLK = 256;      // words per refill block: one uint4 per lane
-constexpr int AHEAD = 640;    // words kept ahead of the consumer: a unit start (128) + a step (4 x 64) and one block
+constexpr int AHEAD = 256;    // words kept ahead of the consumer: a unit start (192) or a step (4 x 64)
 constexpr int LUT_WORDS = 1 << HP_LP;
+constexpr int WAVE_LDS_WORDS = RING + RING_PAD;
 
 struct w64_ptrs { const uint8_t * plane; const uint32_t * lut; const uint32_t * ubase; const uint32_t * stream; };
 __device__ __forceinline__ w64_ptrs w64p(const bf16n_weight & w) {
@@ -34,16 +36,19 @@ __device__ __forceinline__ w64_ptrs w64p(const bf16n_weight & w) {
 __device__ __forceinline__ uint32_t lds_entry(const uint32_t * lut, uint32_t byte_off) {
     return *(const uint32_t *) ((const char *) lut + byte_off);
 }
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t) __builtin_amdgcn_readfirstlane((int) v); }
 
-// Decoder state of one wave.  cons / filled / limit are the same in every lane (kept in scalar registers).
+// Decoder state of one wave.  cons / filled / limit are the same in every lane (scalar registers).
 struct w64_dec {
-    uint32_t w0, w1, P; // per lane: two stream words and the bit position in w0 (< 32)
-    uint32_t cons;      // words consumed, relative to src
-    uint32_t filled;    // words copied into the ring, relative to src (multiple of BLK)
-    uint32_t limit;     // end of this wave's streams, relative to src
+    uint32_t w0, w1, w2, P; // per lane: three stream words and the bit position in w0 (< 32)
+    uint32_t nw;            // the word requested at the last check (becomes w2 where took is set)
+    bool took;              // this lane requested a word at the last check
+    uint32_t cons;          // words consumed, relative to src
+    uint32_t filled;        // words copied into the ring, relative to src (multiple of BLK)
+    uint32_t limit;         // end of this wave's streams, relative to src
     uint32_t * ring;
-    const uint32_t * src; // 16-byte aligned
-    uint4 pend;           // block filled / BLK, in flight
+    const uint32_t * src;   // 16-byte aligned
+    uint4 pend;             // the block that starts at `filled`, in flight
     int lane;
 
     __device__ __forceinline__ uint4 load_block(uint32_t first_word) const {
@@ -56,7 +61,7 @@ struct w64_dec {
     __device__ __forceinline__ void store_block(uint32_t first_word, const uint4 v) {
         const uint32_t off = first_word & (RING - 1);
         *((uint4 *) (ring + off) + lane) = v;
-        if (off == 0 && lane < RING_PAD / 4) {
+        if (off == 0) {
             *((uint4 *) (ring + RING) + lane) = v;
         }
     }
@@ -68,12 +73,10 @@ struct w64_dec {
         src = stream + a;
         cons = first - a;
         limit = end - a;
-        const uint4 b0 = load_block(0), b1 = load_block(BLK), b2 = load_block(2 * BLK);
-        pend = load_block(3 * BLK);
+        const uint4 b0 = load_block(0);
+        pend = load_block(BLK);
         store_block(0, b0);
-        store_block(BLK, b1);
-        store_block(2 * BLK, b2);
-        filled = 3 * BLK;
+        filled = BLK;
     }
     __device__ __forceinline__ void keep_ahead() {
         while (filled - cons < AHEAD) {
@@ -83,13 +86,16 @@ struct w64_dec {
         }
     }
     __device__ __forceinline__ void begin_unit() {
-        const uint32_t * p = ring + (cons & (RING - 1)) + 2 * lane;
+        const uint32_t * p = ring + (cons & (RING - 1)) + 3 * lane;
         w0 = p[0];
         w1 = p[1];
+        w2 = p[2];
         P = 0;
-        cons += 128;
+        took = false;
+        nw = 0;
+        cons = uniform(cons + 192);
     }
-    // two pair codes; afterwards lanes whose position passed a word boundary take the next stream words in lane order
+    // two pair codes; afterwards lanes whose position passed a word boundary request the next stream words in lane order
     __device__ __forceinline__ void two(const uint32_t * lut, uint32_t & e0, uint32_t & e1) {
         const uint32_t W = __builtin_amdgcn_alignbit(w1, w0, P);
         e0 = lds_entry(lut, W & 0x3FFCu);
@@ -99,11 +105,15 @@ struct w64_dec {
         const bool need = P >= 32u;
         const uint64_t m = __ballot(need);
         const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
-        const uint32_t nw = ring[(cons & (RING - 1)) + rank];
+        const uint32_t req = ring[(cons & (RING - 1)) + rank];
+        // the word requested one check ago has arrived by now: it is this lane's w2
+        w2 = took ? nw : w2;
         w0 = need ? w1 : w0;
-        w1 = need ? nw : w1;
+        w1 = need ? w2 : w1;
+        nw = req;
+        took = need;
         P &= 31u;
-        cons += (uint32_t) __builtin_popcountll(m);
+        cons = uniform(cons + (uint32_t) __builtin_popcountll(m));
     }
     // the 16 weights of this lane in one step as 8 BF16 pairs: wp[2j], wp[2j+1] = columns 128j + 4(lane%32) + {0,1}, {2,3}
     __device__ __forceinline__ void step(const uint32_t * lut, const uint4 sm, uint32_t (&wp)[8]) {
@@ -176,15 +186,129 @@ template <int C> struct geom {
     static constexpr int ROWS = C == 1 ? 4 : C == 2 ? 2 : 1; // rows per body
 };
 
-template <typename TX, int C, int NC>
+// One decode chain of a wave: a contiguous range of units with its own stream ring, plane pointer and row counter.
+template <int NB>
+struct chain {
+    w64_dec dec;
+    const uint4 * pp;      // next plane step to load, + 64 per step
+    uint4 sm[NB];          // plane bytes of the body's steps
+    int64_t steps_left;    // steps not yet loaded
+    int64_t row;           // output row of the next body, relative to the product
+    __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t gu0, int64_t n_units, int64_t row0, int R, int K,
+                                          int lane) {
+        dec.start(ring, q.stream, q.ubase[gu0], q.ubase[gu0 + n_units], lane);
+        pp = (const uint4 *) (q.plane + gu0 * R * K) + lane;
+        steps_left = n_units * R * (K / CHUNK) / 2;
+        row = row0;
+#pragma unroll
+        for (int s = 0; s < NB; s++) {
+            sm[s] = pp[64 * s]; // a unit holds whole bodies, so the first NB steps exist
+        }
+        pp += 64 * NB;
+        steps_left -= NB;
+    }
+    // plane bytes of step s of the next body, once step s of this body is consumed
+    __device__ __forceinline__ void reload(int s) {
+        if (steps_left > 0) {
+            sm[s] = pp[0];
+        }
+        pp += 64;
+        steps_left--;
+    }
+};
+
+// N chains advance one unit each, instruction streams interleaved: while one chain waits for a table lookup the
+// other one issues.
+template <typename TX, int C, int NC, int N>
+__device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uint32_t * lut, const xchunk<TX> (&xr)[NC][geom<C>::XS],
+                                          const cols & p, const col_view & cv, int R, int lane) {
+    using G = geom<C>;
+    const int l32 = lane & 31, half = lane >> 5;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        ch[k].dec.keep_ahead();
+        ch[k].dec.begin_unit();
+    }
+    const int bodies = R * C / 2 / G::NB;
+    for (int b = 0; b < bodies; b++) {
+        float acc[N][NC][G::NB];
+#pragma unroll
+        for (int s = 0; s < G::NB; s++) {
+            uint32_t wp[N][8];
+            uint32_t smw[N][4];
+#pragma unroll
+            for (int k = 0; k < N; k++) {
+                ch[k].dec.keep_ahead();
+                smw[k][0] = ch[k].sm[s].x; smw[k][1] = ch[k].sm[s].y; smw[k][2] = ch[k].sm[s].z; smw[k][3] = ch[k].sm[s].w;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+#pragma unroll
+                for (int k = 0; k < N; k++) {
+                    uint32_t e0, e1;
+                    ch[k].dec.two(lut, e0, e1);
+                    wp[k][2 * j] = merge(spread_lo(smw[k][j]), e0);
+                    wp[k][2 * j + 1] = merge(spread_hi(smw[k][j]), e1);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < N; k++) {
+                ch[k].reload(s);
+#pragma unroll
+                for (int n = 0; n < NC; n++) {
+                    if (C >= 4) {
+                        acc[k][n][0] = xr[n][s].dot(wp[k], s == 0 ? 0.f : acc[k][n][0]);
+                    } else {
+                        acc[k][n][s] = xr[n][0].dot(wp[k], 0.f);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < N; k++) {
+            const int64_t row = ch[k].row;
+#pragma unroll
+            for (int n = 0; n < NC; n++) {
+                char * y = cv.y + n * p.y_tok;
+                if (C >= 4) { // a body is one row
+                    const float v = wave_sum(acc[k][n][0]);
+                    if (lane == 0) {
+                        store_y(y, p.y_bf16, row, v);
+                    }
+                } else if (C == 2) { // a step is one row
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+                        const float v = wave_sum(acc[k][n][s]);
+                        if (lane == 0) {
+                            store_y(y, p.y_bf16, row + s, v);
+                        }
+                    }
+                } else { // a step is rows 2s (lanes 0..31) and 2s + 1 (lanes 32..63)
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+                        const float v = half_wave_sum(acc[k][n][s]);
+                        if (l32 == 0) {
+                            store_y(y, p.y_bf16, row + 2 * s + half, v);
+                        }
+                    }
+                }
+            }
+            ch[k].row += G::ROWS;
+        }
+    }
+}
+
+// NCH = 2: a wave splits its units into two halves decoded as two interleaved chains (twice the independent work per
+// wave to cover LDS latency); NCH = 1 where a wave has a single unit.
+template <typename TX, int C, int NC, int NCH>
 __global__ void __launch_bounds__(1024) k_w64_mmv(const bf16n_weight w, const cols p, int units_per_wave) {
     using G = geom<C>;
     constexpr int K = C * CHUNK;
-    extern __shared__ __align__(16) uint32_t shm[];
-    uint32_t * lut = shm;
+    __shared__ __align__(16) uint32_t lut[LUT_WORDS];          // static: sits at LDS address 0
+    extern __shared__ __align__(16) uint32_t rings[];          // per wave and chain: RING + RING_PAD words
     const w64_ptrs q = w64p(w);
     stage_lut(lut, q.lut);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int R = w.R;
     const col_view cv = col_setup(p, blockIdx.y * NC);
@@ -204,71 +328,19 @@ __global__ void __launch_bounds__(1024) k_w64_mmv(const bf16n_weight w, const co
         return;
     }
     const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
+    const int64_t n = u_end - u_begin, nA = NCH == 2 ? (n + 1) / 2 : n, nB = n - nA;
     const int64_t gu0 = cv.rbase / R + u_begin;
-    w64_dec dec;
-    dec.start(shm + LUT_WORDS + wave * (RING + RING_PAD), q.stream, q.ubase[gu0], q.ubase[gu0 + (u_end - u_begin)], lane);
-    const uint4 * pp = (const uint4 *) (q.plane + gu0 * R * K) + lane; // + 64 per step
-    const int64_t steps_total = (u_end - u_begin) * R * C / 2;
-    int64_t steps_loaded = G::NB;
-    uint4 sm[G::NB];
-#pragma unroll
-    for (int s = 0; s < G::NB; s++) {
-        sm[s] = pp[64 * s];
+    chain<G::NB> ch[2];
+    uint32_t * ring = rings + wave * (NCH * WAVE_LDS_WORDS);
+    ch[0].start(ring, q, gu0, nA, u_begin * R, R, K, lane);
+    if (NCH == 2 && nB > 0) {
+        ch[1].start(ring + WAVE_LDS_WORDS, q, gu0 + nA, nB, (u_begin + nA) * R, R, K, lane);
     }
-    pp += 64 * G::NB;
-    const int bodies_per_unit = R * C / 2 / G::NB;
-    int64_t row = u_begin * R; // output row of the body's first row, relative to the product
-    for (int64_t u = u_begin; u < u_end; u++) {
-        dec.keep_ahead();
-        dec.begin_unit();
-        for (int b = 0; b < bodies_per_unit; b++, row += G::ROWS) {
-            float acc[NC][G::NB];
-#pragma unroll
-            for (int s = 0; s < G::NB; s++) {
-                dec.keep_ahead();
-                uint32_t wp[8];
-                dec.step(lut, sm[s], wp);
-                if (steps_loaded < steps_total) { // the same step of the next body
-                    sm[s] = pp[0];
-                }
-                pp += 64;
-                steps_loaded++;
-#pragma unroll
-                for (int n = 0; n < NC; n++) {
-                    const int xi = C >= 4 ? s : 0;
-                    if (C >= 4) {
-                        acc[n][0] = xr[n][xi].dot(wp, s == 0 ? 0.f : acc[n][0]);
-                    } else {
-                        acc[n][s] = xr[n][xi].dot(wp, 0.f);
-                    }
-                }
-            }
-#pragma unroll
-            for (int n = 0; n < NC; n++) {
-                char * y = cv.y + n * p.y_tok;
-                if (C >= 4) {
-                    const float v = wave_sum(acc[n][0]);
-                    if (lane == 0) {
-                        store_y(y, p.y_bf16, row, v);
-                    }
-                } else if (C == 2) {
-#pragma unroll
-                    for (int s = 0; s < 2; s++) {
-                        const float v = wave_sum(acc[n][s]);
-                        if (lane == 0) {
-                            store_y(y, p.y_bf16, row + s, v);
-                        }
-                    }
-                } else { // a step = rows 2s (lanes 0..31) and 2s + 1 (lanes 32..63)
-#pragma unroll
-                    for (int s = 0; s < 2; s++) {
-                        const float v = half_wave_sum(acc[n][s]);
-                        if (l32 == 0) {
-                            store_y(y, p.y_bf16, row + 2 * s + half, v);
-                        }
-                    }
-                }
-            }
+    for (int64_t i = 0; i < nA; i++) {
+        if (NCH == 2 && i < nB) {
+            unit_pass<TX, C, NC, 2>(ch, lut, xr, p, cv, R, lane);
+        } else {
+            unit_pass<TX, C, NC, 1>(ch, lut, xr, p, cv, R, lane);
         }
     }
 }
@@ -308,12 +380,12 @@ __device__ __forceinline__ void w64_unit_rows(w64_dec & dec, const uint32_t * lu
 
 __global__ void __launch_bounds__(256) k_w64_dequant(const bf16n_weight w, int64_t row0, int64_t nrows, uint16_t * __restrict__ out,
                                                      int units_per_wave) {
-    extern __shared__ __align__(16) uint32_t shm[];
-    uint32_t * lut = shm;
+    __shared__ __align__(16) uint32_t lut[LUT_WORDS];
+    extern __shared__ __align__(16) uint32_t rings[];
     const w64_ptrs q = w64p(w);
     stage_lut(lut, q.lut);
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
     const int R = w.R, K = (int) w.K, C = K / CHUNK;
     const int64_t units = nrows / R;
     const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
@@ -323,7 +395,7 @@ __global__ void __launch_bounds__(256) k_w64_dequant(const bf16n_weight w, int64
     const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
     const int64_t gu0 = row0 / R + u_begin;
     w64_dec dec;
-    dec.start(shm + LUT_WORDS + wave * (RING + RING_PAD), q.stream, q.ubase[gu0], q.ubase[gu0 + (u_end - u_begin)], lane);
+    dec.start(rings + wave * WAVE_LDS_WORDS, q.stream, q.ubase[gu0], q.ubase[gu0 + (u_end - u_begin)], lane);
     for (int64_t u = u_begin; u < u_end; u++) {
         dec.keep_ahead();
         dec.begin_unit();
@@ -334,12 +406,12 @@ __global__ void __launch_bounds__(256) k_w64_dequant(const bf16n_weight w, int64
 
 __global__ void __launch_bounds__(256) k_w64_get_rows(const bf16n_weight w, const char * __restrict__ ids, int64_t ids_s0, int64_t n,
                                                       int64_t row0, char * __restrict__ dst, int64_t dst_s1, bool f32) {
-    extern __shared__ __align__(16) uint32_t shm[];
-    uint32_t * lut = shm;
+    __shared__ __align__(16) uint32_t lut[LUT_WORDS];
+    extern __shared__ __align__(16) uint32_t rings[];
     const w64_ptrs q = w64p(w);
     stage_lut(lut, q.lut);
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
     const int R = w.R, K = (int) w.K, C = K / CHUNK;
     const int64_t i = (int64_t) blockIdx.x * nwaves + wave;
     if (i >= n) {
@@ -348,22 +420,25 @@ __global__ void __launch_bounds__(256) k_w64_get_rows(const bf16n_weight w, cons
     const int64_t gr = row0 + *(const int32_t *) (ids + i * ids_s0);
     const int64_t gu = gr / R;
     w64_dec dec;
-    dec.start(shm + LUT_WORDS + wave * (RING + RING_PAD), q.stream, q.ubase[gu], q.ubase[gu + 1], lane);
+    dec.start(rings + wave * WAVE_LDS_WORDS, q.stream, q.ubase[gu], q.ubase[gu + 1], lane);
     dec.keep_ahead();
     dec.begin_unit();
     w64_unit_rows(dec, lut, q.plane + gu * R * (int64_t) K, R, C, lane, gr - gu * R, dst + i * dst_s1, 0, f32);
 }
 
-size_t w64_shm(int waves) { return (size_t) (LUT_WORDS + waves * (RING + RING_PAD)) * 4; }
+size_t w64_shm(int waves) { return (size_t) waves * WAVE_LDS_WORDS * 4; } // dynamic part; the table is static
 
 // waves per block and units per wave for `units` units per column: every wave gets the same number of units (but the
 // last), and a launch fills the device once when it can
 void w64_dims(int64_t units, int ncols, int cus, int & waves_per_block, int & blocks, int & units_per_wave) {
     int64_t max_waves = (int64_t) cus * 16 / (ncols < 1 ? 1 : ncols);
     max_waves = max_waves < 16 ? 16 : max_waves;
-    const int64_t upw = (units + max_waves - 1) / max_waves;
+    int64_t upw = (units + max_waves - 1) / max_waves;
+    if (upw > 1 && (upw & 1)) {
+        upw++; // two chains per wave: an even split
+    }
     const int64_t waves = (units + upw - 1) / upw;
-    waves_per_block = waves >= 16 * (int64_t) cus ? 16 : waves >= 8 * (int64_t) cus ? 8 : 4;
+    waves_per_block = waves >= 8 * (int64_t) cus ? 8 : 4;
     if (waves < waves_per_block) {
         waves_per_block = (int) waves;
     }
@@ -378,27 +453,36 @@ constexpr int max_group() {
     return 64 / per_col < 1 ? 1 : 64 / per_col > 4 ? 4 : 64 / per_col;
 }
 
+template <typename TX, int C, int NC>
+void mmv_launch(dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
+    if (upw >= 2) {
+        hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 2>), grid, dim3(nt), w64_shm(2 * wpb), stream, w, p, upw);
+    } else {
+        hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 1>), grid, dim3(nt), w64_shm(wpb), stream, w, p, upw);
+    }
+}
+
 template <typename TX, int C>
-void mmv_nc(int nc, dim3 grid, int nt, size_t shm, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
+void mmv_nc(int nc, dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
     constexpr int G = max_group<TX, C>();
     if (nc == 1) {
-        hipLaunchKernelGGL((k_w64_mmv<TX, C, 1>), grid, dim3(nt), shm, stream, w, p, upw);
+        mmv_launch<TX, C, 1>(grid, nt, wpb, stream, w, p, upw);
     } else if (nc == 2) {
-        if constexpr (G >= 2) hipLaunchKernelGGL((k_w64_mmv<TX, C, 2>), grid, dim3(nt), shm, stream, w, p, upw);
+        if constexpr (G >= 2) mmv_launch<TX, C, 2>(grid, nt, wpb, stream, w, p, upw);
     } else if (nc == 3) {
-        if constexpr (G >= 3) hipLaunchKernelGGL((k_w64_mmv<TX, C, 3>), grid, dim3(nt), shm, stream, w, p, upw);
+        if constexpr (G >= 3) mmv_launch<TX, C, 3>(grid, nt, wpb, stream, w, p, upw);
     } else {
-        if constexpr (G >= 4) hipLaunchKernelGGL((k_w64_mmv<TX, C, 4>), grid, dim3(nt), shm, stream, w, p, upw);
+        if constexpr (G >= 4) mmv_launch<TX, C, 4>(grid, nt, wpb, stream, w, p, upw);
     }
 }
 
 template <typename TX>
-void mmv_c(int C, int nc, dim3 grid, int nt, size_t shm, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
+void mmv_c(int C, int nc, dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
     switch (C) {
-        case 1: mmv_nc<TX, 1>(nc, grid, nt, shm, stream, w, p, upw); break;
-        case 2: mmv_nc<TX, 2>(nc, grid, nt, shm, stream, w, p, upw); break;
-        case 4: mmv_nc<TX, 4>(nc, grid, nt, shm, stream, w, p, upw); break;
-        default: mmv_nc<TX, 8>(nc, grid, nt, shm, stream, w, p, upw); break;
+        case 1: mmv_nc<TX, 1>(nc, grid, nt, wpb, stream, w, p, upw); break;
+        case 2: mmv_nc<TX, 2>(nc, grid, nt, wpb, stream, w, p, upw); break;
+        case 4: mmv_nc<TX, 4>(nc, grid, nt, wpb, stream, w, p, upw); break;
+        default: mmv_nc<TX, 8>(nc, grid, nt, wpb, stream, w, p, upw); break;
     }
 }
 
@@ -410,7 +494,8 @@ int group_for(int C) {
 template <typename TX, int C, int NC>
 void set_attr() {
     if constexpr (NC <= max_group<TX, C>()) {
-        (void) hipFuncSetAttribute((const void *) k_w64_mmv<TX, C, NC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(16));
+        (void) hipFuncSetAttribute((const void *) k_w64_mmv<TX, C, NC, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(16));
+        (void) hipFuncSetAttribute((const void *) k_w64_mmv<TX, C, NC, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(32));
     }
 }
 template <typename TX, int C>
@@ -453,9 +538,9 @@ void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf
         w64_dims(units, ny, cus, wpb, blocks, upw);
         const dim3 grid(blocks, ny);
         if (x_bf16) {
-            mmv_c<bf16_t>(C, nc, grid, wpb * 64, w64_shm(wpb), stream, w, q, upw);
+            mmv_c<bf16_t>(C, nc, grid, wpb * 64, wpb, stream, w, q, upw);
         } else {
-            mmv_c<float>(C, nc, grid, wpb * 64, w64_shm(wpb), stream, w, q, upw);
+            mmv_c<float>(C, nc, grid, wpb * 64, wpb, stream, w, q, upw);
         }
     }
 }

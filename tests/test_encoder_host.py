@@ -76,7 +76,7 @@ def test_wave64_layout_keeps_plane_and_code(oracle):
     assert np.array_equal(lut[rev], lut_ref)  # same table, index bits reversed
     assert h["off_c"] == h["off_d"] and h["off_d"] % 16 == 0
     ub = a[h["off_b"]: h["off_b"] + 4 * (h["n_a"] + 1)].view(np.uint32)
-    assert ub[0] == 0 and ub[-1] == h["n_b"] and np.all(np.diff(ub.astype(np.int64)) >= 128)
+    assert ub[0] == 0 and ub[-1] == h["n_b"] and np.all(np.diff(ub.astype(np.int64)) >= 192)
     assert a.size == h["off_d"] + 4 * (h["n_b"] + 1024)
 
 
