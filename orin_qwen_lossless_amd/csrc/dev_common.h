@@ -82,6 +82,29 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Cross-lane sums on the VALU only (DPP operand swizzles, no LDS traffic).  After the four in-row steps every lane
+// holds the sum of its row of 16; row_bcast:15 then leaves the sum of lanes 0..31 in lanes 16..31 and of lanes 32..63
+// in lanes 48..63, row_bcast:31 the sum of all 64 in lanes 48..63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float row_sum_dpp(float v) {
+    v = dpp_add<0xB1, 0xf>(v);  // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xf>(v);  // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xf>(v); // row_half_mirror
+    v = dpp_add<0x140, 0xf>(v); // row_mirror
+    return v;
+}
+// valid in lanes 31 and 63: the sums of lanes 0..31 and 32..63
+__device__ __forceinline__ float half_wave_sum_dpp(float v) {
+    return dpp_add<0x142, 0xa>(row_sum_dpp(v)); // row_bcast:15 into rows 1 and 3
+}
+// valid in lane 63: the sum of all 64 lanes
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    return dpp_add<0x143, 0xc>(half_wave_sum_dpp(v)); // row_bcast:31 into rows 2 and 3
+}
+
 // ---------------------------------------------------------------- weight assembly
 // Plane word = 4 sign|mantissa bytes of 4 adjacent columns.  spread_lo/hi put bytes (0,1) / (2,3) into 16-bit halves
 // with the sign in bit 15 and the mantissa in bits 0..6 (other bits hold copies that merge() masks away); merge takes

@@ -37,26 +37,41 @@ __device__ __forceinline__ uint32_t lds_entry(const uint32_t * lut, uint32_t byt
     return *(const uint32_t *) ((const char *) lut + byte_off);
 }
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t) __builtin_amdgcn_readfirstlane((int) v); }
+// lane mask of (a < b), unsigned: one v_cmp into a scalar register pair, used both as the vote and as the select mask
+// (written out because the compiler otherwise materialises the same comparison twice, once per use)
+__device__ __forceinline__ uint64_t lanes_lt(uint32_t a, uint32_t b) {
+    uint64_t m;
+    asm("v_cmp_lt_u32_e64 %0, %1, %2" : "=s"(m) : "v"(a), "v"(b));
+    return m;
+}
+// lane-wise m ? b : a
+__device__ __forceinline__ uint32_t pick(uint32_t a, uint32_t b, uint64_t m) {
+    uint32_t d;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "s"(m));
+    return d;
+}
+__device__ __forceinline__ int64_t uniform64(int64_t v) { // an offset the compiler may keep in scalar registers
+    return (int64_t) (((uint64_t) uniform((uint32_t) ((uint64_t) v >> 32)) << 32) | uniform((uint32_t) v));
+}
 
 // Decoder state of one wave.  cons / filled / limit are the same in every lane (scalar registers).
 struct w64_dec {
     uint32_t w0, w1, w2, P; // per lane: three stream words and the bit position in w0 (< 32)
     uint32_t nw;            // the word requested at the last check (becomes w2 where took is set)
-    bool took;              // this lane requested a word at the last check
+    uint64_t took;          // lanes that requested a word at the last check
     uint32_t cons;          // words consumed, relative to src
     uint32_t filled;        // words copied into the ring, relative to src (multiple of BLK)
-    uint32_t limit;         // end of this wave's streams, relative to src
+    uint32_t last_block;    // first word of the last block that holds words of this wave, relative to src
     uint32_t * ring;
     const uint32_t * src;   // 16-byte aligned
     uint4 pend;             // the block that starts at `filled`, in flight
     int lane;
 
+    // Every load is unconditional (a block or step past the end re-reads the last one) so that the number of loads in
+    // flight at any point of the loop is fixed and the waits for prefetched data never drain newer loads.
     __device__ __forceinline__ uint4 load_block(uint32_t first_word) const {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (first_word < limit) { // a block that starts inside the range may run past it: the stream is padded
-            v = *((const uint4 *) (src + first_word) + lane);
-        }
-        return v;
+        const uint32_t w = first_word < last_block ? first_word : last_block;
+        return *((const uint4 *) (src + w) + lane);
     }
     __device__ __forceinline__ void store_block(uint32_t first_word, const uint4 v) {
         const uint32_t off = first_word & (RING - 1);
@@ -70,20 +85,26 @@ struct w64_dec {
         ring = ring_;
         lane = lane_;
         const uint32_t a = first & ~3u;
-        src = stream + a;
+        src = stream + uniform(a); // kernel-argument pointer + scalar offset: stays a global, scalar address
         cons = first - a;
-        limit = end - a;
+        last_block = (end - a - 1) / BLK * BLK; // the stream is padded: a block may run past `end`
         const uint4 b0 = load_block(0);
         pend = load_block(BLK);
         store_block(0, b0);
         filled = BLK;
     }
+    // at least AHEAD words in the ring beyond the consumer; the block after them in flight.  One block per call is the
+    // steady state (a step consumes 85 words on average, 256 at most); the loop only runs when a wave starts.
     __device__ __forceinline__ void keep_ahead() {
-        while (filled - cons < AHEAD) {
+        if (filled - cons < AHEAD) {
             store_block(filled, pend);
             filled += BLK;
-            pend = load_block(filled);
+            while (filled - cons < AHEAD) {
+                store_block(filled, load_block(filled));
+                filled += BLK;
+            }
         }
+        pend = load_block(filled);
     }
     __device__ __forceinline__ void begin_unit() {
         const uint32_t * p = ring + (cons & (RING - 1)) + 3 * lane;
@@ -91,7 +112,7 @@ struct w64_dec {
         w1 = p[1];
         w2 = p[2];
         P = 0;
-        took = false;
+        took = 0;
         nw = 0;
         cons = uniform(cons + 192);
     }
@@ -101,18 +122,18 @@ struct w64_dec {
         e0 = lds_entry(lut, W & 0x3FFCu);
         const uint32_t W2 = W >> (e0 & 31u);
         e1 = lds_entry(lut, W2 & 0x3FFCu);
-        P += (e0 + e1) & 63u;
-        const bool need = P >= 32u;
-        const uint64_t m = __ballot(need);
+        // entry bits 5 and 6 are zero and P < 32: bits 0..5 of the sum are exact (the exponent fields only add above)
+        const uint32_t t = (P + e0 + e1) & 63u;
+        const uint64_t m = lanes_lt(31u, t);
         const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
         const uint32_t req = ring[(cons & (RING - 1)) + rank];
         // the word requested one check ago has arrived by now: it is this lane's w2
-        w2 = took ? nw : w2;
-        w0 = need ? w1 : w0;
-        w1 = need ? w2 : w1;
+        w2 = pick(w2, nw, took);
+        w0 = pick(w0, w1, m);
+        w1 = pick(w1, w2, m);
         nw = req;
-        took = need;
-        P &= 31u;
+        took = m;
+        P = t & 31u;
         cons = uniform(cons + (uint32_t) __builtin_popcountll(m));
     }
     // the 16 weights of this lane in one step as 8 BF16 pairs: wp[2j], wp[2j+1] = columns 128j + 4(lane%32) + {0,1}, {2,3}
@@ -190,30 +211,32 @@ template <int C> struct geom {
 template <int NB>
 struct chain {
     w64_dec dec;
-    const uint4 * pp;      // next plane step to load, + 64 per step
+    const uint8_t * plane; // first plane byte of the chain's units (uniform)
+    uint32_t off;          // byte offset of the next step to load
+    uint32_t last;         // byte offset of the chain's last step
     uint4 sm[NB];          // plane bytes of the body's steps
-    int64_t steps_left;    // steps not yet loaded
     int64_t row;           // output row of the next body, relative to the product
+    __device__ __forceinline__ uint4 load_step(int lane) const {
+        const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
+        return *((const uint4 *) (plane + o) + lane);
+    }
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t gu0, int64_t n_units, int64_t row0, int R, int K,
                                           int lane) {
-        dec.start(ring, q.stream, q.ubase[gu0], q.ubase[gu0 + n_units], lane);
-        pp = (const uint4 *) (q.plane + gu0 * R * K) + lane;
-        steps_left = n_units * R * (K / CHUNK) / 2;
+        dec.start(ring, q.stream, uniform(q.ubase[gu0]), uniform(q.ubase[gu0 + n_units]), lane);
+        plane = q.plane + uniform64(gu0 * R * K);
+        off = 0;
+        last = (uint32_t) (n_units * R * K - 1024);
         row = row0;
 #pragma unroll
         for (int s = 0; s < NB; s++) {
-            sm[s] = pp[64 * s]; // a unit holds whole bodies, so the first NB steps exist
+            sm[s] = load_step(lane);
+            off += 1024;
         }
-        pp += 64 * NB;
-        steps_left -= NB;
     }
     // plane bytes of step s of the next body, once step s of this body is consumed
-    __device__ __forceinline__ void reload(int s) {
-        if (steps_left > 0) {
-            sm[s] = pp[0];
-        }
-        pp += 64;
-        steps_left--;
+    __device__ __forceinline__ void reload(int s, int lane) {
+        sm[s] = load_step(lane);
+        off += 1024;
     }
 };
 
@@ -226,8 +249,9 @@ __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uin
     const int l32 = lane & 31, half = lane >> 5;
 #pragma unroll
     for (int k = 0; k < N; k++) {
-        ch[k].dec.keep_ahead();
+        ch[k].dec.keep_ahead(); // 256 words ahead cover the 192 of a unit start ...
         ch[k].dec.begin_unit();
+        ch[k].dec.keep_ahead(); // ... and then the first step again
     }
     const int bodies = R * C / 2 / G::NB;
     for (int b = 0; b < bodies; b++) {
@@ -238,7 +262,6 @@ __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uin
             uint32_t smw[N][4];
 #pragma unroll
             for (int k = 0; k < N; k++) {
-                ch[k].dec.keep_ahead();
                 smw[k][0] = ch[k].sm[s].x; smw[k][1] = ch[k].sm[s].y; smw[k][2] = ch[k].sm[s].z; smw[k][3] = ch[k].sm[s].w;
             }
 #pragma unroll
@@ -251,9 +274,15 @@ __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uin
                     wp[k][2 * j + 1] = merge(spread_hi(smw[k][j]), e1);
                 }
             }
+            // all memory traffic of the step in one place, after the decode: the loads waited for here (a stream block
+            // about to enter the ring) were issued a whole step ago, and the new ones have a whole step to arrive
 #pragma unroll
             for (int k = 0; k < N; k++) {
-                ch[k].reload(s);
+                ch[k].dec.keep_ahead();
+            }
+#pragma unroll
+            for (int k = 0; k < N; k++) {
+                ch[k].reload(s, lane);
 #pragma unroll
                 for (int n = 0; n < NC; n++) {
                     if (C >= 4) {
@@ -271,23 +300,23 @@ __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uin
             for (int n = 0; n < NC; n++) {
                 char * y = cv.y + n * p.y_tok;
                 if (C >= 4) { // a body is one row
-                    const float v = wave_sum(acc[k][n][0]);
-                    if (lane == 0) {
+                    const float v = wave_sum_dpp(acc[k][n][0]);
+                    if (lane == 63) {
                         store_y(y, p.y_bf16, row, v);
                     }
                 } else if (C == 2) { // a step is one row
 #pragma unroll
                     for (int s = 0; s < 2; s++) {
-                        const float v = wave_sum(acc[k][n][s]);
-                        if (lane == 0) {
+                        const float v = wave_sum_dpp(acc[k][n][s]);
+                        if (lane == 63) {
                             store_y(y, p.y_bf16, row + s, v);
                         }
                     }
                 } else { // a step is rows 2s (lanes 0..31) and 2s + 1 (lanes 32..63)
 #pragma unroll
                     for (int s = 0; s < 2; s++) {
-                        const float v = half_wave_sum(acc[k][n][s]);
-                        if (l32 == 0) {
+                        const float v = half_wave_sum_dpp(acc[k][n][s]);
+                        if (l32 == 31) {
                             store_y(y, p.y_bf16, row + 2 * s + half, v);
                         }
                     }
