@@ -21,6 +21,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per GEMV launch from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, each factor calibrated
+# on a copy of known size in the same profiler run), for the workloads that were profiled; not measurable in-process.
+MEASURED_TRAFFIC = {(248320, 2048): 709_600_000}
 
 
 def gen_weights(rows: int, K: int, seed: int):
@@ -37,20 +40,25 @@ def gen_weights(rows: int, K: int, seed: int):
 
 
 def time_kernel(fn, steps: int, warmup: int):
-    """Per-launch durations (ms) from HIP events recorded on the launch stream, and the wall time of the timed region."""
+    """Wall time of `steps` back-to-back launches (synchronised on both sides), then per-launch durations (ms) of a
+    second pass from HIP events recorded around every launch on the launch stream (torch's current stream, which is the
+    one the library launches on)."""
     import torch
 
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for i in range(steps):
         ev[i][0].record()
         fn(i)
         ev[i][1].record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     return [a.elapsed_time(b) for a, b in ev], wall
 
 
@@ -68,7 +76,7 @@ def cpu_baseline(wbits, K: int, xf, sample_rows: int):
     nbytes = plane.size + aux.size
     O.decode_gemv(plane, aux, xf, 0, sample_rows, threads)  # warm-up
     reps, t_total, best = 0, 0.0, None
-    while t_total < 12.0 and reps < 200:
+    while t_total < 12.0 and reps < 5000:
         t0 = time.perf_counter()
         O.decode_gemv(plane, aux, xf, 0, sample_rows, threads)
         dt = time.perf_counter() - t0
@@ -144,8 +152,9 @@ def main() -> None:
                    "rows": rows, "K": K, "batch": 1, "compressed_bytes": comp_bytes, "bits_per_weight": round(8 * comp_bytes / (rows * K), 4),
                    "ratio_of_bf16": round(comp_bytes / (2 * rows * K), 4)},
         "roofline": {"bound": "hbm", "achieved": round(algo_bytes / (kern_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_w64_mmv<bf16,4,1>", "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 2),
+                     "unit": "GB/s", "frac": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((rows, K)),
+                     "kernel": "k_w64_mmv<bf16_t, 4, 1, 2>", "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 2),
                      "median_launch_us": round(float(np.median(durs)) * 1e3, 2)},
         "extra": {"pct_of_hbm_peak_compressed": round(100 * comp_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
                   "us_per_matrix": round(ms * 1e3, 2), "blas_bf16_gemv_us": round(blas_us, 2),

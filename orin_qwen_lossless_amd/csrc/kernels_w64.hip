@@ -93,8 +93,9 @@ struct w64_dec {
         store_block(0, b0);
         filled = BLK;
     }
-    // at least AHEAD words in the ring beyond the consumer; the block after them in flight.  One block per call is the
-    // steady state (a step consumes 85 words on average, 256 at most); the loop only runs when a wave starts.
+    // at least AHEAD words in the ring beyond the consumer; the block after them in flight.  At most one block per
+    // call is the steady state (a step consumes 85 words on average, 256 at most); the loop only runs when a wave
+    // starts.  The next block is requested only when the one in flight has been stored: one load per ring slot.
     __device__ __forceinline__ void keep_ahead() {
         if (filled - cons < AHEAD) {
             store_block(filled, pend);
@@ -103,8 +104,8 @@ struct w64_dec {
                 store_block(filled, load_block(filled));
                 filled += BLK;
             }
+            pend = load_block(filled);
         }
-        pend = load_block(filled);
     }
     __device__ __forceinline__ void begin_unit() {
         const uint32_t * p = ring + (cons & (RING - 1)) + 3 * lane;
