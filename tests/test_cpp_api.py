@@ -1,0 +1,32 @@
+"""The C++ API headers (include/bf16n/*.h, the reference's core/include/bf16n/{encode,policy,launch}.h restated over
+the C ABI) compile against the library and translate status codes into the reference's exception types."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIBDIR = os.path.join(ROOT, "orin_qwen_lossless_amd")
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="no hipcc")
+def test_cpp_headers_compile_and_run(tmp_path):
+    from orin_qwen_lossless_amd import _lib
+
+    _lib.lib()  # the library must be built
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    exe = str(tmp_path / "api_smoke")
+    subprocess.run([hipcc, "-std=c++17", "-I" + os.path.join(ROOT, "include"), os.path.join(ROOT, "tests", "cpp", "api_smoke.cpp"),
+                    "-o", exe, "-L" + LIBDIR, "-lbf16n_hip", "-Wl,-rpath," + LIBDIR], check=True, capture_output=True, timeout=300)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=60).stdout.splitlines()
+    got = {ln.split()[0]: ln.split(None, 1)[1] if " " in ln else "" for ln in out}
+    assert got["choose_bad_k"] == "0"
+    assert got["choose_llama"] == "3 16 0 0"      # reference: dense HUFPAIR, largest R leaving >= 512 units
+    assert got["choose_mi355x"] == "3 16 0 1"
+    assert got["encode"] == "16384 3 4 1 1024 0"
+    assert got["encode_wave64"] == "4"
+    assert got["invalid_argument"].startswith("bf16n encode:")
+    assert "no_throw" not in got
+    assert any("fragment" in ln for ln in out if ln.startswith("invalid_argument"))
+    assert got["views"] == "8 1"
