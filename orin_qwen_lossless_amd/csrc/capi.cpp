@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include <climits>
+#include <cstdint>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -46,6 +47,7 @@ void ensure_init() {
         hip_check(hipDeviceGetAttribute(&g_cus, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute");
         hip_check(hipDeviceGetAttribute(&g_lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev), "hipDeviceGetAttribute");
         dev::w64_init();
+        dev::mm_ids_init();
     });
 }
 
@@ -290,6 +292,12 @@ int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x
         check_weight(*w);
         require(dev::mm_ids_shape_ok(*w, up), "no batched kernel for this matrix");
         require(n_experts > 0 && w->rows % n_experts == 0, "rows must split evenly into experts");
+        if (up) {
+            check_weight(*up);
+        }
+        require(x_bf16 && dst && ids_src1 && ids_dst && bounds, "null pointer");
+        require(((uintptr_t) x_bf16 & 15) == 0 && x_row % 8 == 0, "activations must be 16-byte aligned with 16-byte row strides");
+        require(((uintptr_t) dst & 15) == 0 && dst_col % 4 == 0, "dst must be 16-byte aligned with a column stride that is a multiple of 4");
         dev::launch_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, n_tok, n_used,
                            g_cus, (hipStream_t) stream);
         launch_check("mm_ids");

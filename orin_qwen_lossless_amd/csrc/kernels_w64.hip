@@ -14,147 +14,13 @@
 // Activations stay in registers for the whole kernel (a lane always meets the same columns), products are accumulated in
 // FP32 (v_dot2_f32_bf16 for BF16 activations, v_fma_f32 for FP32 ones) and reduced across the wave once per row.
 #include "dev_common.h"
+#include "dev_w64.h"
 #include "launchers.h"
 
 namespace bf16n {
 namespace dev {
 
 namespace {
-
-constexpr int RING = 512;     // ring words per wave (2 KiB)
-constexpr int RING_PAD = 256; // copy of the first ring words behind the end: reads never wrap
-constexpr int BLK = 256;      // words per refill block: one uint4 per lane
-constexpr int AHEAD = 256;    // words kept ahead of the consumer: a unit start (192) or a step (4 x 64)
-constexpr int LUT_WORDS = 1 << HP_LP;
-constexpr int WAVE_LDS_WORDS = RING + RING_PAD;
-
-struct w64_ptrs { const uint8_t * plane; const uint32_t * lut; const uint32_t * ubase; const uint32_t * stream; };
-__device__ __forceinline__ w64_ptrs w64p(const bf16n_weight & w) {
-    return {w.plane, (const uint32_t *) (w.aux + w.off_a), (const uint32_t *) (w.aux + w.off_b), (const uint32_t *) (w.aux + w.off_d)};
-}
-
-__device__ __forceinline__ uint32_t lds_entry(const uint32_t * lut, uint32_t byte_off) {
-    return *(const uint32_t *) ((const char *) lut + byte_off);
-}
-__device__ __forceinline__ uint32_t uniform(uint32_t v) { return (uint32_t) __builtin_amdgcn_readfirstlane((int) v); }
-// lane mask of (a < b), unsigned: one v_cmp into a scalar register pair, used both as the vote and as the select mask
-// (written out because the compiler otherwise materialises the same comparison twice, once per use)
-__device__ __forceinline__ uint64_t lanes_lt(uint32_t a, uint32_t b) {
-    uint64_t m;
-    asm("v_cmp_lt_u32_e64 %0, %1, %2" : "=s"(m) : "v"(a), "v"(b));
-    return m;
-}
-// lane-wise m ? b : a
-__device__ __forceinline__ uint32_t pick(uint32_t a, uint32_t b, uint64_t m) {
-    uint32_t d;
-    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "s"(m));
-    return d;
-}
-__device__ __forceinline__ int64_t uniform64(int64_t v) { // an offset the compiler may keep in scalar registers
-    return (int64_t) (((uint64_t) uniform((uint32_t) ((uint64_t) v >> 32)) << 32) | uniform((uint32_t) v));
-}
-
-// Decoder state of one wave.  cons / filled / limit are the same in every lane (scalar registers).
-struct w64_dec {
-    uint32_t w0, w1, w2, P; // per lane: three stream words and the bit position in w0 (< 32)
-    uint32_t nw;            // the word requested at the last check (becomes w2 where took is set)
-    uint64_t took;          // lanes that requested a word at the last check
-    uint32_t cons;          // words consumed, relative to src
-    uint32_t filled;        // words copied into the ring, relative to src (multiple of BLK)
-    uint32_t last_block;    // first word of the last block that holds words of this wave, relative to src
-    uint32_t * ring;
-    const uint32_t * src;   // 16-byte aligned
-    uint4 pend;             // the block that starts at `filled`, in flight
-    int lane;
-
-    // Every load is unconditional (a block or step past the end re-reads the last one) so that the number of loads in
-    // flight at any point of the loop is fixed and the waits for prefetched data never drain newer loads.
-    __device__ __forceinline__ uint4 load_block(uint32_t first_word) const {
-        const uint32_t w = first_word < last_block ? first_word : last_block;
-        return *((const uint4 *) (src + w) + lane);
-    }
-    __device__ __forceinline__ void store_block(uint32_t first_word, const uint4 v) {
-        const uint32_t off = first_word & (RING - 1);
-        *((uint4 *) (ring + off) + lane) = v;
-        if (off == 0) {
-            *((uint4 *) (ring + RING) + lane) = v;
-        }
-    }
-    // stream words [first, end) of the aux stream belong to this wave
-    __device__ __forceinline__ void start(uint32_t * ring_, const uint32_t * stream, uint32_t first, uint32_t end, int lane_) {
-        ring = ring_;
-        lane = lane_;
-        const uint32_t a = first & ~3u;
-        src = stream + uniform(a); // kernel-argument pointer + scalar offset: stays a global, scalar address
-        cons = first - a;
-        last_block = (end - a - 1) / BLK * BLK; // the stream is padded: a block may run past `end`
-        const uint4 b0 = load_block(0);
-        pend = load_block(BLK);
-        store_block(0, b0);
-        filled = BLK;
-    }
-    // at least AHEAD words in the ring beyond the consumer; the block after them in flight.  At most one block per
-    // call is the steady state (a step consumes 85 words on average, 256 at most); the loop only runs when a wave
-    // starts.  The next block is requested only when the one in flight has been stored: one load per ring slot.
-    __device__ __forceinline__ void keep_ahead() {
-        if (filled - cons < AHEAD) {
-            store_block(filled, pend);
-            filled += BLK;
-            while (filled - cons < AHEAD) {
-                store_block(filled, load_block(filled));
-                filled += BLK;
-            }
-            pend = load_block(filled);
-        }
-    }
-    __device__ __forceinline__ void begin_unit() {
-        const uint32_t * p = ring + (cons & (RING - 1)) + 3 * lane;
-        w0 = p[0];
-        w1 = p[1];
-        w2 = p[2];
-        P = 0;
-        took = 0;
-        nw = 0;
-        cons = uniform(cons + 192);
-    }
-    // two pair codes; afterwards lanes whose position passed a word boundary request the next stream words in lane order
-    __device__ __forceinline__ void two(const uint32_t * lut, uint32_t & e0, uint32_t & e1) {
-        const uint32_t W = __builtin_amdgcn_alignbit(w1, w0, P);
-        e0 = lds_entry(lut, W & 0x3FFCu);
-        const uint32_t W2 = W >> (e0 & 31u);
-        e1 = lds_entry(lut, W2 & 0x3FFCu);
-        // entry bits 5 and 6 are zero and P < 32: bits 0..5 of the sum are exact (the exponent fields only add above)
-        const uint32_t t = (P + e0 + e1) & 63u;
-        const uint64_t m = lanes_lt(31u, t);
-        const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
-        const uint32_t req = ring[(cons & (RING - 1)) + rank];
-        // the word requested one check ago has arrived by now: it is this lane's w2
-        w2 = pick(w2, nw, took);
-        w0 = pick(w0, w1, m);
-        w1 = pick(w1, w2, m);
-        nw = req;
-        took = m;
-        P = t & 31u;
-        cons = uniform(cons + (uint32_t) __builtin_popcountll(m));
-    }
-    // the 16 weights of this lane in one step as 8 BF16 pairs: wp[2j], wp[2j+1] = columns 128j + 4(lane%32) + {0,1}, {2,3}
-    __device__ __forceinline__ void step(const uint32_t * lut, const uint4 sm, uint32_t (&wp)[8]) {
-        const uint32_t smw[4] = {sm.x, sm.y, sm.z, sm.w};
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            uint32_t e0, e1;
-            two(lut, e0, e1);
-            wp[2 * j] = merge(spread_lo(smw[j]), e0);
-            wp[2 * j + 1] = merge(spread_hi(smw[j]), e1);
-        }
-    }
-};
-
-__device__ __forceinline__ void stage_lut(uint32_t * lut, const uint32_t * lut_g) {
-    for (int i = threadIdx.x; i < LUT_WORDS / 4; i += blockDim.x) {
-        ((uint4 *) lut)[i] = ((const uint4 *) lut_g)[i];
-    }
-}
 
 // ---------------------------------------------------------------- activations in registers
 

@@ -36,6 +36,7 @@ void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_e
                         float * weights, hipStream_t stream);
 
 // batched MoE prefill (kernels_mm_ids.hip)
+void mm_ids_init();
 bool mm_ids_shape_ok(const bf16n_weight & w, const bf16n_weight * up);
 void launch_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
                    const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
