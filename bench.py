@@ -89,6 +89,130 @@ def cpu_baseline(wbits, K: int, xf, sample_rows: int):
                       f"{nbytes} compressed bytes), mean of {reps} runs ({med * 1e3:.1f} ms each, best {best * 1e3:.1f} ms)"}
 
 
+def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: str = "mi355x"):
+    """Encode a [rows, K] BF16 device tensor under the mi355x policy (n_matrices stacked experts) and upload `copies`
+    copies; returns (list of weights, compressed bytes, description)."""
+    import numpy as np
+    import torch
+
+    rows, K = w_dev.shape
+    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, K, n_matrices, engine=engine, expert=n_matrices > 1)
+    wbits = w_dev.cpu().view(torch.int16).numpy().view(np.uint16)
+    plane, aux, fmt_out, _ = ops.encode_bits(wbits, fmt, R, cm, wave64=w64)
+    ta = torch.from_numpy(aux)
+    meta = ops.parse_header(ta)
+    ws = [ops.upload(torch.from_numpy(plane), ta, meta, "cuda") for _ in range(copies)]
+    desc = f"{ops.FORMAT_NAMES[fmt_out]} R={R}{' chunk-major' if cm else ''}{' wave64' if w64 else ''}"
+    return ws, plane.size + aux.size, desc
+
+
+def med_us(fn, steps: int = 50, warmup: int = 5) -> float:
+    import numpy as np
+
+    d, _ = time_kernel(fn, steps, warmup)
+    return float(np.median(d)) * 1e3
+
+
+def graph_us(fn, n: int = 16, reps: int = 30) -> float:
+    """Per-call time of a short operation: n calls captured into one HIP graph (alternating weight copies through the
+    call index), the graph replayed `reps` times between HIP events; host launch overhead stays out of the figure."""
+    import numpy as np
+    import torch
+
+    fn(0)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(n):
+            fn(i)
+    d, _ = time_kernel(lambda i: graph.replay(), reps, 3)
+    return float(np.median(d)) * 1e3 / n
+
+
+def suite(ops, w_head, head_copies, x1, K: int) -> dict:
+    """The other configurations of the path, each timed with HIP events (median of 50 launches): batch 4 on the output
+    projection, the small NIBBLE matrices, one MoE layer at batch 1 as a captured HIP graph, and the batched prefill."""
+    import numpy as np
+    import torch
+
+    out = {}
+    g = torch.Generator(device="cuda").manual_seed(3)
+
+    def randw(rows, k):
+        return (torch.randn((rows, k), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+
+    def randx(*shape):
+        return torch.randn(shape, generator=g, device="cuda").to(torch.bfloat16)
+
+    # batch 4 on the output projection (one decode shared by the four columns)
+    x4 = randx(4, K)
+    t4 = med_us(lambda i: ops.mmv(x4, head_copies[i & 1]))
+    out["lm_head_batch4_us"] = round(t4, 2)
+    # small NIBBLE matrices
+    for rows, k in ((512, 2048), (2048, 512)):
+        ws, nbytes, desc = encode_to_device(ops, randw(rows, k), copies=2)
+        xx = randx(1, k)
+        t = graph_us(lambda i: ops.mmv(xx, ws[i & 1]))
+        out[f"gemv_{rows}x{k}"] = {"layout": desc, "us": round(t, 2), "GBps": round(nbytes / t / 1e3, 1),
+                                   "timing": "16 launches per HIP graph replay"}
+    # one MoE layer of the 35B-A3B shape: router 256x2048, 256 experts x (gate 512x2048, up 512x2048, down 2048x512),
+    # top-8 of 256 computed on the device (softmax, renormalised top-k weights)
+    E, topk, N = 256, 8, 512
+    router, rb, rdesc = encode_to_device(ops, randw(E, K))
+    wg, wu = randw(E * N, K), randw(E * N, K)
+    down, db, ddesc = encode_to_device(ops, randw(E * K, N), n_matrices=E)
+    router, down = router[0], down[0]
+    xs = [randx(1, K) for _ in range(8)]
+    xbuf = xs[0].clone()
+    cm_pair = None
+    for engine in ("mi355x", "llama"):  # gate / up: this build's wave64 units, and the reference's chunk-major units
+        gate, gb, gdesc = encode_to_device(ops, wg, n_matrices=E, engine=engine)
+        up, ub, _ = encode_to_device(ops, wu, n_matrices=E, engine=engine)
+        gate, up = gate[0], up[0]
+        if engine == "llama":
+            cm_pair = (gate, up)
+
+        def layer():
+            wts, ids = ops.router_topk(ops.mmv(xbuf, router), topk)
+            return ops.moe_experts(xbuf, gate, up, down, wts, ids, E)
+
+        layer()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            layer()
+
+        def replay(i):
+            xbuf.copy_(xs[i & 7])  # other tokens pick other experts: the 8 routed experts are not cache-resident
+            graph.replay()
+
+        t_layer = med_us(replay, 64, 8)
+        touched = rb + (gb + ub + db) * topk // E
+        out[f"moe_layer_batch1_gate_up_{engine}"] = {
+            "layouts": {"router": rdesc, "gate_up": gdesc, "down": ddesc}, "graph_us": round(t_layer, 2),
+            "compressed_bytes_touched": int(touched), "GBps": round(touched / t_layer / 1e3, 1),
+            "routing": "softmax over 256 logits, top-8 (ties: lower index), weights renormalised to sum 1"}
+        del graph
+    # prefill: fused gate/up + SwiGLU (BF16 out), then down, over routing lists computed on the device
+    gate, up = cm_pair
+    for T in (2048, 8192):
+        xp = randx(T, K)
+        lg = torch.randn((T, E), generator=g, device="cuda")
+        wts, ids = ops.router_topk(lg, topk)
+
+        def prefill(i):
+            a = ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16)
+            return ops.moe_mm_ids(a, ids, down, E)
+
+        t = med_us(prefill, 10, 2)
+        t_gu = med_us(lambda i: ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16), 10, 2)
+        flops = 2.0 * T * topk * (2 * N * K + K * N)
+        out[f"moe_prefill_T{T}"] = {"us": round(t, 1), "gate_up_us": round(t_gu, 1), "TFLOPs": round(flops / t / 1e6, 2),
+                                    "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / 2500.0, 4),
+                                    "tokens_per_s": round(T / t * 1e6, 0)}
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,6 +222,7 @@ def main() -> None:
     ap.add_argument("--K", type=int, default=2048)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=16384)
+    ap.add_argument("--suite", action="store_true", help="also time batch 4, the NIBBLE matrices, a MoE layer and the prefill")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path has no collective); run with --gpus 1")
@@ -161,6 +286,8 @@ def main() -> None:
                   "speedup_vs_blas_bf16": round(blas_us / (ms * 1e3), 3), "tokens_per_s_lm_head_only": round(1e3 / ms, 1),
                   "host_encode_s": round(t_enc, 2), "max_err_over_sum_abs": err, "setup_s": round(time.perf_counter() - t0, 1)},
     }
+    if args.suite:
+        out["extra"]["suite"] = suite(ops, w_dev, copies, x, K)
     if not args.no_cpu:
         xf = x[0].float().cpu().numpy()
         out["cpu_baseline"] = cpu_baseline(wbits, K, xf, min(args.cpu_rows, rows // 16 * 16))

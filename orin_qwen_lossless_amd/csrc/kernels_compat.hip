@@ -221,49 +221,101 @@ __device__ __forceinline__ uint32_t esc_bits(uint32_t rec) { // BF16 bits of an 
     return ((smb & 0x80u) << 8) | (ex << 7) | (smb & 0x7Fu);
 }
 
-// dot(row gr, x); escaped weights read as +0 in the dense part and add their exact product afterwards; result in
-// every lane of the half-wave
-__device__ __forceinline__ float nib_row_dot(const nib_ptrs & w, int64_t gr, int C, const float * xs, int l32) {
-    const int64_t K = (int64_t) C * CHUNK;
-    const uint4 T = *(const uint4 *) (w.table + gr * 16);
-    float acc = 0.f;
-    for (int c = 0; c < C; c++) {
-        const uint4 sm = *((const uint4 *) (w.plane + gr * K + c * CHUNK) + l32);
-        const uint2 cd = *((const uint2 *) (w.codes + gr * (K / 2) + c * 256) + l32);
-        uint32_t wp[8];
-        nib_chunk(sm, cd, T, wp);
-        acc += dot_chunk(wp, xs + c * CHUNK, l32);
+// the 16 activations one lane meets in a 512-column chunk (columns 128 j + 4 l + 0..3), as FP32
+template <typename TX>
+__device__ __forceinline__ void x_chunk16(const char * x, int col0, float (&xv)[16]);
+template <> __device__ __forceinline__ void x_chunk16<float>(const char * x, int col0, float (&xv)[16]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float4 t = *(const float4 *) (x + 4 * (col0 + 128 * j));
+        xv[4 * j] = t.x; xv[4 * j + 1] = t.y; xv[4 * j + 2] = t.z; xv[4 * j + 3] = t.w;
     }
-    const uint32_t e0 = w.esc_off[gr], e1 = w.esc_off[gr + 1];
-    for (uint32_t i = e0 + l32; i < e1; i += 32) {
-        const uint32_t rec = w.esc[i];
-        acc = fmaf(bf16_bits_to_f32(esc_bits(rec)), xs[rec & 0xFFFu], acc);
+}
+template <> __device__ __forceinline__ void x_chunk16<bf16_t>(const char * x, int col0, float (&xv)[16]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint2 t = *(const uint2 *) (x + 2 * (col0 + 128 * j));
+        xv[4 * j] = __uint_as_float(t.x << 16); xv[4 * j + 1] = __uint_as_float(t.x & 0xFFFF0000u);
+        xv[4 * j + 2] = __uint_as_float(t.y << 16); xv[4 * j + 3] = __uint_as_float(t.y & 0xFFFF0000u);
     }
-    return half_wave_sum(acc);
 }
 
-// NIBBLE GEMV; GLU 1: rows_per_matrix = [gate (nrows); up (nrows)] of one matrix; GLU 2: separate gate / up matrices
+// partial dot of (row gr, chunk c) with x; escaped weights read as +0 here.  The four per-position sums are combined
+// as in the reference (kernels.cuh:130-187), then over the 32 lanes; result in every lane of the half-wave.
+__device__ __forceinline__ float nib_chunk_dot(const nib_ptrs & w, int64_t gr, int C, int c, const uint4 T, const float (&xv)[16], int l32) {
+    const int64_t K = (int64_t) C * CHUNK;
+    const uint4 sm = *((const uint4 *) (w.plane + gr * K + c * CHUNK) + l32);
+    const uint2 cd = *((const uint2 *) (w.codes + gr * (K / 2) + c * 256) + l32);
+    uint32_t wp[8];
+    nib_chunk(sm, cd, T, wp);
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        a0 = fmaf(bf16_bits_to_f32(wp[2 * j] & 0xFFFFu), xv[4 * j], a0);
+        a1 = fmaf(__uint_as_float(wp[2 * j] & 0xFFFF0000u), xv[4 * j + 1], a1);
+        a2 = fmaf(bf16_bits_to_f32(wp[2 * j + 1] & 0xFFFFu), xv[4 * j + 2], a2);
+        a3 = fmaf(__uint_as_float(wp[2 * j + 1] & 0xFFFF0000u), xv[4 * j + 3], a3);
+    }
+    return half_wave_sum((a0 + a1) + (a2 + a3));
+}
+
+// the exact products of a row's escaped weights, summed over the half-wave
+template <typename TX>
+__device__ __forceinline__ float nib_escapes(const nib_ptrs & w, int64_t gr, const char * x, int l32) {
+    const uint32_t e0 = w.esc_off[gr], e1 = w.esc_off[gr + 1];
+    float acc = 0.f;
+    for (uint32_t i = e0 + l32; i < e1; i += 32) {
+        const uint32_t rec = w.esc[i];
+        acc = fmaf(bf16_bits_to_f32(esc_bits(rec)), x_at<TX>(x, (int) (rec & 0xFFFu)), acc);
+    }
+    return e1 > e0 ? half_wave_sum(acc) : 0.f;
+}
+
+// NIBBLE GEMV; GLU 1: rows_per_matrix = [gate (nrows); up (nrows)] of one matrix; GLU 2: separate gate / up matrices.
+// These matrices are small (a few MB at most), so the launch is laid out for latency: one half-wave per (row, chunk)
+// pair, every load of a pair issued at once, the C chunk sums of a row combined through LDS in chunk order.
 template <typename TX, int GLU>
 __global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p) {
-    extern __shared__ __align__(16) unsigned char shm_raw[];
-    float * xs = (float *) shm_raw;
-    const int K = (int) w.K, C = K / CHUNK;
+    __shared__ float part[2][HALVES];
+    const int K = (int) w.K, C = K / CHUNK; // 1, 2, 4 or 8: HALVES / C rows per block
     const col_view cv = col_setup(p, blockIdx.y);
-    for (int i = threadIdx.x; i < K; i += NT) {
-        xs[i] = x_at<TX>(cv.x, i);
-    }
-    __syncthreads();
     const nib_ptrs g = nibp(w, 0);
     const nib_ptrs u = GLU == 1 ? nibp(w, p.nrows) : nibp(w_up, 0);
     const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
-    for (int64_t r = (int64_t) blockIdx.x * HALVES + half; r < p.nrows; r += (int64_t) gridDim.x * HALVES) {
-        float v = nib_row_dot(g, cv.rbase + r, C, xs, l32);
+    const int64_t items = p.nrows * C;
+    for (int64_t base = (int64_t) blockIdx.x * HALVES; base < items; base += (int64_t) gridDim.x * HALVES) {
+        const int64_t q = base + half;
+        const bool live = q < items;
+        const int64_t r = live ? q / C : 0;
+        const int c = live ? (int) (q % C) : 0;
+        const int64_t gr = cv.rbase + r;
+        float xv[16];
+        x_chunk16<TX>(cv.x, c * CHUNK + 4 * l32, xv);
+        float v = nib_chunk_dot(g, gr, C, c, *(const uint4 *) (g.table + gr * 16), xv, l32);
+        float vu = 0.f;
         if (GLU) {
-            v = nib_row_dot(u, cv.rbase + r, C, xs, l32) * silu(v);
+            vu = nib_chunk_dot(u, gr, C, c, *(const uint4 *) (u.table + gr * 16), xv, l32);
+        }
+        if (c == 0) {
+            v += nib_escapes<TX>(g, gr, cv.x, l32);
+            if (GLU) {
+                vu += nib_escapes<TX>(u, gr, cv.x, l32);
+            }
         }
         if (l32 == 0) {
-            store_y(cv.y, p.y_bf16, r, v);
+            part[0][half] = v;
+            part[1][half] = vu;
         }
+        __syncthreads();
+        if (live && c == 0 && l32 == 0) {
+            float s = part[0][half], su = part[1][half];
+            for (int i = 1; i < C; i++) {
+                s += part[0][half + i];
+                su += part[1][half + i];
+            }
+            store_y(cv.y, p.y_bf16, r, GLU ? su * silu(s) : s);
+        }
+        __syncthreads();
     }
 }
 
@@ -323,8 +375,8 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
     const int64_t work = w.format == FMT_NIBBLE ? p.nrows : p.nrows / w.R;
     const dim3 grid(grid_for(work, ncols, cus), ncols);
     if (w.format == FMT_NIBBLE) {
-        const size_t shm = (size_t) w.K * 4;
-#define NIB(TX, G) hipLaunchKernelGGL((k_nib_mmv<TX, G>), grid, dim3(NT), shm, stream, w, wu, p)
+        const dim3 grid(grid_for(p.nrows * (w.K / CHUNK), ncols, cus), ncols);
+#define NIB(TX, G) hipLaunchKernelGGL((k_nib_mmv<TX, G>), grid, dim3(NT), 0, stream, w, wu, p)
         if (x_bf16) { if (glu == 0) NIB(bf16_t, 0); else if (glu == 1) NIB(bf16_t, 1); else NIB(bf16_t, 2); }
         else        { if (glu == 0) NIB(float, 0);  else if (glu == 1) NIB(float, 1);  else NIB(float, 2); }
 #undef NIB

@@ -349,9 +349,14 @@ constexpr int max_group() {
     return 64 / per_col < 1 ? 1 : 64 / per_col > 4 ? 4 : 64 / per_col;
 }
 
+// two decode chains per wave only where the activations leave room for them in 128 registers (the instances with
+// more activation registers would spill; they run one chain per wave)
+template <typename TX, int C, int NC>
+constexpr bool two_chains() { return NC * geom<C>::XS * (sizeof(TX) == 2 ? 8 : 16) <= 16; }
+
 template <typename TX, int C, int NC>
 void mmv_launch(dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
-    if (upw >= 2) {
+    if (upw >= 2 && two_chains<TX, C, NC>()) {
         hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 2>), grid, dim3(nt), w64_shm(2 * wpb), stream, w, p, upw);
     } else {
         hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 1>), grid, dim3(nt), w64_shm(wpb), stream, w, p, upw);
