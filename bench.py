@@ -164,13 +164,12 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
     router, down = router[0], down[0]
     xs = [randx(1, K) for _ in range(8)]
     xbuf = xs[0].clone()
-    cm_pair = None
+    pairs = {}
     for engine in ("mi355x", "llama"):  # gate / up: this build's wave64 units, and the reference's chunk-major units
         gate, gb, gdesc = encode_to_device(ops, wg, n_matrices=E, engine=engine)
         up, ub, _ = encode_to_device(ops, wu, n_matrices=E, engine=engine)
         gate, up = gate[0], up[0]
-        if engine == "llama":
-            cm_pair = (gate, up)
+        pairs[engine] = (gate, up, gdesc)
 
         def layer():
             wts, ids = ops.router_topk(ops.mmv(xbuf, router), topk)
@@ -194,22 +193,22 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
             "routing": "softmax over 256 logits, top-8 (ties: lower index), weights renormalised to sum 1"}
         del graph
     # prefill: fused gate/up + SwiGLU (BF16 out), then down, over routing lists computed on the device
-    gate, up = cm_pair
     for T in (2048, 8192):
         xp = randx(T, K)
         lg = torch.randn((T, E), generator=g, device="cuda")
         wts, ids = ops.router_topk(lg, topk)
+        for engine, (gate, up, gdesc) in pairs.items():
 
-        def prefill(i):
-            a = ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16)
-            return ops.moe_mm_ids(a, ids, down, E)
+            def prefill(i):
+                a = ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16)
+                return ops.moe_mm_ids(a, ids, down, E)
 
-        t = med_us(prefill, 10, 2)
-        t_gu = med_us(lambda i: ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16), 10, 2)
-        flops = 2.0 * T * topk * (2 * N * K + K * N)
-        out[f"moe_prefill_T{T}"] = {"us": round(t, 1), "gate_up_us": round(t_gu, 1), "TFLOPs": round(flops / t / 1e6, 2),
-                                    "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / 2500.0, 4),
-                                    "tokens_per_s": round(T / t * 1e6, 0)}
+            t = med_us(prefill, 10, 2)
+            t_gu = med_us(lambda i: ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16), 10, 2)
+            flops = 2.0 * T * topk * (2 * N * K + K * N)
+            out[f"moe_prefill_T{T}_gate_up_{engine}"] = {
+                "gate_up": gdesc, "us": round(t, 1), "gate_up_us": round(t_gu, 1), "TFLOPs": round(flops / t / 1e6, 2),
+                "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / 2500.0, 4), "tokens_per_s": round(T / t * 1e6, 0)}
     return out
 
 

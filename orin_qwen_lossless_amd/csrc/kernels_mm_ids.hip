@@ -12,7 +12,8 @@
 //   * reference chunk-major HUFPAIR, R = 8, K = 2048 (gate / up; also fused gate + up + SwiGLU): a half-wavefront per
 //     unit, 8 units per slab;
 //   * reference row-major HUFPAIR, R = 16, K = 512 (down): a half-wavefront per unit, 4 units per slab;
-//   * wave64 HUFPAIR, R = 16, K = 512 (down under the mi355x policy): a wavefront per unit, 4 units per slab.
+//   * wave64 HUFPAIR, R = 16, K = 512 (down under the mi355x policy): a wavefront per unit, 4 units per slab;
+//   * wave64 HUFPAIR, R = 8, K = 2048 (gate / up under the mi355x policy): k_mm_ids_w64k below.
 #include "dev_common.h"
 #include "dev_compat.h"
 #include "dev_w64.h"
@@ -34,7 +35,7 @@ constexpr int TILE_ROWS = 32;     // rows decoded per phase: one MFMA block of r
 constexpr int TILE_STRIDE = 520;  // BF16 elements per tile row: 512 + 8 (row stride 1040 bytes spreads rows over banks)
 constexpr int TOK_PASS = 128;     // tokens per pass: 32 per wavefront
 
-enum { L_CM8 = 0, L_RM16 = 1, L_W64 = 2 };
+enum { L_CM8 = 0, L_RM16 = 1, L_W64 = 2, L_W64K = 3 };
 
 struct mm_args {
     const uint16_t * x; int64_t x_row;
@@ -213,6 +214,105 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids(const bf16n_weight w, con
     }
 }
 
+// wave64 row-major units of 8 rows, K = 2048 (gate / up under the mi355x policy).  A row-major unit stream yields whole
+// rows, so the tile holds 32 full rows (4 units, one per wavefront; 128.5 KiB) and a work item is one decode phase and
+// one product phase per matrix; the table in LDS is swapped between gate and up.  One block per CU.
+constexpr int WK_ROWS = 32, WK_K = 2048, WK_STRIDE = WK_K + 8, WK_R = 8;
+
+template <bool GLU>
+__global__ void __launch_bounds__(MM_THREADS) k_mm_ids_w64k(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+    constexpr int NM = GLU ? 2 : 1;
+    extern __shared__ __align__(16) uint32_t shm[];
+    uint32_t * lut = shm;
+    uint16_t * tile = (uint16_t *) (shm + LUT_WORDS);
+    uint32_t * rings = shm + LUT_WORDS + WK_ROWS * WK_STRIDE / 2;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, wave = tid >> 6;
+    const int slabs = (int) (a.rows / WK_ROWS);
+    const int64_t units_per_expert = a.rows / WK_R;
+    int staged = -1; // which matrix's table is in LDS
+    for (int item = blockIdx.x; item < a.n_experts * slabs; item += gridDim.x) {
+        const int e = item / slabs, sl = item % slabs;
+        const int j0 = a.bounds[e], n = a.bounds[e + 1] - j0;
+        for (int tp = 0; tp < n; tp += TOK_PASS) {
+            const int tk = tp + wave * 32 + l32;
+            const bool wave_has = tp + wave * 32 < n, valid = tk < n;
+            const int jj = j0 + (valid ? tk : 0);
+            const uint16_t * xrow = a.x + (int64_t) a.ids_src1[jj] * a.x_row + 8 * (lane >> 5);
+            f32x16_t acc[NM];
+#pragma unroll
+            for (int m = 0; m < NM; m++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    acc[m][i] = 0.f;
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < NM; m++) {
+                const bf16n_weight & wm = m == 0 ? w : w_up;
+                __syncthreads(); // tile and table are free
+                if (staged != m) {
+                    stage_lut(lut, (const uint32_t *) (wm.aux + wm.off_a));
+                    staged = m;
+                    __syncthreads();
+                }
+                {   // this wavefront's unit: 8 rows = 16 steps of (row, chunk pair)
+                    const int64_t gu = e * units_per_expert + (int64_t) sl * (WK_ROWS / WK_R) + wave;
+                    const w64_ptrs q = w64p(wm);
+                    const uint8_t * plane = q.plane + gu * WK_R * (int64_t) WK_K;
+                    w64_dec dec;
+                    dec.start(rings + wave * WAVE_LDS_WORDS, q.stream, uniform(q.ubase[gu]), uniform(q.ubase[gu + 1]), lane);
+                    dec.keep_ahead();
+                    dec.begin_unit();
+#pragma unroll 1
+                    for (int st = 0; st < 2 * WK_R; st++) {
+                        uint32_t wp[8];
+                        dec.keep_ahead();
+                        dec.step(lut, *((const uint4 *) (plane + st * 1024) + lane), wp);
+                        // chunk 2 (st % 2) + lane / 32 of row st / 2
+                        uint16_t * trow = tile + (wave * WK_R + st / 2) * WK_STRIDE + (2 * (st & 1) + (lane >> 5)) * CHUNK;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            *(uint2 *) (trow + 128 * j + 4 * l32) = make_uint2(wp[2 * j], wp[2 * j + 1]);
+                        }
+                    }
+                }
+                __syncthreads();
+                if (wave_has) {
+                    const uint16_t * ap = tile + l32 * WK_STRIDE + 8 * (lane >> 5);
+#pragma unroll 8
+                    for (int ks = 0; ks < WK_K / 16; ks++) {
+                        const bf16x8_t av = *(const bf16x8_t *) (ap + 16 * ks);
+                        const bf16x8_t bv = *(const bf16x8_t *) (xrow + 16 * ks);
+                        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[m], 0, 0, 0);
+                    }
+                }
+            }
+            if (valid) { // accumulator element i: tile row 8 (i / 4) + 4 (lane / 32) + i % 4 = row of the slab
+                const int64_t col = (int64_t) a.ids_dst[jj] * a.dst_col + (int64_t) sl * WK_ROWS;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    float v[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float p = acc[0][4 * g + i];
+                        v[i] = GLU ? acc[NM - 1][4 * g + i] * silu(p) : p;
+                    }
+                    const int row = 8 * g + 4 * (lane >> 5);
+                    if (a.dst_bf16) {
+                        *(uint2 *) ((uint16_t *) a.dst + col + row) =
+                            make_uint2(f32_to_bf16_rne(v[0]) | ((uint32_t) f32_to_bf16_rne(v[1]) << 16),
+                                       f32_to_bf16_rne(v[2]) | ((uint32_t) f32_to_bf16_rne(v[3]) << 16));
+                    } else {
+                        *(float4 *) ((float *) a.dst + col + row) = make_float4(v[0], v[1], v[2], v[3]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+size_t wk_shm() { return (size_t) LUT_WORDS * 4 + (size_t) WK_ROWS * WK_STRIDE * 2 + 4 * WAVE_LDS_WORDS * 4; }
+
 int layout_of(const bf16n_weight & w) {
     if (w.format != FMT_HUFPAIR || (w.flags & FLAG_FRAG_ORDER)) {
         return -1;
@@ -223,6 +323,9 @@ int layout_of(const bf16n_weight & w) {
     }
     if (!cm && w.K == 512 && w.R == 16) {
         return w64 ? L_W64 : L_RM16;
+    }
+    if (!cm && w64 && w.K == WK_K && w.R == WK_R) {
+        return L_W64K;
     }
     return -1;
 }
@@ -245,6 +348,8 @@ void mm_ids_init() {
     (void) hipFuncSetAttribute((const void *) k_mm_ids<L_CM8, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mm_shm<L_CM8, false>());
     (void) hipFuncSetAttribute((const void *) k_mm_ids<L_RM16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mm_shm<L_RM16, false>());
     (void) hipFuncSetAttribute((const void *) k_mm_ids<L_W64, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mm_shm<L_W64, false>());
+    (void) hipFuncSetAttribute((const void *) k_mm_ids_w64k<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) wk_shm());
+    (void) hipFuncSetAttribute((const void *) k_mm_ids_w64k<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) wk_shm());
 }
 
 // the reference's rule (launch.cu:446-456) restated for the layouts this build encodes: gate / up in chunk-major
@@ -257,7 +362,7 @@ bool mm_ids_shape_ok(const bf16n_weight & w, const bf16n_weight * up) {
     if (!up) {
         return true;
     }
-    return l == L_CM8 && layout_of(*up) == L_CM8 && up->rows == w.rows;
+    return (l == L_CM8 || l == L_W64K) && layout_of(*up) == l && up->rows == w.rows;
 }
 
 void launch_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
@@ -269,12 +374,24 @@ void launch_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void *
     a.ids_src1 = ids_src1; a.ids_dst = ids_dst; a.bounds = bounds;
     a.dst = (char *) dst; a.dst_col = dst_col; a.dst_bf16 = dst_bf16;
     a.rows = w.rows / n_experts; a.n_experts = n_experts;
-    if (a.rows % SLAB_ROWS != 0) {
+    const int layout = layout_of(w);
+    if (a.rows % (layout == L_W64K ? WK_ROWS : SLAB_ROWS) != 0) {
         throw std::invalid_argument("bf16n: no batched kernel for this matrix (rows per expert must be a multiple of 64)");
+    }
+    if (layout == L_W64K) {
+        const int64_t items = (int64_t) n_experts * (a.rows / WK_ROWS);
+        const dim3 grid((unsigned) (items < (int64_t) cus ? items : (int64_t) cus));
+        const size_t shm = wk_shm();
+        if (up) {
+            hipLaunchKernelGGL(k_mm_ids_w64k<true>, grid, dim3(MM_THREADS), shm, stream, w, *up, a);
+        } else {
+            hipLaunchKernelGGL(k_mm_ids_w64k<false>, grid, dim3(MM_THREADS), shm, stream, w, w, a);
+        }
+        return;
     }
     const int64_t items = (int64_t) n_experts * (a.rows / SLAB_ROWS);
     const int blocks = (int) (items < 2 * (int64_t) cus ? items : 2 * (int64_t) cus);
-    switch (layout_of(w)) {
+    switch (layout) {
         case L_CM8:
             if (up) {
                 mm_launch<L_CM8, true>(w, up, a, blocks, stream);

@@ -16,9 +16,9 @@ from test_gpu_roundtrip import bits, enc
 pytestmark = pytest.mark.gpu
 HP = 3
 
-# (K, rows per expert, R, chunk_major, wave64): gate / up in reference chunk-major units; down in reference row-major
-# units and in the wave64 layout
-SHAPES = [(2048, 128, 8, True, False), (512, 256, 16, False, False), (512, 256, 16, False, True)]
+# (K, rows per expert, R, chunk_major, wave64): gate / up in reference chunk-major units and in wave64 units; down in
+# reference row-major units and in wave64 units
+SHAPES = [(2048, 128, 8, True, False), (2048, 128, 8, False, True), (512, 256, 16, False, False), (512, 256, 16, False, True)]
 
 
 def routing(T: int, k: int, E: int, counts: dict[int, int], seed: int) -> np.ndarray:
@@ -106,10 +106,11 @@ def test_mm_ids_one_hot_is_exact(ops, K, N, R, cm, w64):
             assert np.array_equal(got[t, i], wf[ids[t, i] * N: (ids[t, i] + 1) * N, c] * np.float32(0.125)), (t, i)
 
 
-def test_mm_ids_fused_gate_up_swiglu(ops):
+@pytest.mark.parametrize("cm,w64", [(True, False), (False, True)])
+def test_mm_ids_fused_gate_up_swiglu(ops, cm, w64):
     K, N, E, k, T = 2048, 128, 5, 3, 150
     gb, ub = synth.weights(E * N, K, 31), synth.weights(E * N, K, 32)
-    g, u = enc(ops, gb, HP, 8, True), enc(ops, ub, HP, 8, True)
+    g, u = enc(ops, gb, HP, 8, cm, w64), enc(ops, ub, HP, 8, cm, w64)
     assert ops.mm_ids_supported(g, u)
     ids = routing(T, k, E, {4: 0}, 6)
     xb = synth.activations(T, K, 8)
@@ -145,12 +146,14 @@ def test_mm_ids_contract(ops):
     assert not ops.mm_ids_supported(nib)
 
 
+@pytest.mark.parametrize("cm,w64", [(True, False), (False, True)])
 @pytest.mark.parametrize("T", [8, 9, 40])
-def test_moe_experts_switches_to_batched_kernels(ops, T):
+def test_moe_experts_switches_to_batched_kernels(ops, T, cm, w64):
     # up to 8 tokens: expert GEMVs; more: fused gate/up + SwiGLU (BF16) then down, both against the exact-weight reference
     E, k, Kd, N = 8, 2, 2048, 512
-    gate = enc(ops, synth.weights(E * N, Kd, 51), HP, 8, True)
-    up = enc(ops, synth.weights(E * N, Kd, 52), HP, 8, True)
+    gate = enc(ops, synth.weights(E * N, Kd, 51), HP, 8, cm, w64)
+    up = enc(ops, synth.weights(E * N, Kd, 52), HP, 8, cm, w64)
+    assert ops.mm_ids_supported(gate, up)
     down = enc(ops, synth.weights(E * Kd, N, 53), HP, 16, False, True)
     ids = torch.from_numpy(routing(T, k, E, {}, T)).cuda()
     wts = torch.softmax(torch.randn((T, k), generator=torch.Generator().manual_seed(T)), dim=-1).cuda()
