@@ -211,15 +211,20 @@ int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf1
                 "mmv_glu: product rows out of range");
         require(!(gate->flags & FLAG_CHUNK_MAJOR) && !(up->flags & FLAG_CHUNK_MAJOR),
                 "mmv_glu: chunk-major weights require separate mmv launches");
-        require(!is_w64(*gate) && !is_w64(*up), "mmv_glu: wave64 weights require separate mmv launches");
+        require(is_w64(*gate) == is_w64(*up), "mmv_glu: gate/up layouts must match");
         require(gate->format == FMT_NIBBLE || gate->R == up->R, "mmv_glu: gate/up R must match");
+        require(!is_w64(*gate) || dev::w64_mmv_supported(*gate, a->x_bf16 != 0), "mmv_glu: no fused kernel for this wave64 shape");
         require(a->ncols > 0 && a->ncols <= 65535, "ncols out of range");
         require(gate->format == FMT_NIBBLE || (a->nrows % gate->R == 0 && a->row0 % gate->R == 0 && a->rows_per_matrix % gate->R == 0),
                 "rows of a product must be whole units");
         if (a->nrows == 0) {
             return;
         }
-        dev::launch_compat_mmv(*gate, up, 2, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
+        if (is_w64(*gate)) {
+            dev::launch_w64_glu(*gate, *up, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
+        } else {
+            dev::launch_compat_mmv(*gate, up, 2, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
+        }
         launch_check("mmv_glu");
     });
 }
@@ -335,7 +340,7 @@ int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, in
     return guarded([&] {
         ensure_init();
         require(n_tok > 0 && n_experts > 0 && k > 0 && k <= n_experts && k <= 64, "router_topk: need 0 < k <= min(n_experts, 64)");
-        require(n_experts <= 8192, "router_topk: too many experts");
+        require(n_experts <= 1024, "router_topk: at most 1024 experts");
         dev::launch_router_topk(logits, logits_stride, n_tok, n_experts, k, renorm != 0, ids, weights, (hipStream_t) stream);
         launch_check("router_topk");
     });

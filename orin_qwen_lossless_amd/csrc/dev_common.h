@@ -105,6 +105,29 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return dpp_add<0x143, 0xc>(half_wave_sum_dpp(v)); // row_bcast:31 into rows 2 and 3
 }
 
+// wave-wide maximum (float) and minimum (uint32) with the same operand swizzles; valid in lane 63.  Lanes a swizzle
+// does not reach keep their own value (the "old" operand), which is neutral for max and min.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_take(uint32_t v) {
+    return (uint32_t) __builtin_amdgcn_update_dpp((int) v, (int) v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+#define BF16N_STEP(C, M) v = fmaxf(v, __uint_as_float(dpp_take<C, M>(__float_as_uint(v))))
+    BF16N_STEP(0xB1, 0xf); BF16N_STEP(0x4E, 0xf); BF16N_STEP(0x141, 0xf); BF16N_STEP(0x140, 0xf);
+    BF16N_STEP(0x142, 0xa); BF16N_STEP(0x143, 0xc);
+#undef BF16N_STEP
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_min_dpp(uint32_t v) {
+#define BF16N_STEP(C, M) { const uint32_t o = dpp_take<C, M>(v); v = o < v ? o : v; }
+    BF16N_STEP(0xB1, 0xf) BF16N_STEP(0x4E, 0xf) BF16N_STEP(0x141, 0xf) BF16N_STEP(0x140, 0xf)
+    BF16N_STEP(0x142, 0xa) BF16N_STEP(0x143, 0xc)
+#undef BF16N_STEP
+    return v;
+}
+__device__ __forceinline__ float lane63(float v) { return __uint_as_float((uint32_t) __builtin_amdgcn_readlane((int) __float_as_uint(v), 63)); }
+__device__ __forceinline__ uint32_t lane63(uint32_t v) { return (uint32_t) __builtin_amdgcn_readlane((int) v, 63); }
+
 // ---------------------------------------------------------------- weight assembly
 // Plane word = 4 sign|mantissa bytes of 4 adjacent columns.  spread_lo/hi put bytes (0,1) / (2,3) into 16-bit halves
 // with the sign in bit 15 and the mantissa in bits 0..6 (other bits hold copies that merge() masks away); merge takes

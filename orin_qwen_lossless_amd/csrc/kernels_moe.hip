@@ -96,54 +96,53 @@ __global__ void __launch_bounds__(256) k_route(const char * __restrict__ ids, in
     }
 }
 
-// softmax over the experts, k largest (ties: lower index), weights renormalised to sum 1 if asked; one wave per token
+// softmax over the experts, k largest (ties: lower index), weights renormalised to sum 1 if asked; one wave per token.
+// The logits of a token sit in registers (NQ per lane, expert = lane + 64 q); every selection is two wave reductions
+// on the VALU: the maximum, then the smallest index that holds it.
+template <int NQ>
 __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ logits, int64_t stride, int n_experts, int k, bool renorm,
                                                     int32_t * __restrict__ ids, float * __restrict__ weights) {
-    extern __shared__ float val[]; // logits of this token; taken ones become -inf
     const int t = blockIdx.x, lane = threadIdx.x;
     const float * lg = logits + (int64_t) t * stride;
+    float val[NQ]; // taken ones become -inf
     float mx = -INFINITY;
-    for (int i = lane; i < n_experts; i += 64) {
-        val[i] = lg[i];
-        mx = fmaxf(mx, lg[i]);
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        const int i = lane + 64 * q;
+        val[q] = i < n_experts ? lg[i] : -INFINITY;
+        mx = fmaxf(mx, val[q]);
     }
-    for (int o = 32; o; o >>= 1) {
-        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-    }
+    mx = lane63(wave_max_dpp(mx));
     float sum = 0.f;
-    for (int i = lane; i < n_experts; i += 64) {
-        sum += expf(val[i] - mx);
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        sum += lane + 64 * q < n_experts ? expf(val[q] - mx) : 0.f;
     }
-    sum = wave_sum(sum);
+    sum = lane63(wave_sum_dpp(sum));
     float top = 0.f, mine = 0.f; // lane j keeps the j-th weight
     for (int j = 0; j < k; j++) {
-        float bv = -INFINITY;
-        int bi = 0x7FFFFFFF;
-        for (int i = lane; i < n_experts; i += 64) {
-            const float v = val[i];
-            if (v > bv) { // ascending i within a lane: the first maximum wins
-                bv = v;
-                bi = i;
-            }
+        float bv = val[0];
+#pragma unroll
+        for (int q = 1; q < NQ; q++) {
+            bv = fmaxf(bv, val[q]);
         }
-        for (int o = 32; o; o >>= 1) {
-            const float ov = __shfl_xor(bv, o, 64);
-            const int oi = __shfl_xor(bi, o, 64);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
-            }
+        bv = lane63(wave_max_dpp(bv));
+        uint32_t bi = 0xFFFFFFFFu;
+#pragma unroll
+        for (int q = NQ - 1; q >= 0; q--) {
+            bi = val[q] == bv ? (uint32_t) (lane + 64 * q) : bi; // descending q: the lowest index of the lane stays
         }
+        bi = lane63(wave_min_dpp(bi));
         const float pj = expf(bv - mx) / sum;
         top += pj;
         if (lane == (j & 63)) {
             mine = pj; // k <= 64
-            ids[(int64_t) t * k + j] = bi;
+            ids[(int64_t) t * k + j] = (int32_t) bi;
         }
-        if (lane == (bi & 63)) {
-            val[bi] = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            val[q] = (uint32_t) (lane + 64 * q) == bi ? -INFINITY : val[q];
         }
-        __builtin_amdgcn_wave_barrier();
     }
     if (lane < k) {
         weights[(int64_t) t * k + lane] = renorm ? mine / top : mine;
@@ -172,8 +171,11 @@ void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_
 
 void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
                         float * weights, hipStream_t stream) {
-    hipLaunchKernelGGL(k_router_topk, dim3(n_tok), dim3(64), (size_t) n_experts * 4, stream, logits, stride, n_experts, k, renorm, ids,
-                       weights);
+    if (n_experts <= 256) {
+        hipLaunchKernelGGL(k_router_topk<4>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights);
+    } else {
+        hipLaunchKernelGGL(k_router_topk<16>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights);
+    }
 }
 
 } // namespace dev

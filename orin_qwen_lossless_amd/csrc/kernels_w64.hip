@@ -109,7 +109,9 @@ struct chain {
 
 // N chains advance one unit each, instruction streams interleaved: while one chain waits for a table lookup the
 // other one issues.
-template <typename TX, int C, int NC, int N>
+// GLU (N = 2, NC = 1): chain 0 decodes a unit of the gate matrix, chain 1 the same unit of the up matrix (its table
+// LUT_WORDS behind the first), and the rows come out as silu(gate x) * (up x).
+template <typename TX, int C, int NC, int N, bool GLU = false>
 __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uint32_t * lut, const xchunk<TX> (&xr)[NC][geom<C>::XS],
                                           const cols & p, const col_view & cv, int R, int lane) {
     using G = geom<C>;
@@ -136,7 +138,7 @@ __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uin
 #pragma unroll
                 for (int k = 0; k < N; k++) {
                     uint32_t e0, e1;
-                    ch[k].dec.two(lut, e0, e1);
+                    ch[k].dec.two(GLU ? lut + k * LUT_WORDS : lut, e0, e1);
                     wp[k][2 * j] = merge(spread_lo(smw[k][j]), e0);
                     wp[k][2 * j + 1] = merge(spread_hi(smw[k][j]), e1);
                 }
@@ -161,12 +163,28 @@ __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uin
             }
         }
 #pragma unroll
-        for (int k = 0; k < N; k++) {
+        for (int k = 0; k < (GLU ? 1 : N); k++) {
             const int64_t row = ch[k].row;
 #pragma unroll
             for (int n = 0; n < NC; n++) {
                 char * y = cv.y + n * p.y_tok;
-                if (C >= 4) { // a body is one row
+                if (GLU) {
+                    if (C >= 4) {
+                        const float g = wave_sum_dpp(acc[0][n][0]), u = wave_sum_dpp(acc[N - 1][n][0]);
+                        if (lane == 63) {
+                            store_y(y, p.y_bf16, row, u * silu(g));
+                        }
+                    } else {
+#pragma unroll
+                        for (int s = 0; s < 2; s++) {
+                            const float g = C == 2 ? wave_sum_dpp(acc[0][n][s]) : half_wave_sum_dpp(acc[0][n][s]);
+                            const float u = C == 2 ? wave_sum_dpp(acc[N - 1][n][s]) : half_wave_sum_dpp(acc[N - 1][n][s]);
+                            if (C == 2 ? lane == 63 : l32 == 31) {
+                                store_y(y, p.y_bf16, C == 2 ? row + s : row + 2 * s + half, u * silu(g));
+                            }
+                        }
+                    }
+                } else if (C >= 4) { // a body is one row
                     const float v = wave_sum_dpp(acc[k][n][0]);
                     if (lane == 63) {
                         store_y(y, p.y_bf16, row, v);
@@ -238,6 +256,43 @@ __global__ void __launch_bounds__(1024) k_w64_mmv(const bf16n_weight w, const co
         } else {
             unit_pass<TX, C, NC, 1>(ch, lut, xr, p, cv, R, lane);
         }
+    }
+}
+
+// Fused gate / up + SwiGLU for two matrices of the same shape and unit size: every wave decodes its units of both
+// matrices side by side (the two chains) and writes silu(gate x) * (up x).
+template <typename TX, int C>
+__global__ void __launch_bounds__(1024) k_w64_glu(const bf16n_weight wg, const bf16n_weight wu, const cols p, int units_per_wave) {
+    using G = geom<C>;
+    constexpr int K = C * CHUNK;
+    __shared__ __align__(16) uint32_t lut[2 * LUT_WORDS];
+    extern __shared__ __align__(16) uint32_t rings[];
+    const w64_ptrs qg = w64p(wg), qu = w64p(wu);
+    stage_lut(lut, qg.lut);
+    stage_lut(lut + LUT_WORDS, qu.lut);
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int R = wg.R;
+    const col_view cv = col_setup(p, blockIdx.y);
+    xchunk<TX> xr[1][G::XS];
+#pragma unroll
+    for (int i = 0; i < G::XS; i++) {
+        xr[0][i].load(cv.x, (C == 1 ? 0 : (2 * i + half) * CHUNK) + 4 * l32);
+    }
+    __syncthreads();
+    const int64_t units = p.nrows / R;
+    const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
+    if (u_begin >= units) {
+        return;
+    }
+    const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
+    const int64_t gu0 = cv.rbase / R + u_begin;
+    chain<G::NB> ch[2];
+    uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
+    ch[0].start(ring, qg, gu0, u_end - u_begin, u_begin * R, R, K, lane);
+    ch[1].start(ring + WAVE_LDS_WORDS, qu, gu0, u_end - u_begin, u_begin * R, R, K, lane);
+    for (int64_t i = u_begin; i < u_end; i++) {
+        unit_pass<TX, C, 1, 2, true>(ch, lut, xr, p, cv, R, lane);
     }
 }
 
@@ -406,9 +461,19 @@ void set_attr_c() { set_attr_nc<TX, 1>(); set_attr_nc<TX, 2>(); set_attr_nc<TX, 
 
 } // namespace
 
+template <typename TX>
+void set_attr_glu() {
+    (void) hipFuncSetAttribute((const void *) k_w64_glu<TX, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(32));
+    (void) hipFuncSetAttribute((const void *) k_w64_glu<TX, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(32));
+    (void) hipFuncSetAttribute((const void *) k_w64_glu<TX, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(32));
+    (void) hipFuncSetAttribute((const void *) k_w64_glu<TX, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(32));
+}
+
 void w64_init() {
     set_attr_c<bf16_t>();
     set_attr_c<float>();
+    set_attr_glu<bf16_t>();
+    set_attr_glu<float>();
 }
 
 // shapes with a fused wave64 GEMV: K in {512, 1024, 2048, 4096} and units that hold whole loop bodies
@@ -443,6 +508,34 @@ void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf
         } else {
             mmv_c<float>(C, nc, grid, wpb * 64, wpb, stream, w, q, upw);
         }
+    }
+}
+
+template <typename TX>
+void glu_c(int C, dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & g, const bf16n_weight & u, const cols & p, int upw) {
+    const size_t shm = w64_shm(2 * wpb);
+    switch (C) {
+        case 1: hipLaunchKernelGGL((k_w64_glu<TX, 1>), grid, dim3(nt), shm, stream, g, u, p, upw); break;
+        case 2: hipLaunchKernelGGL((k_w64_glu<TX, 2>), grid, dim3(nt), shm, stream, g, u, p, upw); break;
+        case 4: hipLaunchKernelGGL((k_w64_glu<TX, 4>), grid, dim3(nt), shm, stream, g, u, p, upw); break;
+        default: hipLaunchKernelGGL((k_w64_glu<TX, 8>), grid, dim3(nt), shm, stream, g, u, p, upw); break;
+    }
+}
+
+// y = silu(gate x) * (up x), one column per launch row (dense tokens or (token, slot) pairs with expert ids)
+void launch_w64_glu(const bf16n_weight & gate, const bf16n_weight & up, const cols & p, int ncols, bool x_bf16, int cus,
+                    hipStream_t stream) {
+    const int C = (int) (gate.K / CHUNK);
+    const int64_t units = p.nrows / gate.R;
+    const int64_t max_waves = (int64_t) cus * 16 / (ncols < 1 ? 1 : ncols) < 16 ? 16 : (int64_t) cus * 16 / (ncols < 1 ? 1 : ncols);
+    const int64_t upw = (units + max_waves - 1) / max_waves;
+    const int64_t waves = (units + upw - 1) / upw;
+    const int wpb = (int) (waves < 4 ? waves : 4);
+    const dim3 grid((unsigned) ((waves + wpb - 1) / wpb), ncols);
+    if (x_bf16) {
+        glu_c<bf16_t>(C, grid, wpb * 64, wpb, stream, gate, up, p, (int) upw);
+    } else {
+        glu_c<float>(C, grid, wpb * 64, wpb, stream, gate, up, p, (int) upw);
     }
 }
 

@@ -22,6 +22,8 @@ void launch_compat_get_rows(const bf16n_weight & w, const void * ids, int64_t id
 void w64_init();
 bool w64_mmv_supported(const bf16n_weight & w, bool x_bf16);
 void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf16, bool multi_col, int cus, hipStream_t stream);
+void launch_w64_glu(const bf16n_weight & gate, const bf16n_weight & up, const cols & p, int ncols, bool x_bf16, int cus,
+                    hipStream_t stream);
 void launch_w64_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream);
 void launch_w64_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
                          int64_t dst_s1, int64_t row0, hipStream_t stream);

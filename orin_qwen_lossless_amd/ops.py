@@ -225,8 +225,11 @@ def roundtrip_equal(w: Weight, src: torch.Tensor, chunk_bytes: int = 64 << 20) -
 
 
 def _mmv_common(x: torch.Tensor, w: Weight, ids: torch.Tensor | None, rows_per_matrix: int, out_bf16: bool, glu: bool,
-                multi_col: bool = True) -> torch.Tensor:
+                multi_col: bool = True, up: Weight | None = None) -> torch.Tensor:
+    """glu: w holds [gate; up] per matrix.  up given: w is the gate matrix and up a separate matrix of the same shape
+    (the product is silu(gate x) * (up x) with as many rows as either)."""
     cw = _cweight(w)
+    cu = _cweight(up) if up is not None else None
     K, rows = w.meta.K, w.meta.rows
     _check_x(x, K, "x")
     a = _lib.MmvArgs()
@@ -285,7 +288,9 @@ def _mmv_common(x: torch.Tensor, w: Weight, ids: torch.Tensor | None, rows_per_m
         a.nrows = n_out
     L = _lib.lib()
     with torch.cuda.device(x.device):
-        if glu:
+        if cu is not None:
+            _lib.check(L.bf16n_mmv_glu2(C.byref(cw), C.byref(cu), C.byref(a), _stream()))
+        elif glu:
             _lib.check(L.bf16n_mmv_glu(C.byref(cw), C.byref(a), _stream()))
         else:
             _lib.check(L.bf16n_mmv(C.byref(cw), C.byref(a), _stream(), int(multi_col)))
@@ -303,27 +308,13 @@ def mmv_glu(x: torch.Tensor, w: Weight, ids: torch.Tensor | None = None, rows_pe
     return _mmv_common(x, w, ids, rows_per_matrix or w.meta.rows, out_dtype == torch.bfloat16, True)
 
 
-def mmv_glu2(x: torch.Tensor, gate: Weight, up: Weight, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    """silu(gate x) * (up x) for separate dense gate / up matrices (bf16n::mmv_glu(gate, up), core launch.h:61)."""
-    cg, cu = _cweight(gate), _cweight(up)
-    _check_x(x, gate.meta.K, "x")
-    if x.dim() != 2:
-        raise ValueError("bf16n.mmv_glu: dense x must be [tokens, K]")
-    out_bf16 = out_dtype == torch.bfloat16
-    T, n_out = x.shape[0], gate.meta.rows
-    y = torch.empty((T, n_out), dtype=out_dtype, device=x.device)
-    if T == 0:
-        return y
-    a = _lib.MmvArgs()
-    a.x, a.y = x.data_ptr(), y.data_ptr()
-    a.x_bf16, a.y_bf16 = int(x.dtype == torch.bfloat16), int(out_bf16)
-    a.ncols, a.n_used, a.x_per_slot = T, 1, 1
-    a.x_tok = x.stride(0) * x.element_size()
-    a.y_tok = n_out * (2 if out_bf16 else 4)
-    a.rows_per_matrix, a.nrows = n_out, n_out
-    with torch.cuda.device(x.device):
-        _lib.check(_lib.lib().bf16n_mmv_glu2(C.byref(cg), C.byref(cu), C.byref(a), _stream()))
-    return y
+def mmv_glu2(x: torch.Tensor, gate: Weight, up: Weight, ids: torch.Tensor | None = None, rows_per_matrix: int = 0,
+             out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """silu(gate x) * (up x) for separate gate / up matrices of one shape, dense or with expert ids
+    (bf16n::mmv_glu(gate, up), core launch.h:56-61)."""
+    if (gate.meta.K, gate.meta.rows) != (up.meta.K, up.meta.rows):
+        raise ValueError("bf16n.mmv_glu: gate/up shapes must match")
+    return _mmv_common(x, gate, ids, rows_per_matrix, out_dtype == torch.bfloat16, False, True, up)
 
 
 def linear(x: torch.Tensor, w: Weight, bias: torch.Tensor | None = None) -> torch.Tensor:
@@ -472,6 +463,14 @@ def router_topk(logits: torch.Tensor, k: int, renorm: bool = True) -> tuple[torc
     return wts, ids
 
 
+def glu2_supported(gate: Weight, up: Weight) -> bool:
+    """Layouts with a fused gate / up + SwiGLU GEMV (the rule of bf16n::mmv_glu(gate, up), core launch.h:56-61, plus
+    this build's wave64 units): same format, K, R and layout, not chunk-major."""
+    g, u = gate.meta, up.meta
+    return ((g.format, g.K, g.R, g.flags) == (u.format, u.K, u.R, u.flags) and not g.chunk_major
+            and (not g.wave64 or g.K in (512, 1024, 2048, 4096)))
+
+
 def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_weights: torch.Tensor,
                 topk_ids: torch.Tensor, n_experts: int) -> torch.Tensor:
     """Routed experts of one MoE layer: sum_k w_k * down(silu(gate x) * up x) over the top-k experts, BF16 out.
@@ -485,6 +484,8 @@ def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_we
     if T > GEMV_MAX_TOKENS and mm_ids_supported(gate, up) and mm_ids_supported(down):
         a = moe_mm_ids(x, topk_ids, gate, n_experts, up=up, out_dtype=torch.bfloat16)
         ys = moe_mm_ids(a, topk_ids, down, n_experts, out_dtype=torch.float32)
+    elif glu2_supported(gate, up):
+        ys = mmv(mmv_glu2(x, gate, up, topk_ids, N), down, topk_ids, H)
     else:
         g = mmv(x, gate, topk_ids, N)
         u = mmv(x, up, topk_ids, N)

@@ -169,6 +169,22 @@ def test_separate_gate_up_glu_equals_unfused(ops, fmt, R):
     assert torch.equal(fused, ops.swiglu(ops.mmv(x, g), ops.mmv(x, u)))
 
 
+@pytest.mark.parametrize("K,R", [(512, 16), (1024, 4), (2048, 8), (4096, 4)])
+def test_wave64_gate_up_glu_equals_unfused(ops, K, R):
+    # dense and with expert ids: the fused kernel runs the same two decode chains, so the results are identical
+    E, N, T, k = 4, 64, 3, 2
+    gb, ub = synth.weights(E * N, K, 26), synth.weights(E * N, K, 27)
+    g, u = enc(ops, gb, HP, R, False, True), enc(ops, ub, HP, R, False, True)
+    x = tbf16(synth.activations(T, K, 28))
+    assert torch.equal(ops.mmv_glu2(x, g, u), ops.swiglu(ops.mmv(x, g), ops.mmv(x, u)))
+    ids = torch.tensor([[0, 3], [2, 1], [3, 0]], dtype=torch.int32, device="cuda")
+    fused = ops.mmv_glu2(x, g, u, ids, N)
+    assert fused.shape == (T, k, N)
+    assert torch.equal(fused, ops.swiglu(ops.mmv(x, g, ids, N), ops.mmv(x, u, ids, N)))
+    f16 = ops.mmv_glu2(x, g, u, ids, N, out_dtype=torch.bfloat16)
+    assert np.array_equal(bits(f16), rne_bf16(fused.cpu().numpy()))
+
+
 def test_swiglu_and_combine(ops, oracle):
     rng = np.random.default_rng(1)
     g, u = rng.standard_normal(5000).astype(np.float32) * 3, rng.standard_normal(5000).astype(np.float32)
