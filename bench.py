@@ -129,6 +129,67 @@ def graph_us(fn, n: int = 16, reps: int = 30) -> float:
     return float(np.median(d)) * 1e3 / n
 
 
+def decode_step(ops, head, randw, randx, K: int, n_layers: int = 40, n_sets: int = 4) -> dict:
+    """One decode step of the 35B-A3B shape as a single HIP graph: n_layers x (qkv 5120 x K, o K x 4096, router, top-8 of
+    256 experts, fused gate/up, down, combine, shared expert) + the output projection.  n_sets distinct weight sets are
+    used in turn and every layer's input is the previous layer's output (re-normalised), so that layers sharing a
+    weight set route to different experts; attention itself is not part of this path."""
+    import numpy as np
+    import torch
+
+    E, topk, N = 256, 8, 512
+    sets, nbytes = [], {}
+    for _ in range(n_sets):
+        d = {}
+        for name, (rows, k, nm) in {"qkv": (5120, K, 1), "o": (K, 4096, 1), "router": (E, K, 1), "gate": (E * N, K, E),
+                                    "up": (E * N, K, E), "down": (E * K, N, E), "sh_gate_up": (2 * N, K, 1),
+                                    "sh_down": (K, N, 1)}.items():
+            ws, nb, _ = encode_to_device(ops, randw(rows, k), n_matrices=nm)
+            d[name] = ws[0]
+            nbytes[name] = nb
+        sets.append(d)
+    touched = n_layers * (nbytes["qkv"] + nbytes["o"] + nbytes["router"] + nbytes["sh_gate_up"] + nbytes["sh_down"]
+                          + (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * topk // E)
+    head_bytes = head.plane.numel() + head.aux.numel()
+    res = {"layers": n_layers, "weight_sets": n_sets}
+    for T in (1, 4):
+        xin = [randx(T, K) for _ in range(4)]
+        xbuf = xin[0].clone()
+
+        def step():
+            # the glue between the products is two residual adds and two norms per layer (without the norms the SwiGLU
+            # squares the activations layer after layer); the engine's attention is outside this path
+            h = xbuf
+            for layer in range(n_layers):
+                w = sets[layer % n_sets]
+                q = ops.linear(h, w["qkv"])
+                h = torch.nn.functional.rms_norm(h + ops.linear(q[:, :4096], w["o"]), (K,))
+                wts, ids = ops.router_topk(ops.mmv(h, w["router"]), topk)
+                y = ops.moe_experts(h, w["gate"], w["up"], w["down"], wts, ids, E)
+                sh = ops.mmv(ops.mmv_glu(h, w["sh_gate_up"]), w["sh_down"], out_dtype=torch.bfloat16)
+                h = torch.nn.functional.rms_norm(h + y + sh, (K,))
+            return ops.linear(h, head)
+
+        step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+
+        def replay(i):
+            xbuf.copy_(xin[i & 3])
+            graph.replay()
+
+        d, _ = time_kernel(replay, 12, 3)
+        t = float(np.median(d)) * 1e3
+        # experts touched: at most T * top-k distinct ones per layer
+        tb = touched + (n_layers * (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * topk // E) * (T - 1) + head_bytes
+        res[f"batch{T}"] = {"graph_us": round(t, 1), "compressed_bytes_touched_upper_bound": int(tb),
+                            "GBps": round(tb / t / 1e3, 1), "tokens_per_s": round(T / t * 1e6, 1)}
+        del graph
+    return res
+
+
 def suite(ops, w_head, head_copies, x1, K: int) -> dict:
     """The other configurations of the path, each timed with HIP events (median of 50 launches): batch 4 on the output
     projection, the small NIBBLE matrices, one MoE layer at batch 1 as a captured HIP graph, and the batched prefill."""
@@ -209,6 +270,7 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
             out[f"moe_prefill_T{T}_gate_up_{engine}"] = {
                 "gate_up": gdesc, "us": round(t, 1), "gate_up_us": round(t_gu, 1), "TFLOPs": round(flops / t / 1e6, 2),
                 "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / 2500.0, 4), "tokens_per_s": round(T / t * 1e6, 0)}
+    out["decode_step"] = decode_step(ops, head_copies[0], randw, randx, K)
     return out
 
 

@@ -98,41 +98,46 @@ __global__ void __launch_bounds__(256) k_route(const char * __restrict__ ids, in
 
 // softmax over the experts, k largest (ties: lower index), weights renormalised to sum 1 if asked; one wave per token.
 // The logits of a token sit in registers (NQ per lane, expert = lane + 64 q); every selection is two wave reductions
-// on the VALU: the maximum, then the smallest index that holds it.
+// on the VALU: the maximum, then the smallest index that holds it.  NaN logits count as -inf, and a selection only
+// ever returns an index below n_experts that was not taken before, whatever the values are: the ids feed address
+// arithmetic in the kernels that follow.
 template <int NQ>
 __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ logits, int64_t stride, int n_experts, int k, bool renorm,
                                                     int32_t * __restrict__ ids, float * __restrict__ weights) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float * lg = logits + (int64_t) t * stride;
-    float val[NQ]; // taken ones become -inf
+    float val[NQ];
+    bool open[NQ]; // a real expert that has not been taken yet
     float mx = -INFINITY;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
         const int i = lane + 64 * q;
-        val[q] = i < n_experts ? lg[i] : -INFINITY;
+        open[q] = i < n_experts;
+        const float v = open[q] ? lg[i] : -INFINITY;
+        val[q] = v != v ? -INFINITY : v;
         mx = fmaxf(mx, val[q]);
     }
     mx = lane63(wave_max_dpp(mx));
     float sum = 0.f;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
-        sum += lane + 64 * q < n_experts ? expf(val[q] - mx) : 0.f;
+        sum += open[q] ? expf(val[q] - mx) : 0.f;
     }
     sum = lane63(wave_sum_dpp(sum));
     float top = 0.f, mine = 0.f; // lane j keeps the j-th weight
     for (int j = 0; j < k; j++) {
-        float bv = val[0];
+        float bv = -INFINITY;
 #pragma unroll
-        for (int q = 1; q < NQ; q++) {
-            bv = fmaxf(bv, val[q]);
+        for (int q = 0; q < NQ; q++) {
+            bv = open[q] ? fmaxf(bv, val[q]) : bv;
         }
         bv = lane63(wave_max_dpp(bv));
         uint32_t bi = 0xFFFFFFFFu;
 #pragma unroll
         for (int q = NQ - 1; q >= 0; q--) {
-            bi = val[q] == bv ? (uint32_t) (lane + 64 * q) : bi; // descending q: the lowest index of the lane stays
+            bi = open[q] && val[q] == bv ? (uint32_t) (lane + 64 * q) : bi; // descending q: the lane's lowest index stays
         }
-        bi = lane63(wave_min_dpp(bi));
+        bi = lane63(wave_min_dpp(bi)); // k <= n_experts: an open expert holds the maximum of the open ones
         const float pj = expf(bv - mx) / sum;
         top += pj;
         if (lane == (j & 63)) {
@@ -141,7 +146,7 @@ __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ l
         }
 #pragma unroll
         for (int q = 0; q < NQ; q++) {
-            val[q] = (uint32_t) (lane + 64 * q) == bi ? -INFINITY : val[q];
+            open[q] = open[q] && (uint32_t) (lane + 64 * q) != bi;
         }
     }
     if (lane < k) {

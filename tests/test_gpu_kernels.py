@@ -221,6 +221,20 @@ def test_routing_lists(ops, oracle, T, k, E, idt):
         assert np.array_equal(src1.cpu().numpy(), o_src1)
 
 
+def test_router_topk_ids_stay_valid_on_bad_logits(ops):
+    # NaN / infinite logits: the ids are still k distinct experts below n_experts (they feed address arithmetic)
+    lg = torch.full((4, 200), float("nan"), device="cuda")
+    lg[1] = float("-inf")
+    lg[2] = float("inf")
+    lg[3, ::3] = 1.0
+    _, ids = ops.router_topk(lg, 8)
+    ids = ids.cpu().numpy()
+    for t in range(4):
+        assert ids[t].min() >= 0 and ids[t].max() < 200 and len(set(ids[t].tolist())) == 8
+    assert ids[0].tolist() == list(range(8))          # all equal (-inf after NaN): lowest indices first
+    assert ids[3].tolist() == [0, 3, 6, 9, 12, 15, 18, 21]
+
+
 def test_router_topk(ops, oracle):
     rng = np.random.default_rng(4)
     lg = rng.standard_normal((5, 256)).astype(np.float32) * 2
