@@ -325,6 +325,13 @@ def main() -> None:
     xt = x[0].contiguous()
     bd, _ = time_kernel(lambda i: torch.mv(w2[i & 1], xt), min(args.steps, 100), 10)
     blas_us = float(np.median(bd)) * 1e3
+    # a plain streaming read of as many bytes as the compressed matrix (stock reduction over an FP64 view, two
+    # buffers alternated): what the memory system gives a kernel that does nothing but read
+    nread = comp_bytes // 8 * 8
+    bufs = [torch.randint(0, 255, (nread,), dtype=torch.uint8, device="cuda") for _ in range(2)]
+    sd, _ = time_kernel(lambda i: bufs[i & 1].view(torch.float64).sum(), 30, 5)
+    stream_gbs = nread / (float(np.median(sd)) * 1e-3) / 1e9
+    del bufs
 
     out = {
         "metric": "fused decode+GEMV HBM GB/s (% peak, compressed bytes); us/decode step vs BF16",
@@ -344,7 +351,8 @@ def main() -> None:
                      "median_launch_us": round(float(np.median(durs)) * 1e3, 2)},
         "extra": {"pct_of_hbm_peak_compressed": round(100 * comp_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
                   "us_per_matrix": round(ms * 1e3, 2), "blas_bf16_gemv_us": round(blas_us, 2),
-                  "speedup_vs_blas_bf16": round(blas_us / (ms * 1e3), 3), "tokens_per_s_lm_head_only": round(1e3 / ms, 1),
+                  "speedup_vs_blas_bf16": round(blas_us / (ms * 1e3), 3),
+                  "plain_stream_read_GBps": round(stream_gbs, 1), "kernel_vs_plain_stream_read": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / stream_gbs, 3), "tokens_per_s_lm_head_only": round(1e3 / ms, 1),
                   "host_encode_s": round(t_enc, 2), "max_err_over_sum_abs": err, "setup_s": round(time.perf_counter() - t0, 1)},
     }
     if args.suite:

@@ -1,0 +1,71 @@
+"""The headline configuration at its real size (output projection 248320 x 2048, HUFPAIR under the mi355x policy),
+checked through properties that do not need an oracle run of that size: decode(encode(w)) == w bit for bit over the whole
+matrix, a one-hot activation returns the exact weight column, and the product of a random activation stays within the
+FP64 bound of the exact weights."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+ROWS, K = 248320, 2048
+
+
+@pytest.fixture(scope="module")
+def head(ops):
+    g = torch.Generator(device="cuda").manual_seed(1)
+    w = torch.empty((ROWS, K), dtype=torch.bfloat16, device="cuda")
+    for r0 in range(0, ROWS, 1 << 15):
+        n = min(1 << 15, ROWS - r0)
+        w[r0: r0 + n] = (torch.randn((n, K), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    # a few rows of special values: zeros, denormals, infinities, NaNs, the largest finite magnitudes
+    special = torch.tensor([0x0000, 0x8000, 0x0001, 0x807F, 0x7F7F, 0xFF7F, 0x7F80, 0xFF80, 0x7FC1, 0xFFFF, 0x3F80],
+                           dtype=torch.int32).to(torch.int16)
+    w.view(torch.int16)[ROWS - 7, : special.numel()] = special.cuda()
+    fmt, R, cm, _, w64 = ops.choose(ROWS, K, engine="mi355x")
+    wbits = w.cpu().view(torch.int16).numpy().view(np.uint16)
+    plane, aux, fmt_out, _ = ops.encode_bits(wbits, fmt, R, cm, wave64=w64)
+    ta = torch.from_numpy(aux)
+    enc = ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
+    assert (fmt_out, R, w64) == (3, 16, True)
+    return w, enc
+
+
+def test_full_size_round_trip_is_bit_exact(ops, head):
+    w, enc = head
+    assert ops.roundtrip_equal(enc, w)
+
+
+def test_full_size_one_hot_returns_the_weight_column(ops, head):
+    w, enc = head
+    for col in (0, 777, K - 1):
+        x = torch.zeros((1, K), dtype=torch.bfloat16, device="cuda")
+        x[0, col] = 0.5
+        y = ops.mmv(x, enc)[0]
+        want = w[:, col].float() * 0.5
+        keep = torch.ones(ROWS, dtype=torch.bool, device="cuda")
+        keep[ROWS - 7] = False
+        assert torch.equal(y[keep], want[keep])
+        # the row that holds infinities and NaNs: 0 * inf is NaN in IEEE arithmetic, the product must not hide it
+        assert bool(torch.isnan(y[ROWS - 7]))
+
+
+def test_full_size_product_within_fp64_bound(ops, head):
+    w, enc = head
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn((4, K), generator=g, device="cuda").to(torch.bfloat16)
+    y = ops.mmv(x, enc)
+    keep = torch.ones(ROWS, dtype=torch.bool, device="cuda")
+    keep[ROWS - 7] = False  # the row of special values has no finite bound
+    for t in range(4):
+        ref = torch.zeros(ROWS, dtype=torch.float64, device="cuda")
+        bound = torch.zeros(ROWS, dtype=torch.float64, device="cuda")
+        for r0 in range(0, ROWS, 1 << 15):
+            wd = w[r0: r0 + (1 << 15)].double()
+            ref[r0: r0 + wd.shape[0]] = wd @ x[t].double()
+            bound[r0: r0 + wd.shape[0]] = wd.abs() @ x[t].double().abs()
+        err = (y[t].double() - ref).abs()
+        assert bool((err[keep] <= 1e-5 * bound[keep]).all())
+    # batch columns equal single-column launches bit for bit (compared as bits: one row is NaN)
+    assert torch.equal(ops.mmv(x[1:2], enc)[0].view(torch.int32), y[1].view(torch.int32))
