@@ -12,8 +12,8 @@
 //   * reference chunk-major HUFPAIR, R = 8, K = 2048 (gate / up; also fused gate + up + SwiGLU): a half-wavefront per
 //     unit, 8 units per slab;
 //   * reference row-major HUFPAIR, R = 16, K = 512 (down): a half-wavefront per unit, 4 units per slab;
-//   * wave64 HUFPAIR, R = 16, K = 512 (down under the mi355x policy): a wavefront per unit, 4 units per slab;
-//   * wave64 HUFPAIR, R = 8, K = 2048 (gate / up under the mi355x policy): k_mm_ids_w64k below.
+//   * wave64 HUFPAIR, R = 4, 8 or 16, K = 512 (down under the mi355x policy): a wavefront per 16 rows, 64 rows per slab;
+//   * wave64 HUFPAIR, R = 2, 4 or 8, K = 2048 (gate / up under the mi355x policy): k_mm_ids_w64k below.
 #include "dev_common.h"
 #include "dev_compat.h"
 #include "dev_w64.h"
@@ -63,20 +63,21 @@ template <int LAYOUT>
 struct slab_dec {
     lane_bits bits;        // 32-lane layouts
     w64_dec w64;           // wave64 layout
-    const uint8_t * plane; // first plane byte of this thread's unit
+    const uint8_t * plane; // first plane byte of this thread's unit (wave64: of its run of units)
     bool active;
+    int unit_steps;        // wave64: steps per unit
 
     __device__ __forceinline__ void begin(const bf16n_weight & w, int64_t gu0, uint32_t * ring, int tid) {
         using L = lay<LAYOUT>;
         const int lane = tid & 63, l32 = tid & 31;
-        if (LAYOUT == L_W64) {
-            const int64_t gu = gu0 + (tid >> 6);
+        if (LAYOUT == L_W64) { // 16 rows per wavefront: a run of 16 / R consecutive units (R = 4, 8 or 16)
+            const int run = L::R / w.R;
+            const int64_t gu = (gu0 + (tid >> 6)) * run;
             const w64_ptrs q = w64p(w);
             active = true;
-            plane = q.plane + gu * L::R * (int64_t) (L::C * CHUNK);
-            w64.start(ring + (tid >> 6) * WAVE_LDS_WORDS, q.stream, uniform(q.ubase[gu]), uniform(q.ubase[gu + 1]), lane);
-            w64.keep_ahead();
-            w64.begin_unit();
+            unit_steps = w.R / 2;
+            plane = q.plane + gu * w.R * (int64_t) (L::C * CHUNK);
+            w64.start(ring + (tid >> 6) * WAVE_LDS_WORDS, q.stream, uniform(q.ubase[gu]), uniform(q.ubase[gu + run]), lane);
         } else {
             const int u = tid >> 5;
             active = u < L::UNITS;
@@ -97,6 +98,10 @@ struct slab_dec {
                 const int step = 4 * h + st;
                 uint32_t wp[8];
                 w64.keep_ahead();
+                if (step % unit_steps == 0) {
+                    w64.begin_unit();
+                    w64.keep_ahead();
+                }
                 w64.step(lut, *((const uint4 *) (plane + step * 1024) + lane), wp);
                 tile_put(tile, wv * 8 + 2 * st + (lane >> 5), l32, wp);
             }
@@ -137,7 +142,7 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids(const bf16n_weight w, con
         }
     }
     const int slabs = (int) (a.rows / SLAB_ROWS);
-    const int64_t units_per_expert = a.rows / L::R;
+    const int64_t units_per_expert = a.rows / L::R; // wave64: runs of units that make 16 rows
     for (int item = blockIdx.x; item < a.n_experts * slabs; item += gridDim.x) {
         const int e = item / slabs, sl = item % slabs;
         const int j0 = a.bounds[e], n = a.bounds[e + 1] - j0;
@@ -217,7 +222,7 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids(const bf16n_weight w, con
 // wave64 row-major units of 8 rows, K = 2048 (gate / up under the mi355x policy).  A row-major unit stream yields whole
 // rows, so the tile holds 32 full rows (4 units, one per wavefront; 128.5 KiB) and a work item is one decode phase and
 // one product phase per matrix; the table in LDS is swapped between gate and up.  One block per CU.
-constexpr int WK_ROWS = 32, WK_K = 2048, WK_STRIDE = WK_K + 8, WK_R = 8;
+constexpr int WK_ROWS = 32, WK_K = 2048, WK_STRIDE = WK_K + 8, WK_WAVE_ROWS = 8;
 
 template <bool GLU>
 __global__ void __launch_bounds__(MM_THREADS) k_mm_ids_w64k(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
@@ -228,7 +233,8 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids_w64k(const bf16n_weight w
     uint32_t * rings = shm + LUT_WORDS + WK_ROWS * WK_STRIDE / 2;
     const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, wave = tid >> 6;
     const int slabs = (int) (a.rows / WK_ROWS);
-    const int64_t units_per_expert = a.rows / WK_R;
+    const int run = WK_WAVE_ROWS / w.R, unit_steps = 2 * w.R; // a wavefront decodes 8 rows: a run of 8 / R units (R = 2, 4, 8)
+    const int64_t units_per_expert = a.rows / w.R;
     int staged = -1; // which matrix's table is in LDS
     for (int item = blockIdx.x; item < a.n_experts * slabs; item += gridDim.x) {
         const int e = item / slabs, sl = item % slabs;
@@ -255,21 +261,23 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids_w64k(const bf16n_weight w
                     staged = m;
                     __syncthreads();
                 }
-                {   // this wavefront's unit: 8 rows = 16 steps of (row, chunk pair)
-                    const int64_t gu = e * units_per_expert + (int64_t) sl * (WK_ROWS / WK_R) + wave;
+                {   // this wavefront's 8 rows = 16 steps of (row, chunk pair)
+                    const int64_t gu = e * units_per_expert + ((int64_t) sl * (WK_ROWS / WK_WAVE_ROWS) + wave) * run;
                     const w64_ptrs q = w64p(wm);
-                    const uint8_t * plane = q.plane + gu * WK_R * (int64_t) WK_K;
+                    const uint8_t * plane = q.plane + gu * wm.R * (int64_t) WK_K;
                     w64_dec dec;
-                    dec.start(rings + wave * WAVE_LDS_WORDS, q.stream, uniform(q.ubase[gu]), uniform(q.ubase[gu + 1]), lane);
-                    dec.keep_ahead();
-                    dec.begin_unit();
+                    dec.start(rings + wave * WAVE_LDS_WORDS, q.stream, uniform(q.ubase[gu]), uniform(q.ubase[gu + run]), lane);
 #pragma unroll 1
-                    for (int st = 0; st < 2 * WK_R; st++) {
+                    for (int st = 0; st < 2 * WK_WAVE_ROWS; st++) {
                         uint32_t wp[8];
                         dec.keep_ahead();
+                        if (st % unit_steps == 0) {
+                            dec.begin_unit();
+                            dec.keep_ahead();
+                        }
                         dec.step(lut, *((const uint4 *) (plane + st * 1024) + lane), wp);
                         // chunk 2 (st % 2) + lane / 32 of row st / 2
-                        uint16_t * trow = tile + (wave * WK_R + st / 2) * WK_STRIDE + (2 * (st & 1) + (lane >> 5)) * CHUNK;
+                        uint16_t * trow = tile + (wave * WK_WAVE_ROWS + st / 2) * WK_STRIDE + (2 * (st & 1) + (lane >> 5)) * CHUNK;
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
                             *(uint2 *) (trow + 128 * j + 4 * l32) = make_uint2(wp[2 * j], wp[2 * j + 1]);
@@ -321,10 +329,10 @@ int layout_of(const bf16n_weight & w) {
     if (cm && !w64 && w.K == 2048 && w.R == 8) {
         return L_CM8;
     }
-    if (!cm && w.K == 512 && w.R == 16) {
+    if (!cm && w.K == 512 && (w.R == 16 || (w64 && (w.R == 8 || w.R == 4)))) {
         return w64 ? L_W64 : L_RM16;
     }
-    if (!cm && w64 && w.K == WK_K && w.R == WK_R) {
+    if (!cm && w64 && w.K == WK_K && (w.R == 8 || w.R == 4 || w.R == 2)) {
         return L_W64K;
     }
     return -1;
@@ -362,7 +370,7 @@ bool mm_ids_shape_ok(const bf16n_weight & w, const bf16n_weight * up) {
     if (!up) {
         return true;
     }
-    return (l == L_CM8 || l == L_W64K) && layout_of(*up) == l && up->rows == w.rows;
+    return (l == L_CM8 || l == L_W64K) && layout_of(*up) == l && up->rows == w.rows && up->R == w.R;
 }
 
 void launch_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,

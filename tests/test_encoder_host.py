@@ -168,7 +168,7 @@ def test_policy_mi355x():
     assert ops.choose(248320, 2048) == (HP, 16, False, False, True)
     assert ops.choose(5120, 2048) == (HP, 4, False, False, True)
     assert ops.choose(2048, 4096) == (HP, 2, False, False, True)
-    assert ops.choose(512, 2048, 256, expert=True) == (HP, 8, False, False, True)
+    assert ops.choose(512, 2048, 256, expert=True) == (HP, 4, False, False, True)
     assert ops.choose(2048, 512, 256, expert=True) == (HP, 16, False, False, True)
     assert ops.choose(512, 2048)[0] == NIB and ops.choose(2048, 512)[0] == NIB and ops.choose(256, 2048)[0] == NIB
     # shapes without a wave64 GEMV instance keep the reference layouts

@@ -18,7 +18,8 @@ HP = 3
 
 # (K, rows per expert, R, chunk_major, wave64): gate / up in reference chunk-major units and in wave64 units; down in
 # reference row-major units and in wave64 units
-SHAPES = [(2048, 128, 8, True, False), (2048, 128, 8, False, True), (512, 256, 16, False, False), (512, 256, 16, False, True)]
+SHAPES = [(2048, 128, 8, True, False), (2048, 128, 8, False, True), (2048, 128, 4, False, True), (2048, 128, 2, False, True),
+          (512, 256, 16, False, False), (512, 256, 16, False, True), (512, 256, 8, False, True), (512, 256, 4, False, True)]
 
 
 def routing(T: int, k: int, E: int, counts: dict[int, int], seed: int) -> np.ndarray:
