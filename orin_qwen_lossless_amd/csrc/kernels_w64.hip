@@ -87,9 +87,9 @@ struct chain {
         const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
         return *((const uint4 *) (plane + o) + lane);
     }
+    // first / end: the stream words of units [gu0, gu0 + n_units) (unit bases, read by the caller ahead of time)
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t gu0, int64_t n_units, int64_t row0, int R, int K,
-                                          int lane) {
-        dec.start(ring, q.stream, uniform(q.ubase[gu0]), uniform(q.ubase[gu0 + n_units]), lane);
+                                          int lane, uint32_t first, uint32_t end) {
         plane = q.plane + uniform64(gu0 * R * K);
         off = 0;
         last = (uint32_t) (n_units * R * K - 1024);
@@ -99,6 +99,7 @@ struct chain {
             sm[s] = load_step(lane);
             off += 1024;
         }
+        dec.start(ring, q.stream, uniform(first), uniform(end), lane);
     }
     // plane bytes of step s of the next body, once step s of this body is consumed
     __device__ __forceinline__ void reload(int s, int lane) {
@@ -221,34 +222,37 @@ __global__ void __launch_bounds__(1024) k_w64_mmv(const bf16n_weight w, const co
     __shared__ __align__(16) uint32_t lut[LUT_WORDS];          // static: sits at LDS address 0
     extern __shared__ __align__(16) uint32_t rings[];          // per wave and chain: RING + RING_PAD words
     const w64_ptrs q = w64p(w);
-    stage_lut(lut, q.lut);
     const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int R = w.R;
     const col_view cv = col_setup(p, blockIdx.y * NC);
+    const int64_t units = p.nrows / R;
+    const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
+    const bool live = u_begin < units;
+    const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
+    const int64_t n = live ? u_end - u_begin : 0, nA = NCH == 2 ? (n + 1) / 2 : n, nB = n - nA;
+    const int64_t gu0 = cv.rbase / R + (live ? u_begin : 0);
+    // the unit bases first: the dependent stream loads can then start as soon as the table is staged
+    const uint32_t b0 = q.ubase[gu0], b1 = q.ubase[gu0 + nA], b2 = q.ubase[gu0 + n];
+    stage_lut(lut, q.lut);
     // activations: chunk 2i + half of the row for i < XS (C = 1: chunk 0 for both halves)
     xchunk<TX> xr[NC][G::XS];
 #pragma unroll
-    for (int n = 0; n < NC; n++) {
+    for (int n_ = 0; n_ < NC; n_++) {
 #pragma unroll
         for (int i = 0; i < G::XS; i++) {
-            xr[n][i].load(cv.x + n * p.x_tok, (C == 1 ? 0 : (2 * i + half) * CHUNK) + 4 * l32);
+            xr[n_][i].load(cv.x + n_ * p.x_tok, (C == 1 ? 0 : (2 * i + half) * CHUNK) + 4 * l32);
         }
     }
     __syncthreads();
-    const int64_t units = p.nrows / R;
-    const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
-    if (u_begin >= units) {
+    if (!live) {
         return;
     }
-    const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
-    const int64_t n = u_end - u_begin, nA = NCH == 2 ? (n + 1) / 2 : n, nB = n - nA;
-    const int64_t gu0 = cv.rbase / R + u_begin;
     chain<G::NB> ch[2];
     uint32_t * ring = rings + wave * (NCH * WAVE_LDS_WORDS);
-    ch[0].start(ring, q, gu0, nA, u_begin * R, R, K, lane);
+    ch[0].start(ring, q, gu0, nA, u_begin * R, R, K, lane, b0, b1);
     if (NCH == 2 && nB > 0) {
-        ch[1].start(ring + WAVE_LDS_WORDS, q, gu0 + nA, nB, (u_begin + nA) * R, R, K, lane);
+        ch[1].start(ring + WAVE_LDS_WORDS, q, gu0 + nA, nB, (u_begin + nA) * R, R, K, lane, b1, b2);
     }
     for (int64_t i = 0; i < nA; i++) {
         if (NCH == 2 && i < nB) {
@@ -268,30 +272,33 @@ __global__ void __launch_bounds__(1024) k_w64_glu(const bf16n_weight wg, const b
     __shared__ __align__(16) uint32_t lut[2 * LUT_WORDS];
     extern __shared__ __align__(16) uint32_t rings[];
     const w64_ptrs qg = w64p(wg), qu = w64p(wu);
-    stage_lut(lut, qg.lut);
-    stage_lut(lut + LUT_WORDS, qu.lut);
     const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int R = wg.R;
     const col_view cv = col_setup(p, blockIdx.y);
+    const int64_t units = p.nrows / R;
+    const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
+    const bool live = u_begin < units;
+    const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
+    const int64_t n = live ? u_end - u_begin : 0;
+    const int64_t gu0 = cv.rbase / R + (live ? u_begin : 0);
+    const uint32_t g0 = qg.ubase[gu0], g1 = qg.ubase[gu0 + n], u0 = qu.ubase[gu0], u1 = qu.ubase[gu0 + n];
+    stage_lut(lut, qg.lut);
+    stage_lut(lut + LUT_WORDS, qu.lut);
     xchunk<TX> xr[1][G::XS];
 #pragma unroll
     for (int i = 0; i < G::XS; i++) {
         xr[0][i].load(cv.x, (C == 1 ? 0 : (2 * i + half) * CHUNK) + 4 * l32);
     }
     __syncthreads();
-    const int64_t units = p.nrows / R;
-    const int64_t u_begin = ((int64_t) blockIdx.x * nwaves + wave) * units_per_wave;
-    if (u_begin >= units) {
+    if (!live) {
         return;
     }
-    const int64_t u_end = u_begin + units_per_wave < units ? u_begin + units_per_wave : units;
-    const int64_t gu0 = cv.rbase / R + u_begin;
     chain<G::NB> ch[2];
     uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-    ch[0].start(ring, qg, gu0, u_end - u_begin, u_begin * R, R, K, lane);
-    ch[1].start(ring + WAVE_LDS_WORDS, qu, gu0, u_end - u_begin, u_begin * R, R, K, lane);
-    for (int64_t i = u_begin; i < u_end; i++) {
+    ch[0].start(ring, qg, gu0, n, u_begin * R, R, K, lane, g0, g1);
+    ch[1].start(ring + WAVE_LDS_WORDS, qu, gu0, n, u_begin * R, R, K, lane, u0, u1);
+    for (int64_t i = 0; i < n; i++) {
         unit_pass<TX, C, 1, 2, true>(ch, lut, xr, p, cv, R, lane);
     }
 }
