@@ -91,9 +91,15 @@ struct slab_dec {
     __device__ __forceinline__ void phase(const uint32_t * lut, uint16_t * tile, int c, int h, int tid) {
         using L = lay<LAYOUT>;
         const int lane = tid & 63, l32 = tid & 31;
+        // the plane words of the whole phase are requested first: the decode below then waits for table lookups only
         if (LAYOUT == L_W64) {
             const int wv = tid >> 6;
-#pragma unroll 1
+            uint4 sm[4];
+#pragma unroll
+            for (int st = 0; st < 4; st++) {
+                sm[st] = *((const uint4 *) (plane + (4 * h + st) * 1024) + lane);
+            }
+#pragma unroll
             for (int st = 0; st < 4; st++) { // a step holds rows 2 step (lanes 0..31) and 2 step + 1 (lanes 32..63)
                 const int step = 4 * h + st;
                 uint32_t wp[8];
@@ -102,17 +108,22 @@ struct slab_dec {
                     w64.begin_unit();
                     w64.keep_ahead();
                 }
-                w64.step(lut, *((const uint4 *) (plane + step * 1024) + lane), wp);
+                w64.step(lut, sm[st], wp);
                 tile_put(tile, wv * 8 + 2 * st + (lane >> 5), l32, wp);
             }
         } else if (active) {
             const int u = tid >> 5;
-#pragma unroll 1
+            uint4 sm[L::ROWS_PER_PHASE];
+#pragma unroll
             for (int i = 0; i < L::ROWS_PER_PHASE; i++) {
                 const int rr = L::ROWS_PER_PHASE * h + i;
                 const int64_t o = LAYOUT == L_CM8 ? (int64_t) c * L::R + rr : rr; // position of (row, chunk) in the unit
+                sm[i] = *((const uint4 *) (plane + o * CHUNK) + l32);
+            }
+#pragma unroll
+            for (int i = 0; i < L::ROWS_PER_PHASE; i++) {
                 uint32_t wp[8];
-                decode_chunk<FMT_HUFPAIR>(bits, lut, *((const uint4 *) (plane + o * CHUNK) + l32), wp);
+                decode_chunk<FMT_HUFPAIR>(bits, lut, sm[i], wp);
                 tile_put(tile, u * L::ROWS_PER_PHASE + i, l32, wp);
             }
         }
@@ -127,7 +138,7 @@ __device__ __forceinline__ int slab_row(int t, int h) {
 }
 
 template <int LAYOUT, bool GLU>
-__global__ void __launch_bounds__(MM_THREADS) k_mm_ids(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+__global__ void __launch_bounds__(MM_THREADS, 2) k_mm_ids(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
     using L = lay<LAYOUT>;
     constexpr int NM = GLU ? 2 : 1;
     extern __shared__ __align__(16) uint32_t shm[];
@@ -171,6 +182,13 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids(const bf16n_weight w, con
             }
 #pragma unroll 1
             for (int c = 0; c < L::C; c++) {
+                // the activations of this chunk (B operands of its 32 matrix instructions) are requested before the
+                // decode and stay in registers for the chunk's phases
+                bf16x8_t bv[CHUNK / 16];
+#pragma unroll
+                for (int ks = 0; ks < CHUNK / 16; ks++) {
+                    bv[ks] = *(const bf16x8_t *) (xrow + c * CHUNK + 16 * ks);
+                }
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
 #pragma unroll
@@ -180,12 +198,10 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids(const bf16n_weight w, con
                         __syncthreads();
                         if (wave_has) {
                             const uint16_t * ap = tile + (lane & 31) * TILE_STRIDE + 8 * (lane >> 5);
-                            const uint16_t * bp = xrow + c * CHUNK;
-#pragma unroll 8
+#pragma unroll
                             for (int ks = 0; ks < CHUNK / 16; ks++) {
                                 const bf16x8_t av = *(const bf16x8_t *) (ap + 16 * ks);
-                                const bf16x8_t bv = *(const bf16x8_t *) (bp + 16 * ks);
-                                acc[m][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[m][h], 0, 0, 0);
+                                acc[m][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv[ks], acc[m][h], 0, 0, 0);
                             }
                         }
                     }
@@ -224,9 +240,86 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids(const bf16n_weight w, con
 // one product phase per matrix; the table in LDS is swapped between gate and up.  One block per CU.
 constexpr int WK_ROWS = 32, WK_K = 2048, WK_STRIDE = WK_K + 8, WK_WAVE_ROWS = 8;
 
+// one matrix of a work item: stage its table if needed, decode this wavefront's 8 rows into the tile, multiply
+__device__ __forceinline__ void wk_matrix(const bf16n_weight & wm, int m, int & staged, uint32_t * lut, uint16_t * tile, uint32_t * rings,
+                                          int64_t gu, int run, int unit_steps, const uint16_t * xrow, bool wave_has, f32x16_t & acc) {
+    const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, wave = tid >> 6;
+    __syncthreads(); // tile and table are free
+    if (staged != m) {
+        stage_lut(lut, (const uint32_t *) (wm.aux + wm.off_a));
+        staged = m;
+        __syncthreads();
+    }
+    {   // this wavefront's 8 rows = 16 steps of (row, chunk pair)
+        const w64_ptrs q = w64p(wm);
+        const uint8_t * plane = q.plane + gu * wm.R * (int64_t) WK_K;
+        w64_dec dec;
+        dec.start(rings + wave * WAVE_LDS_WORDS, q.stream, uniform(q.ubase[gu]), uniform(q.ubase[gu + run]), lane);
+#pragma unroll 1
+        for (int s0 = 0; s0 < 2 * WK_WAVE_ROWS; s0 += 4) {
+            uint4 sm[4]; // the plane words of four steps, requested before their decode
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                sm[i] = *((const uint4 *) (plane + (s0 + i) * 1024) + lane);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int st = s0 + i;
+                uint32_t wp[8];
+                dec.keep_ahead();
+                if (st % unit_steps == 0) {
+                    dec.begin_unit();
+                    dec.keep_ahead();
+                }
+                dec.step(lut, sm[i], wp);
+                // chunk 2 (st % 2) + lane / 32 of row st / 2
+                uint16_t * trow = tile + (wave * WK_WAVE_ROWS + st / 2) * WK_STRIDE + (2 * (st & 1) + (lane >> 5)) * CHUNK;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    *(uint2 *) (trow + 128 * j + 4 * l32) = make_uint2(wp[2 * j], wp[2 * j + 1]);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (wave_has) {
+        // B operands (activations, 16 bytes per lane and instruction) in two register sets of 8: the next set is
+        // requested before the current one is multiplied
+        const uint16_t * ap = tile + l32 * WK_STRIDE + 8 * (lane >> 5);
+        constexpr int G = 8;
+        bf16x8_t bv[2][G];
+#pragma unroll
+        for (int i = 0; i < G; i++) {
+            bv[0][i] = *(const bf16x8_t *) (xrow + 16 * i);
+        }
+#pragma unroll 2
+        for (int g = 0; g < WK_K / 16 / G; g += 2) {
+#pragma unroll
+            for (int i = 0; i < G; i++) {
+                bv[1][i] = *(const bf16x8_t *) (xrow + 16 * ((g + 1) * G + i));
+            }
+#pragma unroll
+            for (int i = 0; i < G; i++) {
+                const bf16x8_t av = *(const bf16x8_t *) (ap + 16 * (g * G + i));
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv[0][i], acc, 0, 0, 0);
+            }
+            if (g + 2 < WK_K / 16 / G) {
+#pragma unroll
+                for (int i = 0; i < G; i++) {
+                    bv[0][i] = *(const bf16x8_t *) (xrow + 16 * ((g + 2) * G + i));
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < G; i++) {
+                const bf16x8_t av = *(const bf16x8_t *) (ap + 16 * ((g + 1) * G + i));
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv[1][i], acc, 0, 0, 0);
+            }
+        }
+    }
+}
+
 template <bool GLU>
 __global__ void __launch_bounds__(MM_THREADS) k_mm_ids_w64k(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
-    constexpr int NM = GLU ? 2 : 1;
     extern __shared__ __align__(16) uint32_t shm[];
     uint32_t * lut = shm;
     uint16_t * tile = (uint16_t *) (shm + LUT_WORDS);
@@ -244,56 +337,16 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids_w64k(const bf16n_weight w
             const bool wave_has = tp + wave * 32 < n, valid = tk < n;
             const int jj = j0 + (valid ? tk : 0);
             const uint16_t * xrow = a.x + (int64_t) a.ids_src1[jj] * a.x_row + 8 * (lane >> 5);
-            f32x16_t acc[NM];
+            const int64_t gu = e * units_per_expert + ((int64_t) sl * (WK_ROWS / WK_WAVE_ROWS) + wave) * run;
+            f32x16_t acc_g, acc_u;
 #pragma unroll
-            for (int m = 0; m < NM; m++) {
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    acc[m][i] = 0.f;
-                }
+            for (int i = 0; i < 16; i++) {
+                acc_g[i] = 0.f;
+                acc_u[i] = 0.f;
             }
-#pragma unroll
-            for (int m = 0; m < NM; m++) {
-                const bf16n_weight & wm = m == 0 ? w : w_up;
-                __syncthreads(); // tile and table are free
-                if (staged != m) {
-                    stage_lut(lut, (const uint32_t *) (wm.aux + wm.off_a));
-                    staged = m;
-                    __syncthreads();
-                }
-                {   // this wavefront's 8 rows = 16 steps of (row, chunk pair)
-                    const int64_t gu = e * units_per_expert + ((int64_t) sl * (WK_ROWS / WK_WAVE_ROWS) + wave) * run;
-                    const w64_ptrs q = w64p(wm);
-                    const uint8_t * plane = q.plane + gu * wm.R * (int64_t) WK_K;
-                    w64_dec dec;
-                    dec.start(rings + wave * WAVE_LDS_WORDS, q.stream, uniform(q.ubase[gu]), uniform(q.ubase[gu + run]), lane);
-#pragma unroll 1
-                    for (int st = 0; st < 2 * WK_WAVE_ROWS; st++) {
-                        uint32_t wp[8];
-                        dec.keep_ahead();
-                        if (st % unit_steps == 0) {
-                            dec.begin_unit();
-                            dec.keep_ahead();
-                        }
-                        dec.step(lut, *((const uint4 *) (plane + st * 1024) + lane), wp);
-                        // chunk 2 (st % 2) + lane / 32 of row st / 2
-                        uint16_t * trow = tile + (wave * WK_WAVE_ROWS + st / 2) * WK_STRIDE + (2 * (st & 1) + (lane >> 5)) * CHUNK;
-#pragma unroll
-                        for (int j = 0; j < 4; j++) {
-                            *(uint2 *) (trow + 128 * j + 4 * l32) = make_uint2(wp[2 * j], wp[2 * j + 1]);
-                        }
-                    }
-                }
-                __syncthreads();
-                if (wave_has) {
-                    const uint16_t * ap = tile + l32 * WK_STRIDE + 8 * (lane >> 5);
-#pragma unroll 8
-                    for (int ks = 0; ks < WK_K / 16; ks++) {
-                        const bf16x8_t av = *(const bf16x8_t *) (ap + 16 * ks);
-                        const bf16x8_t bv = *(const bf16x8_t *) (xrow + 16 * ks);
-                        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[m], 0, 0, 0);
-                    }
-                }
+            wk_matrix(w, 0, staged, lut, tile, rings, gu, run, unit_steps, xrow, wave_has, acc_g);
+            if (GLU) {
+                wk_matrix(w_up, 1, staged, lut, tile, rings, gu, run, unit_steps, xrow, wave_has, acc_u);
             }
             if (valid) { // accumulator element i: tile row 8 (i / 4) + 4 (lane / 32) + i % 4 = row of the slab
                 const int64_t col = (int64_t) a.ids_dst[jj] * a.dst_col + (int64_t) sl * WK_ROWS;
@@ -302,8 +355,8 @@ __global__ void __launch_bounds__(MM_THREADS) k_mm_ids_w64k(const bf16n_weight w
                     float v[4];
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const float p = acc[0][4 * g + i];
-                        v[i] = GLU ? acc[NM - 1][4 * g + i] * silu(p) : p;
+                        const float p = acc_g[4 * g + i];
+                        v[i] = GLU ? acc_u[4 * g + i] * silu(p) : p;
                     }
                     const int row = 8 * g + 4 * (lane >> 5);
                     if (a.dst_bf16) {
