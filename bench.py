@@ -39,20 +39,35 @@ def gen_weights(rows: int, K: int, seed: int):
     return w
 
 
-def time_kernel(fn, steps: int, warmup: int):
+def time_kernel(fn, steps: int, warmup: int, graph: bool = False):
     """Wall time of `steps` back-to-back launches (synchronised on both sides), then per-launch durations (ms) of a
     second pass from HIP events recorded around every launch on the launch stream (torch's current stream, which is the
-    one the library launches on)."""
+    one the library launches on).  graph: the `steps` launches of the wall-time pass are captured into one HIP graph
+    first and the timed region is its replay (the launchers only enqueue kernels), which keeps host launch overhead and
+    inter-launch gaps out of the job time."""
     import torch
 
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        fn(i)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(steps):
+                fn(i)
+        g.replay()  # untimed: the first replay uploads the graph
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        g.replay()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        del g
+    else:
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn(i)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for i in range(steps):
         ev[i][0].record()
@@ -283,6 +298,7 @@ def main() -> None:
     ap.add_argument("--K", type=int, default=2048)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=16384)
+    ap.add_argument("--no-graph", action="store_true", help="time the steps as separate launches instead of one HIP graph replay")
     ap.add_argument("--suite", action="store_true", help="also time batch 4, the NIBBLE matrices, a MoE layer and the prefill")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -317,7 +333,7 @@ def main() -> None:
 
     comp_bytes = plane.size + aux.size
     algo_bytes = comp_bytes + K * 2 + rows * 4  # weights (plane + aux incl. table, unit bases, padding) + x + y
-    durs, wall = time_kernel(lambda i: ops.mmv(x, copies[i & 1]), args.steps, args.warmup)
+    durs, wall = time_kernel(lambda i: ops.mmv(x, copies[i & 1]), args.steps, args.warmup, graph=not args.no_graph)
     ms = wall * 1e3 / args.steps
     kern_ms = float(np.mean(durs))
     # stock BF16 GEMV on the uncompressed tensor (the "vs BF16" column), same timing loop
@@ -341,7 +357,8 @@ def main() -> None:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"output projection {rows}x{K} BF16 N(0,0.02), {ops.FORMAT_NAMES[fmt_out]} R={R} "
                                f"{'wave64' if w64 else 'reference'} layout, fused decode+GEMV, batch 1 BF16 activations "
-                               "N(0,1), FP32 accumulate/out; 2 weight copies alternated",
+                               "N(0,1), FP32 accumulate/out; 2 weight copies alternated; the timed steps are "
+                               + ("separate launches" if args.no_graph else "one HIP graph replay"),
                    "rows": rows, "K": K, "batch": 1, "compressed_bytes": comp_bytes, "bits_per_weight": round(8 * comp_bytes / (rows * K), 4),
                    "ratio_of_bf16": round(comp_bytes / (2 * rows * K), 4)},
         "roofline": {"bound": "hbm", "achieved": round(algo_bytes / (kern_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
