@@ -283,3 +283,41 @@ def test_moe_layer_decode(ops, oracle, T, w64):
         acc += float(wts[0, s]) * (synth.bf16_bits_to_f32(down_b[e * H: (e + 1) * H]).astype(np.float64) @ a)
     got = y[0].float().cpu().numpy()
     assert np.all(np.abs(got - acc) <= 2.0 ** -7 * np.abs(acc) + 1e-4)
+
+
+@pytest.mark.parametrize("T", [1, 8, 9, 33])
+@pytest.mark.parametrize("fmt,R,cm,w64", [(NIB, 0, False, False), (HP, 16, False, True), (HP, 8, True, False)])
+def test_linear_both_token_regimes(ops, T, fmt, R, cm, w64):
+    # up to 8 tokens: decode GEMV, FP32 accumulation, bias added in FP32, one rounding to BF16; more: exact dequant +
+    # stock BF16 GEMM (restates the reference's linear, core/torch/torch_bindings.cpp:198-239)
+    K, rows = 1024, 208
+    wb = synth.weights(rows, K, 91)
+    w = enc(ops, wb, fmt, R, cm, w64)
+    xb = synth.activations(T, K, 92)
+    bias = tbf16(synth.weights(1, rows, 93)[0])
+    wf, xf = synth.bf16_bits_to_f32(wb).astype(np.float64), synth.bf16_bits_to_f32(xb).astype(np.float64)
+    ref = xf @ wf.T
+    for b in (None, bias):
+        y = ops.linear(tbf16(xb), w, b)
+        assert y.dtype == torch.bfloat16 and tuple(y.shape) == (T, rows)
+        want = ref + (b.float().cpu().numpy().astype(np.float64) if b is not None else 0.0)
+        got = y.float().cpu().numpy().astype(np.float64)
+        # BF16 has 8 significant bits: one rounding (GEMV path) or two (GEMM path, bias added after the first)
+        eps = 2.0 ** -8 if T <= 8 else 2.0 ** -7
+        assert np.all(np.abs(got - want) <= eps * (np.abs(want) + 0.05))
+    # leading batch dimensions are kept
+    y3 = ops.linear(tbf16(xb).reshape(1, T, K), w)
+    assert tuple(y3.shape) == (1, T, rows)
+    with pytest.raises(ValueError):
+        ops.linear(tbf16(xb).float(), w)
+
+
+def test_embedding_is_the_exact_rows(ops):
+    K, rows = 512, 96
+    wb = synth.weights(rows, K, 94)
+    for fmt, R, w64 in ((HP, 16, True), (HP, 16, False), (NIB, 0, False)):
+        w = enc(ops, wb, fmt, R, False, w64)
+        ids = torch.tensor([[0, 95, 17], [17, 16, 15]], dtype=torch.int64, device="cuda")
+        out = ops.embedding(ids, w)
+        assert tuple(out.shape) == (2, 3, K) and out.dtype == torch.bfloat16
+        assert np.array_equal(bits(out).reshape(6, K), wb[ids.cpu().numpy().reshape(-1)])
