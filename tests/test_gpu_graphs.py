@@ -90,3 +90,29 @@ def test_moe_layer_graph(ops, T):
     ref = ops.moe_experts_reference(x, gate, up, down, *ops.router_topk(ops.mmv(x, router)[:, :E].contiguous(), k), E)
     scale = float(ref.float().abs().max())
     assert float((out.float() - ref.float()).abs().max()) <= 2e-2 * scale
+
+
+def test_batched_moe_graph(ops):
+    # T = 64: routing lists, fused gate/up + SwiGLU and down run as batched kernels inside the graph
+    E, k, K, N, T = 8, 2, 2048, 512, 64
+    gate = enc(ops, synth.weights(E * N, K, 101), HP, 4, False, True)
+    up = enc(ops, synth.weights(E * N, K, 102), HP, 4, False, True)
+    down = enc(ops, synth.weights(E * K, N, 103), HP, 16, False, True)
+    assert ops.mm_ids_supported(gate, up) and ops.mm_ids_supported(down)
+    x = tbf16(synth.activations(T, K, 104))
+    logits = torch.randn((T, E), generator=torch.Generator().manual_seed(1)).cuda()
+
+    def layer():
+        wts, ids = ops.router_topk(logits, k)
+        return ops.moe_experts(x, gate, up, down, wts, ids, E)
+
+    g, out = capture(layer)
+    for rep in range(3):
+        x.copy_(tbf16(synth.activations(T, K, 110 + rep)))
+        logits.copy_(torch.randn((T, E), generator=torch.Generator().manual_seed(2 + rep)))
+        want = layer().clone()
+        torch.cuda.synchronize()
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep

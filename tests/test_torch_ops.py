@@ -103,3 +103,28 @@ def test_ops_equal_the_python_layer():
     assert torch.equal(B.swiglu(g, g * 2), ops.swiglu(g, g * 2))
     wts, ids = B.router_topk(torch.randn((4, 64), device="cuda"), 4, True)
     assert ids.shape == (4, 4) and torch.allclose(wts.sum(-1), torch.ones(4, device="cuda"), atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_opcheck_and_compile():
+    # schema and fake-tensor consistency of the registered ops, and a traced function without graph breaks
+    # (restates tests/core/test_opcheck.py of the reference)
+    B.init()
+    K, rows = 1024, 128
+    plane, aux = B.encode(bf16(synth.weights(rows, K, 81)), 3, 8, False)
+    meta = torch_ops.meta_of(aux)
+    pd, ad = plane.cuda().view(-1), aux.cuda()
+    x = bf16(synth.activations(2, K, 82)).cuda()
+    ids = torch.tensor([[0, 1], [1, 0]], dtype=torch.int32, device="cuda")
+    checks = ("test_schema", "test_faketensor")
+    torch.library.opcheck(B.mmv.default, (x, pd, ad, meta, None, 0, False), test_utils=checks)
+    torch.library.opcheck(B.mmv.default, (x, pd, ad, meta, ids, 64, True), test_utils=checks)
+    torch.library.opcheck(B.dequant.default, (pd, ad, meta, 8, 16), test_utils=checks)
+    torch.library.opcheck(B.linear.default, (x, pd, ad, meta, None), test_utils=checks)
+    torch.library.opcheck(B.swiglu.default, (torch.randn(4, 8, device="cuda"), torch.randn(4, 8, device="cuda")), test_utils=checks)
+
+    def f(x):
+        return B.swiglu(B.mmv(x, pd, ad, meta, None, 0, False), B.mmv(x, pd, ad, meta, None, 0, False))
+
+    got = torch.compile(f, fullgraph=True, backend="eager")(x)
+    assert torch.equal(got, f(x))
