@@ -277,17 +277,16 @@ __device__ __forceinline__ float nib_escapes(const nib_ptrs & w, int64_t gr, con
 template <typename TX, int GLU>
 __global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p) {
     __shared__ float part[2][HALVES];
-    const int K = (int) w.K, C = K / CHUNK; // 1, 2, 4 or 8: HALVES / C rows per block
+    const int K = (int) w.K, C = K / CHUNK; // 1 .. 8
     const col_view cv = col_setup(p, blockIdx.y);
     const nib_ptrs g = nibp(w, 0);
     const nib_ptrs u = GLU == 1 ? nibp(w, p.nrows) : nibp(w_up, 0);
     const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
-    const int64_t items = p.nrows * C;
-    for (int64_t base = (int64_t) blockIdx.x * HALVES; base < items; base += (int64_t) gridDim.x * HALVES) {
-        const int64_t q = base + half;
-        const bool live = q < items;
-        const int64_t r = live ? q / C : 0;
-        const int c = live ? (int) (q % C) : 0;
+    const int rpb = HALVES / C; // rows per block: C half-waves per row (C = 3, 5, 6, 7 leave some half-waves idle)
+    const int lr = half / C, c = half % C;
+    for (int64_t base = (int64_t) blockIdx.x * rpb; base < p.nrows; base += (int64_t) gridDim.x * rpb) {
+        const bool live = lr < rpb && base + lr < p.nrows;
+        const int64_t r = live ? base + lr : 0;
         const int64_t gr = cv.rbase + r;
         float xv[16];
         x_chunk16<TX>(cv.x, c * CHUNK + 4 * l32, xv);
@@ -375,7 +374,8 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
     const int64_t work = w.format == FMT_NIBBLE ? p.nrows : p.nrows / w.R;
     const dim3 grid(grid_for(work, ncols, cus), ncols);
     if (w.format == FMT_NIBBLE) {
-        const dim3 grid(grid_for(p.nrows * (w.K / CHUNK), ncols, cus), ncols);
+        const int rpb = HALVES / (int) (w.K / CHUNK);
+        const dim3 grid(grid_for((p.nrows + rpb - 1) / rpb * HALVES, ncols, cus), ncols);
 #define NIB(TX, G) hipLaunchKernelGGL((k_nib_mmv<TX, G>), grid, dim3(NT), 0, stream, w, wu, p)
         if (x_bf16) { if (glu == 0) NIB(bf16_t, 0); else if (glu == 1) NIB(bf16_t, 1); else NIB(bf16_t, 2); }
         else        { if (glu == 0) NIB(float, 0);  else if (glu == 1) NIB(float, 1);  else NIB(float, 2); }

@@ -321,3 +321,18 @@ def test_embedding_is_the_exact_rows(ops):
         out = ops.embedding(ids, w)
         assert tuple(out.shape) == (2, 3, K) and out.dtype == torch.bfloat16
         assert np.array_equal(bits(out).reshape(6, K), wb[ids.cpu().numpy().reshape(-1)])
+
+
+@pytest.mark.parametrize("K", [512, 1024, 1536, 2048, 2560, 3072, 3584, 4096])
+def test_nibble_every_chunk_count(ops, oracle, K):
+    # one half-wave per (row, chunk): every K / 512 from 1 to 8, row counts that do not fill a block, plain and GLU
+    rows = 2 * 13
+    wb = synth.weights(rows, K, 95 + K)
+    w = enc(ops, wb, NIB)
+    xb = synth.activations(2, K, 96)
+    xf = synth.bf16_bits_to_f32(xb)
+    check_gemv(oracle, ops.mmv(tbf16(xb), w).cpu().numpy(), wb, xf)
+    fused = ops.mmv_glu(tbf16(xb), w)
+    g = ops.mmv(tbf16(xb), enc(ops, wb[: rows // 2], NIB))
+    u = ops.mmv(tbf16(xb), enc(ops, wb[rows // 2:], NIB))
+    assert torch.equal(fused, ops.swiglu(g, u))

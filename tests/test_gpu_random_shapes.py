@@ -1,0 +1,64 @@
+"""Seeded sweep over shapes, unit sizes, layouts, batch sizes and expert routing: every case decodes bit-exactly and its
+products stay within the FP64 bound of the exact weights (|err| <= 1e-5 * sum|w x|) and within 1e-3 relative of them.
+The cases are drawn once from a fixed seed, so a failure names a reproducible configuration."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from orin_qwen_lossless_amd import synth
+from test_gpu_kernels import tbf16
+from test_gpu_roundtrip import bits, enc
+
+pytestmark = pytest.mark.gpu
+NIB, HUF, HP = 1, 2, 3
+
+
+def cases(n: int):
+    rng = np.random.default_rng(20240607)
+    out = []
+    while len(out) < n:
+        K = int(rng.choice([512, 1024, 1536, 2048, 2560, 4096]))
+        fmt = int(rng.choice([NIB, HUF, HP, HP, HP]))
+        R = 0 if fmt == NIB else int(rng.choice([1, 2, 4, 8, 16]))
+        cm = bool(fmt == HP and K > 512 and R >= 4 and rng.random() < 0.3)
+        C = K // 512
+        w64 = bool(fmt == HP and not cm and C in (1, 2, 4, 8) and (R * C // 2) % (4 if C == 8 else 2) == 0 and (R * C) % 2 == 0
+                   and rng.random() < 0.6)
+        units = int(rng.integers(1, 40))
+        E = int(rng.choice([1, 1, 3, 5]))
+        rows_per = units * max(R, 1)
+        T = int(rng.integers(1, 9))
+        out.append((K, fmt, R, cm, w64, rows_per, E, T, int(rng.integers(1 << 30))))
+    return out
+
+
+@pytest.mark.parametrize("K,fmt,R,cm,w64,rows_per,E,T,seed", cases(48))
+def test_random_configuration(ops, K, fmt, R, cm, w64, rows_per, E, T, seed):
+    rows = rows_per * E
+    wb = synth.model_like(rows, K, seed) if seed % 3 == 0 else synth.weights(rows, K, seed)
+    w = enc(ops, wb, fmt, R, cm, w64)
+    assert np.array_equal(bits(ops.dequant(w)), wb)
+    xb = synth.activations(T, K, seed + 1)
+    xf = synth.bf16_bits_to_f32(xb).astype(np.float64)
+    wf = synth.bf16_bits_to_f32(wb).astype(np.float64)
+    finite_rows = np.isfinite(wf).all(axis=1) & (np.abs(wf).max(axis=1) < 1e30)
+    if E == 1:
+        y = ops.mmv(tbf16(xb), w).cpu().numpy().astype(np.float64)
+        with np.errstate(invalid="ignore", over="ignore"):
+            ref, bound = xf @ wf.T, np.abs(xf) @ np.abs(wf).T
+        ok = finite_rows[None, :]
+    else:
+        k = min(2, E)
+        rng = np.random.default_rng(seed)
+        ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+        y = ops.mmv(tbf16(xb), w, torch.from_numpy(ids).cuda(), rows_per).cpu().numpy().astype(np.float64)
+        we = wf.reshape(E, rows_per, K)[ids]                      # [T, k, rows_per, K]
+        ref = np.einsum("tkrc,tc->tkr", we, xf)
+        bound = np.einsum("tkrc,tc->tkr", np.abs(we), np.abs(xf))
+        ok = finite_rows.reshape(E, rows_per)[ids]
+    with np.errstate(invalid="ignore", over="ignore"):
+        err = np.abs(y - ref)
+    assert np.all(err[np.broadcast_to(ok, err.shape)] <= (1e-5 * bound + 1e-30)[np.broadcast_to(ok, err.shape)])
+    assert np.all(err[np.broadcast_to(ok, err.shape)] <= (1e-3 * np.abs(ref) + 1e-5)[np.broadcast_to(ok, err.shape)])
