@@ -34,12 +34,27 @@ def cases(n: int):
     return out
 
 
-@pytest.mark.parametrize("K,fmt,R,cm,w64,rows_per,E,T,seed", cases(48))
+@pytest.mark.parametrize("K,fmt,R,cm,w64,rows_per,E,T,seed", cases(120))
 def test_random_configuration(ops, K, fmt, R, cm, w64, rows_per, E, T, seed):
     rows = rows_per * E
     wb = synth.model_like(rows, K, seed) if seed % 3 == 0 else synth.weights(rows, K, seed)
     w = enc(ops, wb, fmt, R, cm, w64)
     assert np.array_equal(bits(ops.dequant(w)), wb)
+    rng = np.random.default_rng(seed + 7)
+    # a row range of whole units decodes to the same bits as the slice
+    unit = max(R, 1)
+    u0 = int(rng.integers(0, rows // unit))
+    un = int(rng.integers(1, rows // unit - u0 + 1))
+    assert np.array_equal(bits(ops.dequant(w, u0 * unit, un * unit)), wb[u0 * unit: (u0 + un) * unit])
+    if fmt == NIB or (fmt == HP and not cm):
+        # row gather with a base row that is not unit-aligned; BF16 and FP32 outputs are the exact weights
+        row0 = int(rng.integers(0, rows))
+        idn = rng.integers(0, rows - row0, size=5)
+        for idt in (torch.int32, torch.int64):
+            ids = torch.from_numpy(idn).to(idt).cuda()
+            assert np.array_equal(bits(ops.get_rows(ids, w, torch.bfloat16, row0)), wb[row0 + idn])
+        got32 = ops.get_rows(torch.from_numpy(idn).to(torch.int32).cuda(), w, torch.float32, row0).cpu().numpy()
+        assert np.array_equal(got32.view(np.uint32), synth.bf16_bits_to_f32(wb[row0 + idn]).view(np.uint32))
     xb = synth.activations(T, K, seed + 1)
     xf = synth.bf16_bits_to_f32(xb).astype(np.float64)
     wf = synth.bf16_bits_to_f32(wb).astype(np.float64)
