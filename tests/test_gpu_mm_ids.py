@@ -163,3 +163,44 @@ def test_moe_experts_switches_to_batched_kernels(ops, T, cm, w64):
     ref = ops.moe_experts_reference(x, gate, up, down, wts, ids, E).float().cpu().numpy()
     scale = np.abs(ref).max()
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
+
+
+def sweep_cases(n: int):
+    rng = np.random.default_rng(4242)
+    layouts = [(2048, 8, True, False), (2048, 8, False, True), (2048, 4, False, True), (2048, 2, False, True),
+               (512, 16, False, False), (512, 16, False, True), (512, 8, False, True), (512, 4, False, True)]
+    out = []
+    for i in range(n):
+        K, R, cm, w64 = layouts[i % len(layouts)]
+        E = int(rng.integers(2, 10))
+        N = 64 * int(rng.integers(1, 4))
+        k = int(rng.integers(1, min(E, 4) + 1))
+        T = int(rng.integers(9, 300))
+        out.append((K, R, cm, w64, E, N, k, T, bool(rng.integers(2)), int(rng.integers(1 << 30))))
+    return out
+
+
+@pytest.mark.parametrize("K,R,cm,w64,E,N,k,T,fused,seed", sweep_cases(24))
+def test_mm_ids_seeded_sweep(ops, K, R, cm, w64, E, N, k, T, fused, seed):
+    rng = np.random.default_rng(seed)
+    wb = synth.weights(E * N, K, seed)
+    w = enc(ops, wb, HP, R, cm, w64)
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    per_slot = K == 512
+    xb = synth.activations(T * (k if per_slot else 1), K, seed + 1).reshape((T, k, K) if per_slot else (T, K))
+    xf = synth.bf16_bits_to_f32(xb)
+    it = torch.from_numpy(ids).cuda()
+    y, s = reference(synth.bf16_bits_to_f32(wb), xf, ids, N, per_slot)
+    got = ops.moe_mm_ids(tbf16(xb), it, w, E).cpu().numpy()
+    assert np.all(np.abs(got - y) <= 1e-5 * s + 1e-30)
+    if fused and K == 2048:
+        ub = synth.weights(E * N, K, seed + 2)
+        u = enc(ops, ub, HP, R, cm, w64)
+        yu, _ = reference(synth.bf16_bits_to_f32(ub), xf, ids, N, False)
+        ref = yu * (y / (1.0 + np.exp(-y)))
+        f = ops.moe_mm_ids(tbf16(xb), it, w, E, up=u).cpu().numpy()
+        assert np.all(np.abs(f - ref) <= 1e-3 * np.abs(ref) + 1e-5)
+        # the decode-side fused kernel agrees with the batched one on the first tokens (different summation orders)
+        if ops.glu2_supported(w, u):
+            g8 = ops.mmv_glu2(tbf16(xb[:8]), w, u, it[:8].contiguous(), N).cpu().numpy()
+            assert np.all(np.abs(g8 - f[:8]) <= 1e-3 * np.abs(ref[:8]) + 1e-5)
