@@ -28,6 +28,11 @@ constexpr uint32_t FLAG_FRAG_ORDER  = 2; // reference only (NVIDIA mma fragment 
 // The plane is unchanged.  Lanes 0..31 own the even, lanes 32..63 the odd 512-column chunks of the unit in stream
 // order (so R * K / 512 must be even); see encode_w64() in csrc/encode.cpp for the stream definition.
 constexpr uint32_t FLAG_WAVE64      = 4;
+// FLAG_WAVE64 with R = 32: the units are tiles of TILE_R rows x TILE_K columns in the operand order of the 32x32x16
+// matrix instruction (lane l: row l % 32, two runs of 8 consecutive columns per step); unit g * (K / 256) + t is the
+// tile of row group g and column slab t.  Each tile is stored as a wave64 unit of 16 rows of 512 columns; the element
+// mapping is tile32_index() in csrc/encode.cpp.
+constexpr int TILE_R = 32, TILE_K = 256;
 
 // First bytes of every aux buffer (the header occupies HEADER_BYTES); offsets are bytes from the aux start.
 //   NIBBLE : off_a codes (rows*K/2), off_b row tables (rows*16), off_c u32 esc_off[rows+1], off_d u32 escapes; n_a escapes

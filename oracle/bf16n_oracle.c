@@ -448,11 +448,7 @@ int orc_decode(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, uin
  * (lanes in ascending order) as its new w2, moves w2 to w1 and w1 to w0 and subtracts 32.  The unit stream is: the
  * lanes' first three words (lane 0 words 0, 1, 2, lane 1 words 0, 1, 2, ...), then the refill words in the order taken.
  * off_b: u32 unit_base[units + 1] (word index of each unit's stream), off_d: words. */
-int orc_decode_w64(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, uint16_t *out) {
-    orc_header h;
-    if (aux_bytes < 256) return -1;
-    memcpy(&h, aux, sizeof h);
-    if (h.magic != MAGIC || h.format != ORC_FMT_HUFPAIR || !(h.flags & ORC_FLAG_WAVE64) || h.R == 0) return -1;
+static int decode_w64_units(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, orc_header h, uint16_t *out) {
     const int64_t K = h.K, C = K / CHUNK, R = h.R;
     const int cm = (h.flags & ORC_FLAG_CHUNK_MAJOR) != 0;
     if ((R * C) % 2) return -1;
@@ -491,6 +487,38 @@ int orc_decode_w64(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes,
         if (next != h.off_d + 4ull * rd32(aux, h.off_b + 4 * (u + 1))) return -1; /* stream length must match exactly */
     }
     return 0;
+}
+
+/* R = 32 (only with flag bit 2): tiles in matrix-core operand order.  Unit u = g * (K / 256) + t holds rows
+ * [32 g, 32 g + 32) x columns [256 t, 256 t + 256); it is stored exactly as a wave64 unit of 16 rows of a 512-column
+ * matrix V (plane and stream), where V[16 u + 2 s + h][128 j + 4 l + q] = W[32 g + l][256 t + 32 s + 16 (j / 2) + 8 h
+ * + 4 (j % 2) + q] for s < 8, h < 2, j < 4, l < 32, q < 4: in step s lane 32 h + l holds, in slot order, columns
+ * 32 s + 8 h + [0, 8) and 32 s + 16 + 8 h + [0, 8) of row l of the tile. */
+int64_t orc_tile32_index(int64_t vrow, int64_t vcol, int64_t K) {
+    const int64_t u = vrow / 16, sh = vrow % 16, s = sh / 2, hh = sh % 2;
+    const int64_t j = vcol / 128, l = (vcol % 128) / 4, q = vcol % 4;
+    const int64_t slabs = K / 256, g = u / slabs, t = u % slabs;
+    return (32 * g + l) * K + 256 * t + 32 * s + 16 * (j / 2) + 8 * hh + 4 * (j % 2) + q;
+}
+
+int orc_decode_w64(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, uint16_t *out) {
+    orc_header h;
+    if (aux_bytes < 256) return -1;
+    memcpy(&h, aux, sizeof h);
+    if (h.magic != MAGIC || h.format != ORC_FMT_HUFPAIR || !(h.flags & ORC_FLAG_WAVE64) || h.R == 0) return -1;
+    if (h.R != 32) return decode_w64_units(plane, aux, aux_bytes, h, out);
+    if ((h.flags & ORC_FLAG_CHUNK_MAJOR) || h.rows % 32 || h.K % 256) return -1;
+    const int64_t K = h.K, n = (int64_t) h.rows * K, vrows = n / CHUNK;
+    orc_header v = h;
+    v.K = CHUNK; v.R = 16; v.rows = (uint64_t) vrows;
+    uint16_t *tmp = (uint16_t *) malloc((size_t) n * 2);
+    if (!tmp) return -1;
+    int rc = decode_w64_units(plane, aux, aux_bytes, v, tmp);
+    if (rc == 0)
+        for (int64_t r = 0; r < vrows; r++)
+            for (int64_t c = 0; c < CHUNK; c++) out[orc_tile32_index(r, c, K)] = tmp[r * CHUNK + c];
+    free(tmp);
+    return rc;
 }
 
 /* ---------------------------------------------------------------- GEMV references */

@@ -67,6 +67,9 @@ int orc_decode(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, uin
  * semantics, 64 lanes per unit, one interleaved word stream per unit.  No reference counterpart: pinned only by
  * decode(encode(w)) == w and by comparing with orc_decode of the reference layout of the same tensor. */
 int orc_decode_w64(const uint8_t *plane, const uint8_t *aux, uint64_t aux_bytes, uint16_t *out);
+/* R = 32 tiles of the wave64 layout: index into the row-major rows x K matrix of element (vrow, vcol) of the 512-column
+ * matrix the tile units are stored as. */
+int64_t orc_tile32_index(int64_t vrow, int64_t vcol, int64_t K);
 
 /* y[r] = sum_k W[r,k] x[k] with FP32 fmaf in the summation order of the reference GEMV kernels:
  * lane accumulators a0..a3 over (chunk, j), (a0+a1)+(a2+a3), then a 32-lane xor butterfly

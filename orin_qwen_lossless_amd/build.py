@@ -16,7 +16,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libbf16n_hip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip"]
+SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall", "-Wno-unused-function"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

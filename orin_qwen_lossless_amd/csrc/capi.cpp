@@ -48,6 +48,7 @@ void ensure_init() {
         hip_check(hipDeviceGetAttribute(&g_lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev), "hipDeviceGetAttribute");
         dev::w64_init();
         dev::mm_ids_init();
+        dev::tile_init();
     });
 }
 
@@ -75,6 +76,7 @@ void check_weight(const bf16n_weight & w) {
     require(!(w.flags & FLAG_WAVE64) || (w.format == FMT_HUFPAIR && !(w.flags & FLAG_CHUNK_MAJOR)),
             "the wave64 layout exists only for row-major HUFPAIR");
     require(!(w.flags & ~(FLAG_CHUNK_MAJOR | FLAG_FRAG_ORDER | FLAG_WAVE64)), "unknown layout flags");
+    require(w.format == FMT_NIBBLE || w.R <= 16 || dev::is_tile_layout(w), "R = 32 exists only as wave64 HUFPAIR tiles");
 }
 
 bool is_w64(const bf16n_weight & w) { return (w.flags & FLAG_WAVE64) != 0; }
@@ -173,7 +175,9 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
             return;
         }
         const dev::cols p = make_cols(*a);
-        if (is_w64(*w)) {
+        if (dev::is_tile_layout(*w)) {
+            dev::launch_tile_mmv(*w, nullptr, p, a->ncols, a->x_bf16 != 0, (hipStream_t) stream);
+        } else if (is_w64(*w)) {
             require(dev::w64_mmv_supported(*w, a->x_bf16 != 0), "no wave64 GEMV kernel for this K / R (K in {512, 1024, 2048, 4096})");
             dev::launch_w64_mmv(*w, p, a->ncols, a->x_bf16 != 0, multi_col != 0, g_cus, (hipStream_t) stream);
         } else {
@@ -213,14 +217,17 @@ int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf1
                 "mmv_glu: chunk-major weights require separate mmv launches");
         require(is_w64(*gate) == is_w64(*up), "mmv_glu: gate/up layouts must match");
         require(gate->format == FMT_NIBBLE || gate->R == up->R, "mmv_glu: gate/up R must match");
-        require(!is_w64(*gate) || dev::w64_mmv_supported(*gate, a->x_bf16 != 0), "mmv_glu: no fused kernel for this wave64 shape");
+        require(!is_w64(*gate) || dev::is_tile_layout(*gate) || dev::w64_mmv_supported(*gate, a->x_bf16 != 0),
+                "mmv_glu: no fused kernel for this wave64 shape");
         require(a->ncols > 0 && a->ncols <= 65535, "ncols out of range");
         require(gate->format == FMT_NIBBLE || (a->nrows % gate->R == 0 && a->row0 % gate->R == 0 && a->rows_per_matrix % gate->R == 0),
                 "rows of a product must be whole units");
         if (a->nrows == 0) {
             return;
         }
-        if (is_w64(*gate)) {
+        if (dev::is_tile_layout(*gate)) {
+            dev::launch_tile_mmv(*gate, up, make_cols(*a), a->ncols, a->x_bf16 != 0, (hipStream_t) stream);
+        } else if (is_w64(*gate)) {
             dev::launch_w64_glu(*gate, *up, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
         } else {
             dev::launch_compat_mmv(*gate, up, 2, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
@@ -241,7 +248,9 @@ int bf16n_dequant(const bf16n_weight * w, int64_t row0, int64_t nrows, uint16_t 
         if (w->format != FMT_NIBBLE) {
             require(nrows % w->R == 0 && row0 % w->R == 0, "dequant rows must be whole units");
         }
-        if (is_w64(*w)) {
+        if (dev::is_tile_layout(*w)) {
+            dev::launch_tile_dequant(*w, row0, nrows, out, (hipStream_t) stream);
+        } else if (is_w64(*w)) {
             dev::launch_w64_dequant(*w, row0, nrows, out, g_cus, (hipStream_t) stream);
         } else {
             dev::launch_compat_dequant(*w, row0, nrows, out, g_cus, (hipStream_t) stream);
@@ -263,7 +272,9 @@ int bf16n_get_rows(const bf16n_weight * w, const void * ids, int64_t ids_s0, int
         if (n == 0) {
             return;
         }
-        if (is_w64(*w)) {
+        if (dev::is_tile_layout(*w)) {
+            dev::launch_tile_get_rows(*w, ids, ids_s0, n, dst, dst_bf16 != 0, dst_s1, row0, (hipStream_t) stream);
+        } else if (is_w64(*w)) {
             dev::launch_w64_get_rows(*w, ids, ids_s0, n, dst, dst_bf16 != 0, dst_s1, row0, (hipStream_t) stream);
         } else {
             dev::launch_compat_get_rows(*w, ids, ids_s0, n, dst, dst_bf16 != 0, dst_s1, row0, (hipStream_t) stream);
@@ -303,8 +314,13 @@ int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x
         require(x_bf16 && dst && ids_src1 && ids_dst && bounds, "null pointer");
         require(((uintptr_t) x_bf16 & 15) == 0 && x_row % 8 == 0, "activations must be 16-byte aligned with 16-byte row strides");
         require(((uintptr_t) dst & 15) == 0 && dst_col % 4 == 0, "dst must be 16-byte aligned with a column stride that is a multiple of 4");
-        dev::launch_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, n_tok, n_used,
-                           g_cus, (hipStream_t) stream);
+        if (dev::is_tile_layout(*w)) {
+            dev::launch_tile_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, g_cus,
+                                    (hipStream_t) stream);
+        } else {
+            dev::launch_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, n_tok, n_used,
+                               g_cus, (hipStream_t) stream);
+        }
         launch_check("mm_ids");
     });
 }

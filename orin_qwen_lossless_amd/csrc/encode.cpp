@@ -673,6 +673,47 @@ std::vector<uint8_t> encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_
     return aux;
 }
 
+// ---------------------------------------------------------------------------------------------- HUFPAIR, wave64 tiles
+//
+// R = 32 with the wave64 layout: units are tiles of 32 rows x 256 columns in the operand order of the 32x32x16 matrix
+// instruction, so that a wavefront decodes straight into A operands (lane l holds row l % 32; its 16 weights of a
+// step are two runs of 8 consecutive columns, 8 (l / 32) into each 16-column block of the step's 32 columns).
+// Unit u = g * (K / 256) + t is the tile of rows [32 g, 32 g + 32), columns [256 t, 256 t + 256): the tiles of a row
+// group are consecutive units, a wavefront can decode them as one run.  A tile is stored exactly as a wave64 unit
+// of 16 rows of the 512-column matrix V (same plane and stream rules), with
+//   V[16 u + 2 s + h][128 j + 4 l + q] = W[32 g + l][256 t + 32 s + 16 (j / 2) + 8 h + 4 (j % 2) + q]
+// for step s < 8, half-wave h < 2, j < 4, l < 32, q < 4.  The header keeps the matrix's own K and rows, R = 32.
+int64_t tile32_index(int64_t vrow, int64_t vcol, int64_t K) {
+    const int64_t u = vrow / 16, s = (vrow % 16) / 2, h = vrow % 2;
+    const int64_t j = vcol / 128, l = (vcol % 128) / 4, q = vcol % 4;
+    const int64_t slabs = K / TILE_K, g = u / slabs, t = u % slabs;
+    return (TILE_R * g + l) * K + TILE_K * t + 32 * s + 16 * (j / 2) + 8 * h + 4 * (j % 2) + q;
+}
+
+bool encode_tile32(const uint16_t * w, int64_t rows, int64_t K, encoded_buffers & out) {
+    const int64_t vrows = rows * K / CHUNK;
+    std::vector<uint16_t> v((size_t) (rows * K));
+    parallel_blocks(vrows, 64, [&](int64_t r0, int64_t r1) {
+        for (int64_t r = r0; r < r1; r++) {
+            for (int64_t c = 0; c < CHUNK; c++) {
+                v[(size_t) (r * CHUNK + c)] = w[tile32_index(r, c, K)];
+            }
+        }
+    });
+    out.aux = encode_hufpair_w64(v.data(), vrows, CHUNK, 16, false);
+    if (out.aux.empty()) {
+        return false;
+    }
+    aux_header h;
+    std::memcpy(&h, out.aux.data(), sizeof(h));
+    h.K = (uint32_t) K; h.R = TILE_R; h.rows = (uint64_t) rows;
+    std::memcpy(out.aux.data(), &h, sizeof(h));
+    write_plane(v.data(), vrows, CHUNK, 16, false, out.plane.data());
+    out.format = FMT_HUFPAIR;
+    out.R = TILE_R;
+    return true;
+}
+
 // ---------------------------------------------------------------------------------------------- entry point
 
 // argument contract of the reference (encode.cpp:443-474) plus the wave64 layout of this build
@@ -693,8 +734,9 @@ encoded_buffers encode(const uint16_t * w, int64_t rows, int64_t K, int format, 
             bad("NIBBLE takes R = 0 and no chunk-major or fragment-order layout");
         }
     } else if (format == FMT_HUFFMAN || format == FMT_HUFPAIR) {
-        if (R != 1 && R != 2 && R != 4 && R != 8 && R != 16) {
-            bad("R must be one of 1, 2, 4, 8, 16, got " + std::to_string(R));
+        const bool tiles = R == TILE_R && w64 && format == FMT_HUFPAIR; // matrix-core tiles, see encode_tile32()
+        if (R != 1 && R != 2 && R != 4 && R != 8 && R != 16 && !tiles) {
+            bad("R must be one of 1, 2, 4, 8, 16 (or 32 for wave64 HUFPAIR tiles), got " + std::to_string(R));
         }
         if (rows % R != 0) {
             bad("rows (" + std::to_string(rows) + ") must be a multiple of R (" + std::to_string(R) + ")");
@@ -730,7 +772,13 @@ encoded_buffers encode(const uint16_t * w, int64_t rows, int64_t K, int format, 
         out.format = FMT_NIBBLE;
         return out;
     }
-    if (format == FMT_HUFPAIR) {
+    if (format == FMT_HUFPAIR && R == TILE_R) {
+        if (encode_tile32(w, rows, K, out)) {
+            return out;
+        }
+        R = 16; // more than 4096 distinct pairs: single-symbol fallback below, which has no special layouts
+        out.R = R;
+    } else if (format == FMT_HUFPAIR) {
         out.aux = w64 ? encode_hufpair_w64(w, rows, K, R, cm) : encode_hufpair(w, rows, K, R, cm);
     }
     if (!out.aux.empty()) {

@@ -1,0 +1,510 @@
+// Kernels for the tile form of the wave64 layout (FLAG_WAVE64 with R = 32; include/bf16n/format.h): units are 32-row x
+// 256-column tiles whose decode order is the A-operand order of v_mfma_f32_32x32x16_bf16.  In step s (of 8) of a tile,
+// lane 32 h + l holds, in slot order, columns 32 s + 8 h + [0, 8) and 32 s + 16 + 8 h + [0, 8) of row l: the eight
+// BF16 pairs that the decoder produces are, as they stand, the A operands of two matrix instructions.  The tiles of a
+// row group are consecutive units, so a wavefront decodes them as one run of its stream.
+//
+//   * k_mm_tile: batched MoE prefill (reference mm_ids / k_hp_mm_ids, core/src/launch.cu:473-535,
+//     core/src/kernels.cuh:1162-1505).  Weights go from the decoder's registers into the matrix cores; the activations
+//     of up to 128 tokens are staged in LDS, 128 columns at a time, and shared by the eight wavefronts of a block.
+//   * k_tile_mmv: GEMV / fused gate-up GEMV at decode (reference mmv / mmv_glu, launch.cu:313-365): a lane accumulates
+//     one row over the whole tile, so a tile ends with one cross-half add instead of a reduction per row.
+//   * k_tile_dequant, k_tile_get_rows: exact BF16 rows (launch.cu:367-443).
+#include "dev_common.h"
+#include "dev_w64.h"
+#include "launchers.h"
+
+#include <stdexcept>
+
+namespace bf16n {
+namespace dev {
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int T_STEPS = 8;                      // steps per tile
+constexpr int T_BYTES = TILE_R * TILE_K;        // plane bytes per tile
+constexpr int STEP_BYTES = 1024;
+
+// column (inside the tile) of the first of the four weights that plane word j of a lane holds in step s
+__device__ __forceinline__ int tile_col(int s, int j, int half) { return 32 * s + 16 * (j >> 1) + 8 * half + 4 * (j & 1); }
+
+// One decode chain: the tiles [first unit, first unit + n) of one matrix, with the plane bytes of the next four steps
+// in registers (reloaded as soon as a step is consumed).
+struct tchain {
+    w64_dec dec;
+    const uint8_t * plane;
+    uint32_t off, last;
+    uint4 sm[4];
+    __device__ __forceinline__ uint4 load_step(int lane) const {
+        const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
+        return *((const uint4 *) (plane + o) + lane);
+    }
+    __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane) {
+        plane = q.plane + uniform64(unit0 * T_BYTES);
+        off = 0;
+        last = (uint32_t) (n_units * T_BYTES - STEP_BYTES);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            sm[s] = load_step(lane);
+            off += STEP_BYTES;
+        }
+        dec.start(ring, q.stream, uniform(q.ubase[unit0]), uniform(q.ubase[unit0 + n_units]), lane);
+    }
+    __device__ __forceinline__ void reload(int s, int lane) {
+        sm[s] = load_step(lane);
+        off += STEP_BYTES;
+    }
+    __device__ __forceinline__ void begin_tile() {
+        dec.keep_ahead();
+        dec.begin_unit();
+        dec.keep_ahead();
+    }
+};
+
+// one step of N chains, instruction streams interleaved; lut of chain k at lut + k * lut_stride
+template <int N>
+__device__ __forceinline__ void tile_step(tchain * ch, const uint32_t * lut, int lut_stride, int s, uint32_t (&wp)[N][8]) {
+    uint32_t smw[N][4];
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        smw[k][0] = ch[k].sm[s].x; smw[k][1] = ch[k].sm[s].y; smw[k][2] = ch[k].sm[s].z; smw[k][3] = ch[k].sm[s].w;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int k = 0; k < N; k++) {
+            uint32_t e0, e1;
+            ch[k].dec.two(lut + k * lut_stride, e0, e1);
+            wp[k][2 * j] = merge(spread_lo(smw[k][j]), e0);
+            wp[k][2 * j + 1] = merge(spread_hi(smw[k][j]), e1);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        ch[k].dec.keep_ahead();
+    }
+}
+
+// ---------------------------------------------------------------- batched MoE prefill
+
+constexpr int MT_WAVES = 8, MT_THREADS = MT_WAVES * 64;
+constexpr int MT_TOK = 128;        // tokens per pass: four 32-token blocks per wavefront
+constexpr int MT_HK = 128;         // activation columns staged at a time (half a tile)
+constexpr int MT_BSTRIDE = 136;    // BF16 elements per staged token row: 272 bytes spread 16 lanes over all banks
+
+struct mm_args {
+    const uint16_t * x; int64_t x_row;
+    const int32_t * ids_src1, * ids_dst, * bounds;
+    char * dst; int64_t dst_col; bool dst_bf16;
+    int64_t rows; // per expert
+    int n_experts;
+};
+
+// A work item is (expert, slab of row groups): every wavefront owns two decode chains — gate and up of one row group
+// (GLU), or two row groups of the matrix — and keeps their 2 x 4 accumulator blocks (32 rows x 32 tokens each) for
+// the whole pass over the expert's K columns.  Per step a chain yields two A operands (32 rows x 16 columns); the B
+// operands (16 columns x 32 tokens) come from the staged activations and are used by both chains.
+template <bool GLU>
+__global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+    constexpr int NM = GLU ? 2 : 1;
+    extern __shared__ __align__(16) uint32_t shm[];
+    uint32_t * lut = shm;
+    uint32_t * rings = shm + NM * LUT_WORDS;
+    uint16_t * bbuf = (uint16_t *) (rings + MT_WAVES * 2 * WAVE_LDS_WORDS); // two buffers of MT_TOK x MT_BSTRIDE
+    const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
+    stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
+    if (GLU) {
+        stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
+    }
+    const int slabs = (int) (w.K / TILE_K), halves = 2 * slabs;
+    const int groups = (int) (a.rows / TILE_R);               // row groups per expert
+    constexpr int GPI = GLU ? MT_WAVES : 2 * MT_WAVES;        // row groups per work item
+    const int slabs_per_expert = (groups + GPI - 1) / GPI;
+    const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
+    const int b_tok = tid >> 2, b_part = tid & 3;             // this thread's share of a staged block: 32 columns of one token
+    __syncthreads();
+    for (int item = blockIdx.x; item < a.n_experts * slabs_per_expert; item += gridDim.x) {
+        const int e = item / slabs_per_expert, sl = item % slabs_per_expert;
+        const int j0 = a.bounds[e], n = a.bounds[e + 1] - j0;
+        // this wavefront's row groups (inside the expert); a missing second group repeats the first and is dropped
+        const int g0 = GLU ? sl * GPI + wave : sl * GPI + 2 * wave;
+        const bool live = g0 < groups, has1 = GLU || g0 + 1 < groups;
+        const int g1 = GLU ? g0 : (has1 ? g0 + 1 : g0);
+        for (int tp = 0; tp < n; tp += MT_TOK) {
+            const int left = n - tp, nt = left >= MT_TOK ? 4 : (left + 31) >> 5;
+            const int btk = tp + b_tok;
+            const uint16_t * xsrc = a.x + (int64_t) a.ids_src1[j0 + (btk < n ? btk : 0)] * a.x_row + 32 * b_part;
+            uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + 32 * b_part;
+            uint4 breg[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                breg[i] = *((const uint4 *) xsrc + i);
+            }
+            tchain ch[2];
+            if (live) {
+                uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
+                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * slabs, slabs, lane);
+                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * slabs, slabs, lane);
+            }
+            f32x16_t acc[2][4];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        acc[c][t][i] = 0.f;
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                *((uint4 *) bdst + i) = breg[i];
+            }
+            __syncthreads();
+#pragma unroll 1
+            for (int hs = 0; hs < halves; hs++) {
+                const uint16_t * bcur = bbuf + (hs & 1) * (MT_TOK * MT_BSTRIDE);
+                if (hs + 1 < halves) { // the next block of activations: requested now, staged after this block's steps
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        breg[i] = *((const uint4 *) (xsrc + (hs + 1) * MT_HK) + i);
+                    }
+                }
+                if (live) {
+                    if ((hs & 1) == 0) {
+                        ch[0].begin_tile();
+                        ch[1].begin_tile();
+                    }
+#pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        uint32_t wp[2][8];
+                        tile_step<2>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
+                        ch[0].reload(s, lane);
+                        ch[1].reload(s, lane);
+                        const uint16_t * bp = bcur + l32 * MT_BSTRIDE + 32 * s + 8 * half;
+#pragma unroll
+                        for (int kb = 0; kb < 2; kb++) {
+                            const u32x4_t a0 = {wp[0][4 * kb], wp[0][4 * kb + 1], wp[0][4 * kb + 2], wp[0][4 * kb + 3]};
+                            const u32x4_t a1 = {wp[1][4 * kb], wp[1][4 * kb + 1], wp[1][4 * kb + 2], wp[1][4 * kb + 3]};
+                            const bf16x8_t av0 = __builtin_bit_cast(bf16x8_t, a0), av1 = __builtin_bit_cast(bf16x8_t, a1);
+#pragma unroll
+                            for (int t = 0; t < 4; t++) {
+                                if (t < nt) {
+                                    const bf16x8_t bv = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE + 16 * kb);
+                                    acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av0, bv, acc[0][t], 0, 0, 0);
+                                    acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av1, bv, acc[1][t], 0, 0, 0);
+                                }
+                            }
+                        }
+                    }
+                }
+                if (hs + 1 < halves) {
+                    uint16_t * bn = bdst + ((hs + 1) & 1) * (MT_TOK * MT_BSTRIDE);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        *((uint4 *) bn + i) = breg[i];
+                    }
+                }
+                __syncthreads();
+            }
+            // accumulator element i of a lane: row 8 (i / 4) + 4 (lane / 32) + i % 4 of the group, token lane % 32
+            if (live) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const int tk = tp + 32 * t + l32;
+                    if (t < nt && tk < n) {
+                        const int64_t col = (int64_t) a.ids_dst[j0 + tk] * a.dst_col;
+#pragma unroll
+                        for (int c = 0; c < (GLU ? 1 : 2); c++) {
+                            if (c == 1 && !has1) {
+                                continue;
+                            }
+                            const int64_t row0 = (int64_t) (c ? g1 : g0) * TILE_R + 4 * half;
+#pragma unroll
+                            for (int g = 0; g < 4; g++) {
+                                float v[4];
+#pragma unroll
+                                for (int i = 0; i < 4; i++) {
+                                    const float p = acc[c][t][4 * g + i];
+                                    v[i] = GLU ? acc[1][t][4 * g + i] * silu(p) : p;
+                                }
+                                const int64_t o = col + row0 + 8 * g;
+                                if (a.dst_bf16) {
+                                    *(uint2 *) ((uint16_t *) a.dst + o) =
+                                        make_uint2(f32_to_bf16_rne(v[0]) | ((uint32_t) f32_to_bf16_rne(v[1]) << 16),
+                                                   f32_to_bf16_rne(v[2]) | ((uint32_t) f32_to_bf16_rne(v[3]) << 16));
+                                } else {
+                                    *(float4 *) ((float *) a.dst + o) = make_float4(v[0], v[1], v[2], v[3]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+size_t mt_shm(bool glu) {
+    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) MT_WAVES * 2 * WAVE_LDS_WORDS * 4 + (size_t) 2 * MT_TOK * MT_BSTRIDE * 2;
+}
+
+// ---------------------------------------------------------------- GEMV
+
+// 8 consecutive activations as FP32
+template <typename TX> struct x8;
+template <> struct x8<bf16_t> {
+    uint4 r;
+    __device__ __forceinline__ void load(const char * x, int k) { r = *(const uint4 *) (x + 2 * (int64_t) k); }
+    __device__ __forceinline__ float dot(const uint32_t * wp, float acc) const {
+        const uint32_t xw[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            acc = fmaf(__uint_as_float(wp[i] << 16), __uint_as_float(xw[i] << 16), acc);
+            acc = fmaf(__uint_as_float(wp[i] & 0xFFFF0000u), __uint_as_float(xw[i] & 0xFFFF0000u), acc);
+        }
+        return acc;
+    }
+};
+template <> struct x8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const char * x, int k) {
+        a = *(const float4 *) (x + 4 * (int64_t) k);
+        b = *(const float4 *) (x + 4 * (int64_t) k + 16);
+    }
+    __device__ __forceinline__ float dot(const uint32_t * wp, float acc) const {
+        const float xv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            acc = fmaf(__uint_as_float(wp[i] << 16), xv[2 * i], acc);
+            acc = fmaf(__uint_as_float(wp[i] & 0xFFFF0000u), xv[2 * i + 1], acc);
+        }
+        return acc;
+    }
+};
+
+constexpr int TV_WAVES = 8;
+
+// A block covers `gpb` row groups of one column; the `wpg` wavefronts of a group take `upw` consecutive tiles each and
+// their partial sums (one per lane and row) are added in tile order.  GLU: every wavefront decodes its tiles of the
+// gate and the up matrix side by side and the block writes silu(gate x) * (up x).
+template <typename TX, bool GLU>
+__global__ void __launch_bounds__(TV_WAVES * 64) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw) {
+    constexpr int NM = GLU ? 2 : 1;
+    __shared__ __align__(16) uint32_t lut[NM * LUT_WORDS];
+    __shared__ float part[NM][TV_WAVES][32];
+    extern __shared__ __align__(16) uint32_t rings[];
+    const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
+    const int slabs = (int) (w.K / TILE_K), gpb = TV_WAVES / wpg;
+    const int gi = wave / wpg, wi = wave % wpg;
+    const col_view cv = col_setup(p, blockIdx.y);
+    const int64_t groups = p.nrows / TILE_R, g = (int64_t) blockIdx.x * gpb + gi;
+    const bool live = gi < gpb && g < groups;
+    stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
+    if (GLU) {
+        stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
+    }
+    const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
+    const int64_t unit0 = live ? (cv.rbase / TILE_R + g) * slabs + wi * upw : 0;
+    tchain ch[NM];
+    if (live) {
+        uint32_t * ring = rings + wave * (NM * WAVE_LDS_WORDS);
+        ch[0].start(ring, q0, unit0, upw, lane);
+        if (GLU) {
+            ch[NM - 1].start(ring + WAVE_LDS_WORDS, q1, unit0, upw, lane);
+        }
+    }
+    __syncthreads();
+    float acc[NM] = {};
+    if (live) {
+        for (int u = 0; u < upw; u++) {
+            const int k0 = (wi * upw + u) * TILE_K + 8 * half;
+#pragma unroll
+            for (int k = 0; k < NM; k++) {
+                ch[k].begin_tile();
+            }
+#pragma unroll 1
+            for (int hh = 0; hh < 2; hh++) { // two halves of four steps: the step index into the plane registers stays static
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    const int kk = k0 + 32 * (4 * hh + s);
+                    x8<TX> xa, xb;
+                    xa.load(cv.x, kk);
+                    xb.load(cv.x, kk + 16);
+                    uint32_t wp[NM][8];
+                    tile_step<NM>(ch, lut, LUT_WORDS, s, wp);
+#pragma unroll
+                    for (int k = 0; k < NM; k++) {
+                        ch[k].reload(s, lane);
+                        acc[k] = xb.dot(wp[k] + 4, xa.dot(wp[k], acc[k]));
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < NM; k++) {
+            const float v = acc[k] + __shfl_xor(acc[k], 32, 64);
+            if (half == 0) {
+                part[k][wave][l32] = v;
+            }
+        }
+    }
+    __syncthreads();
+    if (live && wi == 0 && half == 0) {
+        float s[NM];
+#pragma unroll
+        for (int k = 0; k < NM; k++) {
+            s[k] = part[k][wave][l32];
+            for (int i = 1; i < wpg; i++) {
+                s[k] += part[k][wave + i][l32];
+            }
+        }
+        store_y(cv.y, p.y_bf16, g * TILE_R + l32, GLU ? s[NM - 1] * silu(s[0]) : s[0]);
+    }
+}
+
+// ---------------------------------------------------------------- dequant / row gather
+
+// one step of a tile as exact BF16 (or FP32) values; only_l >= 0: just that row of the tile, to `out`
+__device__ __forceinline__ void tile_store_step(const uint32_t (&wp)[8], int s, int l32, int half, int only_l, char * out,
+                                                int64_t row_bytes, bool f32) {
+    if (only_l >= 0 && l32 != only_l) {
+        return;
+    }
+    char * dst = out + (only_l >= 0 ? 0 : l32) * row_bytes;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int col = tile_col(s, j, half);
+        if (f32) {
+            *(float4 *) (dst + 4 * col) = make_float4(__uint_as_float(wp[2 * j] << 16), __uint_as_float(wp[2 * j] & 0xFFFF0000u),
+                                                      __uint_as_float(wp[2 * j + 1] << 16), __uint_as_float(wp[2 * j + 1] & 0xFFFF0000u));
+        } else {
+            *(uint2 *) (dst + 2 * col) = make_uint2(wp[2 * j], wp[2 * j + 1]);
+        }
+    }
+}
+
+// decode the `n` tiles from unit0 on (one row group: consecutive column slabs from slab t0) and store them
+__device__ __forceinline__ void tile_run(const bf16n_weight & w, const uint32_t * lut, uint32_t * ring, int64_t unit0, int n, int t0,
+                                         int lane, int only_l, char * out, int64_t row_bytes, bool f32) {
+    const w64_ptrs q = w64p(w);
+    tchain ch[1];
+    ch[0].start(ring, q, unit0, n, lane);
+    for (int u = 0; u < n; u++) {
+        ch[0].begin_tile();
+#pragma unroll 1
+        for (int hh = 0; hh < 2; hh++) {
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                uint32_t wp[1][8];
+                tile_step<1>(ch, lut, 0, s, wp);
+                ch[0].reload(s, lane);
+                tile_store_step(wp[0], 4 * hh + s, lane & 31, lane >> 5, only_l, out + (int64_t) (t0 + u) * TILE_K * (f32 ? 4 : 2), row_bytes,
+                                f32);
+            }
+        }
+    }
+}
+
+// rows [row0, row0 + nrows) (whole row groups) as BF16, row-major; one wavefront per (row group, run of slabs)
+__global__ void __launch_bounds__(256) k_tile_dequant(const bf16n_weight w, int64_t row0, int64_t nrows, uint16_t * __restrict__ out) {
+    __shared__ __align__(16) uint32_t lut[LUT_WORDS];
+    extern __shared__ __align__(16) uint32_t rings[];
+    stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
+    const int slabs = (int) (w.K / TILE_K);
+    const int64_t g = (int64_t) blockIdx.x * nwaves + wave;
+    if (g >= nrows / TILE_R) {
+        return;
+    }
+    tile_run(w, lut, rings + wave * WAVE_LDS_WORDS, (row0 / TILE_R + g) * slabs, slabs, 0, lane, -1,
+             (char *) (out + g * TILE_R * w.K), w.K * 2, false);
+}
+
+__global__ void __launch_bounds__(256) k_tile_get_rows(const bf16n_weight w, const char * __restrict__ ids, int64_t ids_s0, int64_t n,
+                                                       int64_t row0, char * __restrict__ dst, int64_t dst_s1, bool f32) {
+    __shared__ __align__(16) uint32_t lut[LUT_WORDS];
+    extern __shared__ __align__(16) uint32_t rings[];
+    stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
+    const int slabs = (int) (w.K / TILE_K);
+    const int64_t i = (int64_t) blockIdx.x * nwaves + wave;
+    if (i >= n) {
+        return;
+    }
+    const int64_t gr = row0 + *(const int32_t *) (ids + i * ids_s0);
+    tile_run(w, lut, rings + wave * WAVE_LDS_WORDS, gr / TILE_R * slabs, slabs, 0, lane, (int) (gr % TILE_R), dst + i * dst_s1, 0, f32);
+}
+
+} // namespace
+
+bool is_tile_layout(const bf16n_weight & w) {
+    return w.format == FMT_HUFPAIR && (w.flags & FLAG_WAVE64) && !(w.flags & FLAG_CHUNK_MAJOR) && w.R == TILE_R;
+}
+
+void tile_init() {
+    (void) hipFuncSetAttribute((const void *) k_mm_tile<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm(true));
+    (void) hipFuncSetAttribute((const void *) k_mm_tile<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm(false));
+}
+
+void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
+                        const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
+                        int cus, hipStream_t stream) {
+    mm_args a;
+    a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
+    a.ids_src1 = ids_src1; a.ids_dst = ids_dst; a.bounds = bounds;
+    a.dst = (char *) dst; a.dst_col = dst_col; a.dst_bf16 = dst_bf16;
+    a.rows = w.rows / n_experts; a.n_experts = n_experts;
+    if (a.rows % TILE_R != 0) {
+        throw std::invalid_argument("bf16n: rows per expert must be a multiple of 32 for the tile layout");
+    }
+    const int groups = (int) (a.rows / TILE_R), gpi = up ? MT_WAVES : 2 * MT_WAVES;
+    const int64_t items = (int64_t) n_experts * ((groups + gpi - 1) / gpi);
+    const dim3 grid((unsigned) (items < (int64_t) cus ? items : (int64_t) cus));
+    if (up) {
+        hipLaunchKernelGGL(k_mm_tile<true>, grid, dim3(MT_THREADS), mt_shm(true), stream, w, *up, a);
+    } else {
+        hipLaunchKernelGGL(k_mm_tile<false>, grid, dim3(MT_THREADS), mt_shm(false), stream, w, w, a);
+    }
+}
+
+// y = W x (up == nullptr) or silu(gate x) * (up x), one column per launch row
+void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols & p, int ncols, bool x_bf16, hipStream_t stream) {
+    const int slabs = (int) (w.K / TILE_K);
+    const int wpg = slabs <= TV_WAVES ? slabs : (slabs + 1) / 2, upw = slabs / wpg, gpb = TV_WAVES / wpg;
+    const int64_t groups = p.nrows / TILE_R;
+    const dim3 grid((unsigned) ((groups + gpb - 1) / gpb), ncols);
+    const size_t shm = (size_t) TV_WAVES * (up ? 2 : 1) * WAVE_LDS_WORDS * 4;
+    if (up) {
+        if (x_bf16) {
+            hipLaunchKernelGGL((k_tile_mmv<bf16_t, true>), grid, dim3(TV_WAVES * 64), shm, stream, w, *up, p, wpg, upw);
+        } else {
+            hipLaunchKernelGGL((k_tile_mmv<float, true>), grid, dim3(TV_WAVES * 64), shm, stream, w, *up, p, wpg, upw);
+        }
+    } else if (x_bf16) {
+        hipLaunchKernelGGL((k_tile_mmv<bf16_t, false>), grid, dim3(TV_WAVES * 64), shm, stream, w, w, p, wpg, upw);
+    } else {
+        hipLaunchKernelGGL((k_tile_mmv<float, false>), grid, dim3(TV_WAVES * 64), shm, stream, w, w, p, wpg, upw);
+    }
+}
+
+void launch_tile_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, hipStream_t stream) {
+    const int64_t groups = nrows / TILE_R;
+    hipLaunchKernelGGL(k_tile_dequant, dim3((unsigned) ((groups + 3) / 4)), dim3(256), 4 * WAVE_LDS_WORDS * 4, stream, w, row0, nrows, out);
+}
+
+void launch_tile_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
+                          int64_t dst_s1, int64_t row0, hipStream_t stream) {
+    hipLaunchKernelGGL(k_tile_get_rows, dim3((unsigned) ((n + 3) / 4)), dim3(256), 4 * WAVE_LDS_WORDS * 4, stream, w,
+                       (const char *) ids, ids_s0, n, row0, (char *) dst, dst_s1, !dst_bf16);
+}
+
+} // namespace dev
+} // namespace bf16n

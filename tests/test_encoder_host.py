@@ -188,3 +188,45 @@ def test_parse_header_rejects_garbage():
         ops.parse_header(aux)
     with pytest.raises(ValueError):
         ops.parse_header(torch.zeros(10, dtype=torch.uint8))
+
+
+def tile32_virtual(w: np.ndarray) -> np.ndarray:
+    """The 512-column matrix V whose wave64 units (16 rows) are the 32 x 256 tiles of w, from the layout's definition:
+    V[16u + 2s + h][128j + 4l + q] = w[32g + l][256t + 32s + 16(j//2) + 8h + 4(j%2) + q], u = g * (K/256) + t."""
+    rows, K = w.shape
+    u, s, h, j, l, q = np.meshgrid(np.arange(rows * K // 8192), np.arange(8), np.arange(2), np.arange(4), np.arange(32),
+                                   np.arange(4), indexing="ij")
+    g, t = u // (K // 256), u % (K // 256)
+    v = np.empty((rows * K // 512, 512), dtype=w.dtype)
+    v[16 * u + 2 * s + h, 128 * j + 4 * l + q] = w[32 * g + l, 256 * t + 32 * s + 16 * (j // 2) + 8 * h + 4 * (j % 2) + q]
+    return v
+
+
+@pytest.mark.parametrize("rows,K", [(32, 512), (64, 2048), (96, 1024)])
+def test_tile32_layout_is_the_wave64_layout_of_the_permuted_matrix(oracle, rows, K):
+    w = synth.model_like(rows, K, rows + K)
+    plane, aux, f, R = ops.encode_bits(w, HP, 32, False, wave64=True)
+    h = oracle.parse_header(aux)
+    assert (f, R, h["R"], h["K"], h["rows"], h["flags"]) == (HP, 32, 32, K, rows, 4)
+    assert np.array_equal(oracle.decode(plane, aux), w)
+    v = tile32_virtual(w)
+    pv, av, _, _ = ops.encode_bits(v, HP, 16, False, wave64=True)
+    assert np.array_equal(plane.reshape(-1), pv.reshape(-1))
+    assert np.array_equal(aux[256:], av[256:])          # table, unit bases and stream; the headers differ in K, R, rows
+    # a lane's 16 weights of a step are two runs of 8 consecutive columns of one row: the A operand of two 32x32x16
+    # matrix instructions (lane l: row l % 32, columns 8 (l // 32) .. + 8 of each 16-column block)
+    vi = tile32_virtual(np.arange(rows * K, dtype=np.int64).reshape(rows, K))
+    for step, lane in ((0, 0), (3, 17), (7, 63), (5, 32)):
+        slots = [vi[2 * step + lane // 32, 128 * (i // 4) + 4 * (lane % 32) + i % 4] for i in range(16)]
+        r0, k0 = lane % 32, 32 * step + 8 * (lane // 32)
+        assert slots == [r0 * K + k0 + i for i in range(8)] + [r0 * K + k0 + 16 + i for i in range(8)]
+
+
+def test_tile32_contract():
+    w = synth.model_like(64, 1024, 5)
+    for bad in (lambda: ops.encode_bits(w, HP, 32, False),                      # only with the wave64 layout
+                lambda: ops.encode_bits(w, HUF, 32, False, wave64=True),
+                lambda: ops.encode_bits(w, HP, 32, True, wave64=True),
+                lambda: ops.encode_bits(w[:48], HP, 32, False, wave64=True)):   # rows must be a multiple of 32
+        with pytest.raises(ValueError):
+            bad()

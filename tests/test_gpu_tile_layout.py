@@ -1,0 +1,177 @@
+"""The tile form of the wave64 layout (R = 32: 32-row x 256-column units in matrix-core operand order) on the GPU:
+bit-exact dequant and row gather against the source bits and the oracle decoder, GEMV / fused gate-up GEMV against the
+oracle (1e-3 relative, 1e-5 absolute floor; FP64 bound 1e-5 * sum|w x|), one-hot activations bit for bit, and the batched
+MoE kernel against FP64 products with the exact weights (reference tests/core/test_kernels.py:248-360)."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GEMV_REL
+from orin_qwen_lossless_amd import synth
+from test_gpu_kernels import check_gemv, rne_bf16, tbf16
+from test_gpu_mm_ids import reference, routing
+from test_gpu_roundtrip import bits, enc
+
+pytestmark = pytest.mark.gpu
+HP = 3
+
+
+@pytest.mark.parametrize("K", [512, 1024, 1536, 2048, 4096])
+def test_dequant_and_get_rows_are_bit_exact(ops, oracle, K):
+    rows = 32 * 5
+    wb = synth.model_like(rows, K, K + 1)
+    plane, aux, _, R = ops.encode_bits(wb, HP, 32, False, wave64=True)
+    assert R == 32 and np.array_equal(oracle.decode(plane, aux), wb)
+    w = enc(ops, wb, HP, 32, False, True)
+    assert np.array_equal(bits(ops.dequant(w)), wb)
+    assert np.array_equal(bits(ops.dequant(w, 64, 96)), wb[64:160])
+    assert ops.roundtrip_equal(w, tbf16(wb))
+    ids = np.array([0, 31, 32, 159, 77, 77, 5], dtype=np.int32)
+    got = ops.get_rows(torch.from_numpy(ids).cuda(), w)
+    assert np.array_equal(bits(got), wb[ids])
+    got32 = ops.get_rows(torch.from_numpy(ids).cuda(), w, out_dtype=torch.float32).cpu().numpy()
+    assert np.array_equal(got32.view(np.uint32), wb[ids].astype(np.uint32) << 16)
+    with pytest.raises(ValueError, match="whole units"):
+        ops.dequant(w, 16, 32)
+
+
+@pytest.mark.parametrize("K", [512, 1024, 1536, 2048, 2560, 4096])
+def test_gemv_dense(ops, oracle, K):
+    rows = 32 * 7
+    wb = synth.weights(rows, K, K + 32)
+    w = enc(ops, wb, HP, 32, False, True)
+    xb = synth.activations(3, K, 7)
+    xf = synth.bf16_bits_to_f32(xb)
+    y_bf = ops.mmv(tbf16(xb), w).cpu().numpy()
+    y_f32 = ops.mmv(torch.from_numpy(xf).cuda(), w).cpu().numpy()
+    check_gemv(oracle, y_bf, wb, xf)
+    check_gemv(oracle, y_f32, wb, xf)
+    y16 = ops.mmv(tbf16(xb), w, out_dtype=torch.bfloat16)
+    assert np.array_equal(bits(y16), rne_bf16(y_bf))
+    y1 = np.stack([ops.mmv(tbf16(xb[t: t + 1]), w).cpu().numpy()[0] for t in range(3)])
+    assert np.array_equal(y1, y_bf)
+
+
+def test_one_hot_activations_give_exact_weights(ops):
+    K, rows = 2048, 64
+    wb = synth.model_like(rows, K, 3)
+    wb[(wb & 0x7F80) == 0x7F80] = 0x3F80
+    w = enc(ops, wb, HP, 32, False, True)
+    for k, scale in ((0, 1.0), (3, -2.0), (517, 0.5), (2047, 4.0), (24, 1.0), (1000, 2.0)):
+        x = np.zeros((1, K), dtype=np.float32)
+        x[0, k] = scale
+        want = synth.bf16_bits_to_f32(wb[:, k]) * np.float32(scale)
+        for xt in (torch.from_numpy(x).cuda(), torch.from_numpy(x).cuda().to(torch.bfloat16)):
+            got = ops.mmv(xt, w).cpu().numpy()[0]
+            nz = np.abs(want) >= np.float32(2.0 ** -126)
+            assert np.array_equal(got[nz], want[nz]), (k, scale)
+
+
+@pytest.mark.parametrize("K,N", [(2048, 64), (512, 128), (4096, 32)])
+def test_routed_gemv_and_fused_gate_up(ops, oracle, K, N):
+    E, T, k = 6, 3, 2
+    gb, ub = synth.weights(E * N, K, 61 + K), synth.weights(E * N, K, 62 + K)
+    g, u = enc(ops, gb, HP, 32, False, True), enc(ops, ub, HP, 32, False, True)
+    assert ops.glu2_supported(g, u)
+    ids = np.array([[0, 5], [3, 1], [5, 2]], dtype=np.int32)
+    xb = synth.activations(T, K, 9)
+    xf = synth.bf16_bits_to_f32(xb)
+    it = torch.from_numpy(ids).cuda()
+    yg = ops.mmv(tbf16(xb), g, ids=it, rows_per_matrix=N).cpu().numpy()
+    yu = ops.mmv(torch.from_numpy(xf).cuda(), u, ids=it, rows_per_matrix=N).cpu().numpy()
+    for t in range(T):
+        for i in range(k):
+            e = ids[t, i]
+            check_gemv(oracle, yg[t, i][None], gb[e * N:(e + 1) * N], xf[t][None])
+            check_gemv(oracle, yu[t, i][None], ub[e * N:(e + 1) * N], xf[t][None])
+    for xt in (tbf16(xb), torch.from_numpy(xf).cuda()):
+        fused = ops.mmv_glu2(xt, g, u, ids=it, rows_per_matrix=N).cpu().numpy()
+        want = yu.astype(np.float64) * (yg.astype(np.float64) / (1.0 + np.exp(-yg.astype(np.float64))))
+        assert np.all(np.abs(fused - want) <= 2e-6 * np.abs(want) + 1e-12)
+    dense = ops.mmv_glu2(tbf16(xb), g, u).cpu().numpy()   # all experts as one dense matrix
+    u0 = ops.mmv(tbf16(xb), u).cpu().numpy().astype(np.float64)
+    g0 = ops.mmv(tbf16(xb), g).cpu().numpy().astype(np.float64)
+    want0 = u0 * (g0 / (1.0 + np.exp(-g0)))
+    assert np.all(np.abs(dense - want0) <= 2e-6 * np.abs(want0) + 1e-12)
+
+
+# (K, rows per expert): gate / up and down shapes, row counts that fill a work item, half of one, and an odd group count
+MM_SHAPES = [(2048, 128), (2048, 512), (512, 256), (512, 544), (1024, 96), (4096, 32)]
+
+
+@pytest.mark.parametrize("K,N", MM_SHAPES)
+def test_mm_ids_against_exact_weights(ops, K, N):
+    E, k, T = 6, 2, 260
+    wb = synth.weights(E * N, K, 11 + K + N)
+    w = enc(ops, wb, HP, 32, False, True)
+    assert ops.mm_ids_supported(w)
+    wf = synth.bf16_bits_to_f32(wb)
+    ids = routing(T, k, E, {0: 129, 1: 128, 2: 127, 3: 0}, 5)
+    per_slot = K == 512
+    xb = synth.activations(T * (k if per_slot else 1), K, 3).reshape((T, k, K) if per_slot else (T, K))
+    xf = synth.bf16_bits_to_f32(xb)
+    got = ops.moe_mm_ids(tbf16(xb), torch.from_numpy(ids).cuda(), w, E).cpu().numpy()
+    y, s = reference(wf, xf, ids, N, per_slot)
+    assert np.all(np.abs(got - y) <= GEMV_REL * s + 1e-30)
+    assert np.all(np.abs(got - y) <= 1e-3 * np.abs(y) + 1e-5)
+    got16 = ops.moe_mm_ids(tbf16(xb), torch.from_numpy(ids).cuda(), w, E, out_dtype=torch.bfloat16)
+    assert np.array_equal(bits(got16), rne_bf16(got))
+
+
+@pytest.mark.parametrize("K,N", MM_SHAPES)
+def test_mm_ids_one_hot_is_exact(ops, K, N):
+    E, k, T = 4, 2, 70
+    wb = synth.weights(E * N, K, 21 + K)
+    w = enc(ops, wb, HP, 32, False, True)
+    wf = synth.bf16_bits_to_f32(wb)
+    ids = routing(T, k, E, {}, 9)
+    per_slot = K == 512
+    shape = (T, k, K) if per_slot else (T, K)
+    xf = np.zeros(shape, dtype=np.float32)
+    cols = np.random.default_rng(2).integers(0, K, size=shape[:-1])
+    np.put_along_axis(xf, cols[..., None], 0.125, axis=-1)
+    got = ops.moe_mm_ids(torch.from_numpy(xf).cuda().to(torch.bfloat16), torch.from_numpy(ids).cuda(), w, E).cpu().numpy()
+    for t in range(T):
+        for i in range(k):
+            c = cols[t, i] if per_slot else cols[t]
+            assert np.array_equal(got[t, i], wf[ids[t, i] * N: (ids[t, i] + 1) * N, c] * np.float32(0.125)), (t, i)
+
+
+@pytest.mark.parametrize("K,N", [(2048, 128), (2048, 512), (1024, 96)])
+def test_mm_ids_fused_gate_up_swiglu(ops, K, N):
+    E, k, T = 5, 3, 150
+    gb, ub = synth.weights(E * N, K, 31), synth.weights(E * N, K, 32)
+    g, u = enc(ops, gb, HP, 32, False, True), enc(ops, ub, HP, 32, False, True)
+    assert ops.mm_ids_supported(g, u)
+    ids = routing(T, k, E, {4: 0}, 6)
+    xb = synth.activations(T, K, 8)
+    xt, it = tbf16(xb), torch.from_numpy(ids).cuda()
+    fused = ops.moe_mm_ids(xt, it, g, E, up=u).cpu().numpy()
+    yg = ops.moe_mm_ids(xt, it, g, E).cpu().numpy()
+    yu = ops.moe_mm_ids(xt, it, u, E).cpu().numpy()
+    want = (yu.astype(np.float64) * (yg.astype(np.float64) / (1.0 + np.exp(-yg.astype(np.float64)))))
+    assert np.all(np.abs(fused - want) <= 2e-6 * np.abs(want) + 1e-12)
+    xf = synth.bf16_bits_to_f32(xb)
+    y1, _ = reference(synth.bf16_bits_to_f32(gb), xf, ids, N, False)
+    y2, _ = reference(synth.bf16_bits_to_f32(ub), xf, ids, N, False)
+    ref = y2 * (y1 / (1.0 + np.exp(-y1)))
+    assert np.all(np.abs(fused - ref) <= 1e-3 * np.abs(ref) + 1e-5)
+    f16 = ops.moe_mm_ids(xt, it, g, E, up=u, out_dtype=torch.bfloat16)
+    assert np.array_equal(bits(f16), rne_bf16(fused))
+
+
+@pytest.mark.parametrize("T", [8, 9, 40])
+def test_moe_experts_in_both_token_regimes(ops, T):
+    E, k, Kd, N = 8, 2, 2048, 512
+    gate = enc(ops, synth.weights(E * N, Kd, 51), HP, 32, False, True)
+    up = enc(ops, synth.weights(E * N, Kd, 52), HP, 32, False, True)
+    down = enc(ops, synth.weights(E * Kd, N, 53), HP, 32, False, True)
+    ids = torch.from_numpy(routing(T, k, E, {}, T)).cuda()
+    wts = torch.softmax(torch.randn((T, k), generator=torch.Generator().manual_seed(T)), dim=-1).cuda()
+    x = tbf16(synth.activations(T, Kd, 54))
+    got = ops.moe_experts(x, gate, up, down, wts, ids, E).float().cpu().numpy()
+    ref = ops.moe_experts_reference(x, gate, up, down, wts, ids, E).float().cpu().numpy()
+    scale = np.abs(ref).max()
+    assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
