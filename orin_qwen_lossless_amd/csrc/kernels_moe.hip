@@ -33,65 +33,64 @@ __global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ 
 
 // Routing lists (reference mmid_helper.cu:48-136): block e lists the (token, slot) pairs of expert e in token order at
 // positions bounds[e].., where bounds[e] = number of pairs of experts < e.  ids element i of token t at byte
-// ids + (t * stride + i) * elem (low 32 bits are read).
+// ids + (t * stride + i) * elem (low 32 bits are read).  Every thread owns a run of consecutive tokens: it counts its
+// pairs of lower experts and its own hits, one block-wide scan turns the hit counts into positions, and a second walk
+// over the run writes the lists.
 __global__ void __launch_bounds__(256) k_route(const char * __restrict__ ids, int elem, int64_t stride, int32_t * __restrict__ ids_src1,
                                                int32_t * __restrict__ ids_dst, int32_t * __restrict__ bounds, int n_tok, int n_used,
                                                int nchannels_y, int sis1) {
     __shared__ int wave_hits[4], wave_lower[4];
-    __shared__ int s_lower_total;
     const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // pass 1: pairs of lower experts (the start of this expert's range)
-    int lower = 0;
-    for (int64_t i = tid; i < (int64_t) n_tok * n_used; i += 256) {
-        const int64_t t = i / n_used, k = i % n_used;
-        lower += *(const int32_t *) (ids + (t * stride + k) * elem) < e;
+    const int per = (n_tok + 255) / 256;
+    const int t_begin = tid * per < n_tok ? tid * per : n_tok, t_end = t_begin + per < n_tok ? t_begin + per : n_tok;
+    int lower = 0, hits = 0;
+    for (int t = t_begin; t < t_end; t++) {
+        bool hit = false;
+        for (int k = 0; k < n_used; k++) {
+            const int v = *(const int32_t *) (ids + ((int64_t) t * stride + k) * elem);
+            lower += v < e;
+            hit |= v == e;
+        }
+        hits += hit;
     }
+    // inclusive scan of the hit counts and sum of the lower counts inside the wavefront, then over the four wavefronts
+    int scan = hits;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(scan, o, 64);
+        scan += lane >= o ? up : 0;
+    }
+#pragma unroll
     for (int o = 32; o; o >>= 1) {
         lower += __shfl_xor(lower, o, 64);
     }
-    if (lane == 0) {
+    if (lane == 63) {
+        wave_hits[wave] = scan;
         wave_lower[wave] = lower;
     }
     __syncthreads();
-    if (tid == 0) {
-        s_lower_total = wave_lower[0] + wave_lower[1] + wave_lower[2] + wave_lower[3];
+    const int base = wave_lower[0] + wave_lower[1] + wave_lower[2] + wave_lower[3];
+    int j = base + scan - hits;
+    for (int w2 = 0; w2 < wave; w2++) {
+        j += wave_hits[w2];
     }
-    __syncthreads();
-    const int base = s_lower_total;
-    // pass 2: compact the tokens that use expert e, 256 tokens per round, in token order
-    int run = 0;
-    for (int t0 = 0; t0 < n_tok; t0 += 256) {
-        const int t = t0 + tid;
+    for (int t = t_begin; t < t_end; t++) {
         int slot = -1;
-        if (t < n_tok) {
-            for (int k = 0; k < n_used; k++) {
-                if (*(const int32_t *) (ids + ((int64_t) t * stride + k) * elem) == e) {
-                    slot = k;
-                }
+        for (int k = 0; k < n_used; k++) {
+            if (*(const int32_t *) (ids + ((int64_t) t * stride + k) * elem) == e) {
+                slot = k; // a token lists an expert once; were it listed twice, the last slot counts
             }
         }
-        const uint64_t m = __ballot(slot >= 0);
-        const int before = (int) __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
-        if (lane == 0) {
-            wave_hits[wave] = (int) __builtin_popcountll(m);
-        }
-        __syncthreads();
-        int off = run;
-        for (int w2 = 0; w2 < wave; w2++) {
-            off += wave_hits[w2];
-        }
         if (slot >= 0) {
-            const int j = base + off + before;
             ids_dst[j] = t * n_used + slot;
             ids_src1[j] = t * sis1 + slot % nchannels_y;
+            j++;
         }
-        run += wave_hits[0] + wave_hits[1] + wave_hits[2] + wave_hits[3];
-        __syncthreads();
     }
     if (tid == 0) {
         bounds[e] = base;
         if (e == (int) gridDim.x - 1) {
-            bounds[gridDim.x] = base + run;
+            bounds[gridDim.x] = base + wave_hits[0] + wave_hits[1] + wave_hits[2] + wave_hits[3];
         }
     }
 }
