@@ -44,6 +44,11 @@ struct tchain {
         return *((const uint4 *) (plane + o) + lane);
     }
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane) {
+        start(ring, q, unit0, n_units, lane, q.ubase[unit0], q.ubase[unit0 + n_units]);
+    }
+    // first / end: the stream words of the units (their unit bases, read by the caller ahead of time)
+    __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane, uint32_t first,
+                                          uint32_t end) {
         plane = q.plane + uniform64(unit0 * T_BYTES);
         off = 0;
         last = (uint32_t) (n_units * T_BYTES - STEP_BYTES);
@@ -52,7 +57,7 @@ struct tchain {
             sm[s] = load_step(lane);
             off += STEP_BYTES;
         }
-        dec.start(ring, q.stream, uniform(q.ubase[unit0]), uniform(q.ubase[unit0 + n_units]), lane);
+        dec.start(ring, q.stream, uniform(first), uniform(end), lane);
     }
     __device__ __forceinline__ void reload(int s, int lane) {
         sm[s] = load_step(lane);
@@ -139,11 +144,9 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
             const int btk = tp + b_tok;
             const uint16_t * xsrc = a.x + (int64_t) a.ids_src1[j0 + (btk < n ? btk : 0)] * a.x_row + 32 * b_part;
             uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + 32 * b_part;
-            uint4 breg[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                breg[i] = *((const uint4 *) xsrc + i);
-            }
+            // (four named registers, not an array: under this kernel's register pressure an array stays in scratch)
+            const uint4 f0 = *((const uint4 *) xsrc), f1 = *((const uint4 *) xsrc + 1), f2 = *((const uint4 *) xsrc + 2),
+                        f3 = *((const uint4 *) xsrc + 3);
             tchain ch[2];
             if (live) {
                 uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
@@ -161,20 +164,21 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
                     }
                 }
             }
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                *((uint4 *) bdst + i) = breg[i];
-            }
+            *((uint4 *) bdst) = f0;
+            *((uint4 *) bdst + 1) = f1;
+            *((uint4 *) bdst + 2) = f2;
+            *((uint4 *) bdst + 3) = f3;
             __syncthreads();
 #pragma unroll 1
             for (int hs = 0; hs < halves; hs++) {
                 const uint16_t * bcur = bbuf + (hs & 1) * (MT_TOK * MT_BSTRIDE);
-                if (hs + 1 < halves) { // the next block of activations: requested now, staged after this block's steps
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        breg[i] = *((const uint4 *) (xsrc + (hs + 1) * MT_HK) + i);
-                    }
-                }
+                // the next block of activations: requested now, staged after this block's steps.  Unconditional and
+                // local to the iteration (after the last block the same block goes into the buffer nobody reads any
+                // more): registers that are loaded under a condition and live around the loop are filled through a
+                // temporary with a full wait per load.
+                const int nxt = hs + 1 < halves ? hs + 1 : hs;
+                const uint4 * bsrc = (const uint4 *) (xsrc + nxt * MT_HK);
+                const uint4 b0 = bsrc[0], b1 = bsrc[1], b2 = bsrc[2], b3 = bsrc[3];
                 if (live) {
                     if ((hs & 1) == 0) {
                         ch[0].begin_tile();
@@ -187,29 +191,35 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
                         ch[0].reload(s, lane);
                         ch[1].reload(s, lane);
                         const uint16_t * bp = bcur + l32 * MT_BSTRIDE + 32 * s + 8 * half;
+                        bf16x8_t av[2][2]; // [chain][16-column block]
 #pragma unroll
-                        for (int kb = 0; kb < 2; kb++) {
-                            const u32x4_t a0 = {wp[0][4 * kb], wp[0][4 * kb + 1], wp[0][4 * kb + 2], wp[0][4 * kb + 3]};
-                            const u32x4_t a1 = {wp[1][4 * kb], wp[1][4 * kb + 1], wp[1][4 * kb + 2], wp[1][4 * kb + 3]};
-                            const bf16x8_t av0 = __builtin_bit_cast(bf16x8_t, a0), av1 = __builtin_bit_cast(bf16x8_t, a1);
+                        for (int c = 0; c < 2; c++) {
 #pragma unroll
-                            for (int t = 0; t < 4; t++) {
-                                if (t < nt) {
-                                    const bf16x8_t bv = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE + 16 * kb);
-                                    acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av0, bv, acc[0][t], 0, 0, 0);
-                                    acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av1, bv, acc[1][t], 0, 0, 0);
-                                }
+                            for (int kb = 0; kb < 2; kb++) {
+                                const u32x4_t v = {wp[c][4 * kb], wp[c][4 * kb + 1], wp[c][4 * kb + 2], wp[c][4 * kb + 3]};
+                                av[c][kb] = __builtin_bit_cast(bf16x8_t, v);
+                            }
+                        }
+                        // token blocks beyond the first are there only for experts with that many tokens (one branch
+                        // per block: both B operands are read together, then four matrix instructions)
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            if (t == 0 || t < nt) {
+                                const bf16x8_t bv0 = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE);
+                                const bf16x8_t bv1 = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE + 16);
+                                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0][0], bv0, acc[0][t], 0, 0, 0);
+                                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][0], bv0, acc[1][t], 0, 0, 0);
+                                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0][1], bv1, acc[0][t], 0, 0, 0);
+                                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][1], bv1, acc[1][t], 0, 0, 0);
                             }
                         }
                     }
                 }
-                if (hs + 1 < halves) {
-                    uint16_t * bn = bdst + ((hs + 1) & 1) * (MT_TOK * MT_BSTRIDE);
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        *((uint4 *) bn + i) = breg[i];
-                    }
-                }
+                uint4 * bn = (uint4 *) (bdst + ((hs + 1) & 1) * (MT_TOK * MT_BSTRIDE));
+                bn[0] = b0;
+                bn[1] = b1;
+                bn[2] = b2;
+                bn[3] = b3;
                 __syncthreads();
             }
             // accumulator element i of a lane: row 8 (i / 4) + 4 (lane / 32) + i % 4 of the group, token lane % 32
@@ -305,18 +315,20 @@ __global__ void __launch_bounds__(TV_WAVES * 64) k_tile_mmv(const bf16n_weight w
     const col_view cv = col_setup(p, blockIdx.y);
     const int64_t groups = p.nrows / TILE_R, g = (int64_t) blockIdx.x * gpb + gi;
     const bool live = gi < gpb && g < groups;
+    const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
+    const int64_t unit0 = live ? (cv.rbase / TILE_R + g) * slabs + wi * upw : 0;
+    // the unit bases first: the stream loads that depend on them can start as soon as the tables are requested
+    const uint32_t f0 = q0.ubase[unit0], e0 = q0.ubase[unit0 + upw], f1 = q1.ubase[unit0], e1 = q1.ubase[unit0 + upw];
     stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
     if (GLU) {
         stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
     }
-    const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
-    const int64_t unit0 = live ? (cv.rbase / TILE_R + g) * slabs + wi * upw : 0;
     tchain ch[NM];
     if (live) {
         uint32_t * ring = rings + wave * (NM * WAVE_LDS_WORDS);
-        ch[0].start(ring, q0, unit0, upw, lane);
+        ch[0].start(ring, q0, unit0, upw, lane, f0, e0);
         if (GLU) {
-            ch[NM - 1].start(ring + WAVE_LDS_WORDS, q1, unit0, upw, lane);
+            ch[NM - 1].start(ring + WAVE_LDS_WORDS, q1, unit0, upw, lane, f1, e1);
         }
     }
     __syncthreads();
