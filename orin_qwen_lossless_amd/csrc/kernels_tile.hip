@@ -298,48 +298,44 @@ template <> struct x8<float> {
     }
 };
 
-constexpr int TV_WAVES = 8;
+constexpr int TV_WAVES = 16;
 
-// A block covers `gpb` row groups of one column; the `wpg` wavefronts of a group take `upw` consecutive tiles each and
-// their partial sums (one per lane and row) are added in tile order.  GLU: every wavefront decodes its tiles of the
-// gate and the up matrix side by side and the block writes silu(gate x) * (up x).
+// A block covers `gpb` row groups of one column.  Each wavefront runs one decode chain — `upw` consecutive tiles of
+// one matrix (at decode a launch is a few hundred tiles and its time is the length of a chain: one short chain per
+// wavefront, many wavefronts) — and the partial sums (one per lane and row) of a group's `wpg` wavefronts per matrix
+// are added in tile order.  GLU: the group has wpg wavefronts on the gate matrix and wpg on the up matrix, and the
+// block writes silu(gate x) * (up x).
 template <typename TX, bool GLU>
-__global__ void __launch_bounds__(TV_WAVES * 64) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw) {
+__global__ void __launch_bounds__(GLU ? TV_WAVES * 64 : TV_WAVES * 32) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw) {
     constexpr int NM = GLU ? 2 : 1;
     __shared__ __align__(16) uint32_t lut[NM * LUT_WORDS];
-    __shared__ float part[NM][TV_WAVES][32];
+    __shared__ float part[TV_WAVES][32];
     extern __shared__ __align__(16) uint32_t rings[];
     const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
-    const int slabs = (int) (w.K / TILE_K), gpb = TV_WAVES / wpg;
-    const int gi = wave / wpg, wi = wave % wpg;
+    const int slabs = (int) (w.K / TILE_K), wpgm = NM * wpg, gpb = (int) (blockDim.x >> 6) / wpgm;
+    const int gi = wave / wpgm, m = (wave % wpgm) / wpg, wi = wave % wpg; // group in the block, matrix, position in K
     const col_view cv = col_setup(p, blockIdx.y);
     const int64_t groups = p.nrows / TILE_R, g = (int64_t) blockIdx.x * gpb + gi;
     const bool live = gi < gpb && g < groups;
-    const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
+    const w64_ptrs q = w64p(GLU && m ? w_up : w);
     const int64_t unit0 = live ? (cv.rbase / TILE_R + g) * slabs + wi * upw : 0;
     // the unit bases first: the stream loads that depend on them can start as soon as the tables are requested
-    const uint32_t f0 = q0.ubase[unit0], e0 = q0.ubase[unit0 + upw], f1 = q1.ubase[unit0], e1 = q1.ubase[unit0 + upw];
+    const uint32_t first = q.ubase[unit0], end = q.ubase[unit0 + upw];
     stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
     if (GLU) {
         stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
     }
-    tchain ch[NM];
+    tchain ch[1];
     if (live) {
-        uint32_t * ring = rings + wave * (NM * WAVE_LDS_WORDS);
-        ch[0].start(ring, q0, unit0, upw, lane, f0, e0);
-        if (GLU) {
-            ch[NM - 1].start(ring + WAVE_LDS_WORDS, q1, unit0, upw, lane, f1, e1);
-        }
+        ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end);
     }
     __syncthreads();
-    float acc[NM] = {};
     if (live) {
+        const uint32_t * my_lut = lut + m * LUT_WORDS;
+        float acc = 0.f;
         for (int u = 0; u < upw; u++) {
             const int k0 = (wi * upw + u) * TILE_K + 8 * half;
-#pragma unroll
-            for (int k = 0; k < NM; k++) {
-                ch[k].begin_tile();
-            }
+            ch[0].begin_tile();
 #pragma unroll 1
             for (int hh = 0; hh < 2; hh++) { // two halves of four steps: the step index into the plane registers stays static
 #pragma unroll
@@ -348,32 +344,26 @@ __global__ void __launch_bounds__(TV_WAVES * 64) k_tile_mmv(const bf16n_weight w
                     x8<TX> xa, xb;
                     xa.load(cv.x, kk);
                     xb.load(cv.x, kk + 16);
-                    uint32_t wp[NM][8];
-                    tile_step<NM>(ch, lut, LUT_WORDS, s, wp);
-#pragma unroll
-                    for (int k = 0; k < NM; k++) {
-                        ch[k].reload(s, lane);
-                        acc[k] = xb.dot(wp[k] + 4, xa.dot(wp[k], acc[k]));
-                    }
+                    uint32_t wp[1][8];
+                    tile_step<1>(ch, my_lut, 0, s, wp);
+                    ch[0].reload(s, lane);
+                    acc = xb.dot(wp[0] + 4, xa.dot(wp[0], acc));
                 }
             }
         }
-#pragma unroll
-        for (int k = 0; k < NM; k++) {
-            const float v = acc[k] + __shfl_xor(acc[k], 32, 64);
-            if (half == 0) {
-                part[k][wave][l32] = v;
-            }
+        const float v = acc + __shfl_xor(acc, 32, 64);
+        if (half == 0) {
+            part[wave][l32] = v;
         }
     }
     __syncthreads();
-    if (live && wi == 0 && half == 0) {
+    if (live && m == 0 && wi == 0 && half == 0) {
         float s[NM];
 #pragma unroll
         for (int k = 0; k < NM; k++) {
-            s[k] = part[k][wave][l32];
+            s[k] = part[wave + k * wpg][l32];
             for (int i = 1; i < wpg; i++) {
-                s[k] += part[k][wave + i][l32];
+                s[k] += part[wave + k * wpg + i][l32];
             }
         }
         store_y(cv.y, p.y_bf16, g * TILE_R + l32, GLU ? s[NM - 1] * silu(s[0]) : s[0]);
@@ -490,20 +480,24 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
 // y = W x (up == nullptr) or silu(gate x) * (up x), one column per launch row
 void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols & p, int ncols, bool x_bf16, hipStream_t stream) {
     const int slabs = (int) (w.K / TILE_K);
-    const int wpg = slabs <= TV_WAVES ? slabs : (slabs + 1) / 2, upw = slabs / wpg, gpb = TV_WAVES / wpg;
+    // wavefronts per row group and matrix: one per tile up to 8 tiles (K <= 2048), two tiles each beyond
+    const int wpg = slabs <= 8 ? slabs : (slabs + 1) / 2, upw = slabs / wpg, wpgm = wpg * (up ? 2 : 1);
+    // blocks of four wavefronts where a row group takes at most four: more, smaller blocks spread a routed GEMV (a
+    // few hundred tiles) over more compute units
+    const int waves = wpgm <= 4 ? 4 : wpgm <= 8 ? 8 : TV_WAVES, gpb = waves / wpgm;
     const int64_t groups = p.nrows / TILE_R;
     const dim3 grid((unsigned) ((groups + gpb - 1) / gpb), ncols);
-    const size_t shm = (size_t) TV_WAVES * (up ? 2 : 1) * WAVE_LDS_WORDS * 4;
+    const size_t shm = (size_t) waves * WAVE_LDS_WORDS * 4;
     if (up) {
         if (x_bf16) {
-            hipLaunchKernelGGL((k_tile_mmv<bf16_t, true>), grid, dim3(TV_WAVES * 64), shm, stream, w, *up, p, wpg, upw);
+            hipLaunchKernelGGL((k_tile_mmv<bf16_t, true>), grid, dim3(waves * 64), shm, stream, w, *up, p, wpg, upw);
         } else {
-            hipLaunchKernelGGL((k_tile_mmv<float, true>), grid, dim3(TV_WAVES * 64), shm, stream, w, *up, p, wpg, upw);
+            hipLaunchKernelGGL((k_tile_mmv<float, true>), grid, dim3(waves * 64), shm, stream, w, *up, p, wpg, upw);
         }
     } else if (x_bf16) {
-        hipLaunchKernelGGL((k_tile_mmv<bf16_t, false>), grid, dim3(TV_WAVES * 64), shm, stream, w, w, p, wpg, upw);
+        hipLaunchKernelGGL((k_tile_mmv<bf16_t, false>), grid, dim3(waves * 64), shm, stream, w, w, p, wpg, upw);
     } else {
-        hipLaunchKernelGGL((k_tile_mmv<float, false>), grid, dim3(TV_WAVES * 64), shm, stream, w, w, p, wpg, upw);
+        hipLaunchKernelGGL((k_tile_mmv<float, false>), grid, dim3(waves * 64), shm, stream, w, w, p, wpg, upw);
     }
 }
 
