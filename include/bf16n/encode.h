@@ -20,8 +20,9 @@ struct encoded {
 // rows x K BF16 bit patterns, row-major.  K a multiple of 512 in [512, 4096]; NIBBLE takes R = 0 and no layout;
 // the Huffman formats take R in {1, 2, 4, 8, 16} dividing rows; chunk_major needs HUFPAIR, K > 512, R in {4, 8, 16};
 // frag_order is the reference's NVIDIA operand order and is refused; wave64 (HUFPAIR, row-major, R * K / 512 even)
-// asks for the 64-lane stream layout.  std::invalid_argument on a broken rule, std::runtime_error on an encoder
-// invariant.
+// asks for the 64-lane stream layout; with it R = 32 (rows a multiple of 32) asks for 32-row x 256-column tiles in the
+// operand order of the matrix cores (format.h: TILE_R, TILE_K).  std::invalid_argument on a broken rule,
+// std::runtime_error on an encoder invariant.
 inline encoded encode(const uint16_t * w, int64_t rows, int64_t K, int format, int R, bool chunk_major, bool frag_order = false,
                       bool wave64 = false) {
     const uint32_t flags = (chunk_major ? FLAG_CHUNK_MAJOR : 0u) | (frag_order ? FLAG_FRAG_ORDER : 0u) | (wave64 ? FLAG_WAVE64 : 0u);

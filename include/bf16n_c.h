@@ -31,7 +31,8 @@ const char * bf16n_last_error(void);
 /* ---- host encoder: bf16n::encode, core/include/bf16n/encode.h:12-26, core/src/encode.cpp:443-526 ----------------- */
 typedef struct bf16n_encoded bf16n_encoded; /* owns plane + aux (struct encoded, encode.h:12-17) */
 /* w: rows x K BF16 bit patterns, row-major (host).  flags: BF16N_FLAG_* layout bits (chunk_major / frag_order arguments
- * of the reference; FRAG_ORDER is rejected with EINVAL, WAVE64 is this build's wave64 stream layout). */
+ * of the reference; FRAG_ORDER is rejected with EINVAL, WAVE64 is this build's wave64 stream layout).  R: rows per unit,
+ * {1, 2, 4, 8, 16} as in the reference, or 32 with WAVE64 for 32-row x 256-column tiles in matrix-core operand order. */
 int bf16n_encode(const uint16_t * w, int64_t rows, int64_t K, int format, int R, uint32_t flags, bf16n_encoded ** out);
 const uint8_t * bf16n_encoded_plane(const bf16n_encoded * e, uint64_t * bytes);
 const uint8_t * bf16n_encoded_aux(const bf16n_encoded * e, uint64_t * bytes);
@@ -44,7 +45,7 @@ void bf16n_set_encode_threads(int n);
 /* ---- shape policy: bf16n::choose, core/include/bf16n/policy.h:12-38, core/src/policy.cpp:45-69 -------------------- */
 /* out[5] = {format, R, chunk_major, frag_order, wave64}.  Returns 1 if a choice was made, 0 if the shape stays BF16
  * (std::nullopt).  Never fails.  engine MI355X: the reference's llama rules with unit sizes chosen for 256 CUs of
- * wave64 and the wave64 stream layout where the shape allows it. */
+ * wave64 and the wave64 stream layout where the shape allows it; experts with a multiple of 32 rows get R = 32 tiles. */
 int bf16n_choose(int64_t rows, int64_t K, int64_t n_matrices, int engine, int mode, int64_t dense_min, int expert,
                  int dense_frag_order, int * out);
 

@@ -77,10 +77,18 @@ bool choose(int64_t rows, int64_t K, int64_t n, int engine, int mode, int64_t de
     const int64_t C = K / CHUNK;
     if (mi355x) {
         int R;
+        if (n > 1 && rows % TILE_R == 0) {
+            // experts whose row count allows it: 32-row x 256-column tiles in matrix-core operand order.  The batched
+            // kernel (more than 8 tokens: prefill, and decode at serving batch sizes) decodes them straight into MFMA
+            // operands, about 2x faster than through a tile in LDS; a tile is 8 decode steps, as short a chain for the
+            // routed GEMV at decode as the 4-row units below (measured: +2 us on a 47 us MoE layer at batch 1).
+            out = {FMT_HUFPAIR, TILE_R, false, false, true};
+            return true;
+        }
         if (n > 1) {
-            // experts: the reference's rule (policy.cpp:59-61), except that matrices with long rows take units of 4
-            // rows: at decode only top-k experts are read, a routed GEMV is a few hundred units, and its time is the
-            // length of one unit's decode chain (8 steps instead of 16; +1.9 % bytes on a 35B-A3B layer)
+            // other experts: the reference's rule (policy.cpp:59-61), except that matrices with long rows take units
+            // of 4 rows: at decode only top-k experts are read, a routed GEMV is a few hundred units, and its time is
+            // the length of one unit's decode chain (8 steps instead of 16; +1.9 % bytes on a 35B-A3B layer)
             R = rows % 16 == 0 && rows >= 2048 ? 16 : rows % 8 == 0 ? 8 : rows % 4 == 0 ? 4 : 1;
             if ((C == 2 || C == 4 || C == 8) && rows % 4 == 0) { // the shapes that get the wave64 layout below
                 R = 4;

@@ -168,12 +168,15 @@ def test_policy_mi355x():
     assert ops.choose(248320, 2048) == (HP, 16, False, False, True)
     assert ops.choose(5120, 2048) == (HP, 4, False, False, True)
     assert ops.choose(2048, 4096) == (HP, 2, False, False, True)
-    assert ops.choose(512, 2048, 256, expert=True) == (HP, 4, False, False, True)
-    assert ops.choose(2048, 512, 256, expert=True) == (HP, 16, False, False, True)
+    # experts: 32 x 256 tiles in matrix-core operand order where the rows per expert allow it, else units of 4 rows
+    assert ops.choose(512, 2048, 256, expert=True) == (HP, 32, False, False, True)
+    assert ops.choose(2048, 512, 256, expert=True) == (HP, 32, False, False, True)
+    assert ops.choose(96, 1536, 8, expert=True) == (HP, 32, False, False, True)
+    assert ops.choose(144, 2048, 8, expert=True) == (HP, 4, False, False, True)
     assert ops.choose(512, 2048)[0] == NIB and ops.choose(2048, 512)[0] == NIB and ops.choose(256, 2048)[0] == NIB
     # shapes without a wave64 GEMV instance keep the reference layouts
     assert ops.choose(16384, 1536) == (HP, 4, False, False, False)
-    assert ops.choose(512, 1536, 8, expert=True) == (HP, 8, True, False, False)
+    assert ops.choose(520, 1536, 8, expert=True) == (HP, 8, True, False, False)
 
 
 def test_parse_header_rejects_garbage():
