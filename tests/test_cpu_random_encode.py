@@ -23,6 +23,9 @@ def cases(n: int):
         rows = int(rng.integers(1, 12)) * max(R, 1)
         kind = int(rng.integers(0, 3))
         out.append((K, fmt, R, cm, w64, rows, kind, int(rng.integers(1 << 30))))
+    for _ in range(n // 4):  # the tile form of the wave64 layout: R = 32, any K
+        K = int(rng.choice([512, 1024, 1536, 2048, 3072, 4096]))
+        out.append((K, HP, 32, False, True, 32 * int(rng.integers(1, 5)), int(rng.integers(0, 3)), int(rng.integers(1 << 30))))
     return out
 
 
@@ -36,7 +39,8 @@ def test_random_encode(oracle, K, fmt, R, cm, w64, rows, kind, seed):
         rng = np.random.default_rng(seed)
         w = (rng.integers(0, 2, (rows, K)) << 15 | rng.integers(90, 140, (rows, K)) << 7 | rng.integers(0, 128, (rows, K))).astype(np.uint16)
     plane, aux, fmt_out, R_out = ops.encode_bits(w, fmt, R, cm, wave64=w64)
-    assert fmt_out in (fmt, HUF) and R_out == R
+    # more than 4096 distinct exponent pairs: the single-symbol format, which has no tiles (units of 16 rows instead)
+    assert fmt_out in (fmt, HUF) and R_out == (16 if R == 32 and fmt_out == HUF else R)
     assert np.array_equal(oracle.decode(plane, aux), w)
     if oracle.ref() is not None and not w64:
         rp, ra, rf, _ = oracle.ref_encode(w, fmt, R, cm)

@@ -180,7 +180,18 @@ def sweep_cases(n: int):
     return out
 
 
-@pytest.mark.parametrize("K,R,cm,w64,E,N,k,T,fused,seed", sweep_cases(24))
+def tile_sweep_cases(n: int):
+    rng = np.random.default_rng(2424)
+    out = []
+    for i in range(n):
+        K = [2048, 512, 1024, 4096, 1536][i % 5]
+        E = int(rng.integers(2, 10))
+        out.append((K, 32, False, True, E, 32 * int(rng.integers(1, 20)), int(rng.integers(1, min(E, 4) + 1)), int(rng.integers(9, 300)),
+                    bool(rng.integers(2)), int(rng.integers(1 << 30))))
+    return out
+
+
+@pytest.mark.parametrize("K,R,cm,w64,E,N,k,T,fused,seed", sweep_cases(24) + tile_sweep_cases(20))
 def test_mm_ids_seeded_sweep(ops, K, R, cm, w64, E, N, k, T, fused, seed):
     rng = np.random.default_rng(seed)
     wb = synth.weights(E * N, K, seed)
@@ -193,7 +204,7 @@ def test_mm_ids_seeded_sweep(ops, K, R, cm, w64, E, N, k, T, fused, seed):
     y, s = reference(synth.bf16_bits_to_f32(wb), xf, ids, N, per_slot)
     got = ops.moe_mm_ids(tbf16(xb), it, w, E).cpu().numpy()
     assert np.all(np.abs(got - y) <= 1e-5 * s + 1e-30)
-    if fused and K == 2048:
+    if fused and (K == 2048 or R == 32) and not per_slot:
         ub = synth.weights(E * N, K, seed + 2)
         u = enc(ops, ub, HP, R, cm, w64)
         yu, _ = reference(synth.bf16_bits_to_f32(ub), xf, ids, N, False)

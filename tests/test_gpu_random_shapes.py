@@ -34,7 +34,18 @@ def cases(n: int):
     return out
 
 
-@pytest.mark.parametrize("K,fmt,R,cm,w64,rows_per,E,T,seed", cases(120))
+def tile_cases(n: int):
+    """The tile form of the wave64 layout (R = 32): any K, row groups per matrix, experts, batch."""
+    rng = np.random.default_rng(31337)
+    out = []
+    for _ in range(n):
+        K = int(rng.choice([512, 1024, 1536, 2048, 2560, 3072, 3584, 4096]))
+        out.append((K, HP, 32, False, True, 32 * int(rng.integers(1, 12)), int(rng.choice([1, 1, 3, 5])), int(rng.integers(1, 9)),
+                    int(rng.integers(1 << 30))))
+    return out
+
+
+@pytest.mark.parametrize("K,fmt,R,cm,w64,rows_per,E,T,seed", cases(120) + tile_cases(40))
 def test_random_configuration(ops, K, fmt, R, cm, w64, rows_per, E, T, seed):
     rows = rows_per * E
     wb = synth.model_like(rows, K, seed) if seed % 3 == 0 else synth.weights(rows, K, seed)
