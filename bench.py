@@ -117,7 +117,7 @@ def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: s
     ta = torch.from_numpy(aux)
     meta = ops.parse_header(ta)
     ws = [ops.upload(torch.from_numpy(plane), ta, meta, "cuda") for _ in range(copies)]
-    desc = f"{ops.FORMAT_NAMES[fmt_out]} R={R}{' chunk-major' if cm else ''}{' wave64' if w64 else ''}"
+    desc = f"{ops.FORMAT_NAMES[fmt_out]} R={R}{' chunk-major' if cm else ''}{' wave64' if w64 else ''}{' tiles 32x256' if R == 32 else ''}"
     return ws, plane.size + aux.size, desc
 
 

@@ -33,64 +33,130 @@ __global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ 
 
 // Routing lists (reference mmid_helper.cu:48-136): block e lists the (token, slot) pairs of expert e in token order at
 // positions bounds[e].., where bounds[e] = number of pairs of experts < e.  ids element i of token t at byte
-// ids + (t * stride + i) * elem (low 32 bits are read).  Every thread owns a run of consecutive tokens: it counts its
-// pairs of lower experts and its own hits, one block-wide scan turns the hit counts into positions, and a second walk
-// over the run writes the lists.
-__global__ void __launch_bounds__(256) k_route(const char * __restrict__ ids, int elem, int64_t stride, int32_t * __restrict__ ids_src1,
-                                               int32_t * __restrict__ ids_dst, int32_t * __restrict__ bounds, int n_tok, int n_used,
-                                               int nchannels_y, int sis1) {
-    __shared__ int wave_hits[4], wave_lower[4];
-    const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int per = (n_tok + 255) / 256;
-    const int t_begin = tid * per < n_tok ? tid * per : n_tok, t_end = t_begin + per < n_tok ? t_begin + per : n_tok;
-    int lower = 0, hits = 0;
-    for (int t = t_begin; t < t_end; t++) {
-        bool hit = false;
+// ids + (t * stride + i) * elem (low 32 bits are read).  Thread i of a round takes token (round * 1024 + i), so a
+// wavefront reads adjacent tokens.  First the pairs of lower experts are counted; then, 64 rounds at a time, every
+// wavefront records how many of its tokens of a round use the expert, one wavefront turns the (round, wavefront)
+// counts into positions, and the tokens that hit write their pair at position + rank inside the wavefront.
+constexpr int ROUTE_THREADS = 1024, ROUTE_WAVES = ROUTE_THREADS / 64, ROUTE_ROUNDS = 64;
+
+// what the ids of one token say about expert e: how many are lower, and the last slot that names e (-1: none).
+// NU > 0: NU int32 ids per token in 16-byte aligned rows, read four at a time; NU = 0: any element size and count.
+template <int NU>
+__device__ __forceinline__ void token_ids(const char * __restrict__ ids, int elem, int64_t stride, int n_used, int t, int e, int & lower,
+                                          int & slot) {
+    if (NU > 0) {
+        const int4 * row = (const int4 *) (ids + (int64_t) t * stride * 4);
+#pragma unroll
+        for (int q = 0; q < NU / 4; q++) {
+            const int4 v = row[q];
+            const int a[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                lower += a[i] < e;
+                slot = a[i] == e ? 4 * q + i : slot;
+            }
+        }
+    } else {
         for (int k = 0; k < n_used; k++) {
             const int v = *(const int32_t *) (ids + ((int64_t) t * stride + k) * elem);
             lower += v < e;
-            hit |= v == e;
+            slot = v == e ? k : slot;
         }
-        hits += hit;
     }
-    // inclusive scan of the hit counts and sum of the lower counts inside the wavefront, then over the four wavefronts
-    int scan = hits;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const int up = __shfl_up(scan, o, 64);
-        scan += lane >= o ? up : 0;
+}
+
+template <int NU>
+__global__ void __launch_bounds__(ROUTE_THREADS) k_route(const char * __restrict__ ids, int elem, int64_t stride,
+                                                         int32_t * __restrict__ ids_src1, int32_t * __restrict__ ids_dst,
+                                                         int32_t * __restrict__ bounds, int n_tok, int n_used, int nchannels_y, int sis1) {
+    __shared__ int cnt[ROUTE_ROUNDS][ROUTE_WAVES];
+    __shared__ int wave_lower[ROUTE_WAVES];
+    __shared__ int chunk_total;
+    const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int lower = 0;
+#pragma unroll 4
+    for (int t = tid; t < n_tok; t += ROUTE_THREADS) {
+        int slot = -1;
+        token_ids<NU>(ids, elem, stride, n_used, t, e, lower, slot);
     }
 #pragma unroll
     for (int o = 32; o; o >>= 1) {
         lower += __shfl_xor(lower, o, 64);
     }
-    if (lane == 63) {
-        wave_hits[wave] = scan;
+    if (lane == 0) {
         wave_lower[wave] = lower;
     }
     __syncthreads();
-    const int base = wave_lower[0] + wave_lower[1] + wave_lower[2] + wave_lower[3];
-    int j = base + scan - hits;
-    for (int w2 = 0; w2 < wave; w2++) {
-        j += wave_hits[w2];
+    int base = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < ROUTE_WAVES; w2++) {
+        base += wave_lower[w2];
     }
-    for (int t = t_begin; t < t_end; t++) {
-        int slot = -1;
-        for (int k = 0; k < n_used; k++) {
-            if (*(const int32_t *) (ids + ((int64_t) t * stride + k) * elem) == e) {
-                slot = k; // a token lists an expert once; were it listed twice, the last slot counts
+    int done = 0; // pairs of this expert in the chunks before
+    for (int c0 = 0; c0 < n_tok; c0 += ROUTE_ROUNDS * ROUTE_THREADS) {
+        const int left = n_tok - c0;
+        const int rounds = left >= ROUTE_ROUNDS * ROUTE_THREADS ? ROUTE_ROUNDS : (left + ROUTE_THREADS - 1) / ROUTE_THREADS;
+        uint64_t mine = 0; // rounds in which this thread's token uses the expert
+#pragma unroll 4
+        for (int r = 0; r < rounds; r++) {
+            const int t = c0 + r * ROUTE_THREADS + tid;
+            int slot = -1, unused = 0;
+            if (t < n_tok) {
+                token_ids<NU>(ids, elem, stride, n_used, t, e, unused, slot);
+            }
+            const bool hit = slot >= 0;
+            mine |= (uint64_t) hit << r;
+            const uint64_t m = __ballot(hit);
+            if (lane == 0) {
+                cnt[r][wave] = (int) __builtin_popcountll(m);
             }
         }
-        if (slot >= 0) {
-            ids_dst[j] = t * n_used + slot;
-            ids_src1[j] = t * sis1 + slot % nchannels_y;
-            j++;
+        __syncthreads();
+        if (wave == 0) { // exclusive prefix over (round, wavefront) in that order; lane r owns round r
+            int row = 0;
+            if (lane < rounds) {
+                for (int w2 = 0; w2 < ROUTE_WAVES; w2++) {
+                    const int v = cnt[lane][w2];
+                    cnt[lane][w2] = row;
+                    row += v;
+                }
+            }
+            int scan = row;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(scan, o, 64);
+                scan += lane >= o ? up : 0;
+            }
+            if (lane < rounds) {
+                for (int w2 = 0; w2 < ROUTE_WAVES; w2++) {
+                    cnt[lane][w2] += scan - row;
+                }
+            }
+            if (lane == 63) {
+                chunk_total = scan;
+            }
         }
+        __syncthreads();
+        for (int r = 0; r < rounds; r++) {
+            const bool hit = (mine >> r) & 1;
+            const uint64_t m = __ballot(hit);
+            if (hit) {
+                const int t = c0 + r * ROUTE_THREADS + tid;
+                int slot = -1, unused = 0; // a token lists an expert once; were it listed twice, the last slot counts
+                token_ids<NU>(ids, elem, stride, n_used, t, e, unused, slot);
+                const int rank = (int) __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
+                const int j = base + done + cnt[r][wave] + rank;
+                ids_dst[j] = t * n_used + slot;
+                ids_src1[j] = t * sis1 + slot % nchannels_y;
+            }
+        }
+        done += chunk_total;
+        __syncthreads(); // cnt and chunk_total are rewritten by the next chunk
     }
     if (tid == 0) {
         bounds[e] = base;
         if (e == (int) gridDim.x - 1) {
-            bounds[gridDim.x] = base + wave_hits[0] + wave_hits[1] + wave_hits[2] + wave_hits[3];
+            bounds[gridDim.x] = base + done;
         }
     }
 }
@@ -169,8 +235,14 @@ void launch_moe_combine(const float * ys, const void * w, bool w_bf16, void * y,
 
 void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds,
                   int n_experts, int n_tok, int n_used, int nchannels_y, int sis1, hipStream_t stream) {
-    hipLaunchKernelGGL(k_route, dim3(n_experts), dim3(256), 0, stream, (const char *) ids, ids_i64 ? 8 : 4, ids_row_stride, ids_src1,
-                       ids_dst, bounds, n_tok, n_used, nchannels_y, sis1);
+    const bool rows_of_8 = !ids_i64 && n_used == 8 && ids_row_stride % 4 == 0 && ((uintptr_t) ids & 15) == 0;
+    if (rows_of_8) { // top-8 routing with int32 ids: vector loads
+        hipLaunchKernelGGL(k_route<8>, dim3(n_experts), dim3(ROUTE_THREADS), 0, stream, (const char *) ids, 4, ids_row_stride, ids_src1,
+                           ids_dst, bounds, n_tok, n_used, nchannels_y, sis1);
+    } else {
+        hipLaunchKernelGGL(k_route<0>, dim3(n_experts), dim3(ROUTE_THREADS), 0, stream, (const char *) ids, ids_i64 ? 8 : 4, ids_row_stride,
+                           ids_src1, ids_dst, bounds, n_tok, n_used, nchannels_y, sis1);
+    }
 }
 
 void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,

@@ -24,7 +24,8 @@ int main() {
             w[(rnd() % rows) * K + rnd() % K] = special[i];
         }
         impl::encode(w.data(), rows, K, FMT_NIBBLE, 0, 0);
-        done++;
+        impl::encode(w.data(), rows, K, FMT_HUFPAIR, 32, FLAG_WAVE64); // 32 x 256 tiles
+        done += 2;
         for (int R : {1, 2, 4, 8, 16}) {
             impl::encode(w.data(), rows, K, FMT_HUFFMAN, R, 0);
             impl::encode(w.data(), rows, K, FMT_HUFPAIR, R, 0);
@@ -47,7 +48,10 @@ int main() {
             w[i + 1] = (uint16_t) ((60 + p / 70) << 7);
         }
         const auto e = impl::encode(w.data(), 16, 1024, FMT_HUFPAIR, 8, 0);
-        std::printf("fallback format %d\n", e.format);
+        std::vector<uint16_t> w2(w);
+        w2.insert(w2.end(), w.begin(), w.end());
+        const auto t = impl::encode(w2.data(), 32, 1024, FMT_HUFPAIR, 32, FLAG_WAVE64); // tiles fall back the same way
+        std::printf("fallback format %d, tiles %d R %d\n", e.format, t.format, t.R);
     }
     int thrown = 0;
     const std::vector<uint16_t> w(16 * 512);

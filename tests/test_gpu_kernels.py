@@ -203,7 +203,8 @@ def test_swiglu_and_combine(ops, oracle):
     assert np.array_equal(got, oracle.moe_combine(ys, wt16.float().cpu().numpy()))
 
 
-@pytest.mark.parametrize("T,k,E", [(1, 8, 256), (9, 8, 256), (130, 8, 64), (33, 3, 7), (2048, 8, 256)])
+@pytest.mark.parametrize("T,k,E", [(1, 8, 256), (9, 8, 256), (130, 8, 64), (33, 3, 7), (2048, 8, 256), (1024, 4, 32), (1025, 4, 32),
+                                   (8192, 8, 256), (70001, 2, 16)])  # the last one: more than one chunk of 64 rounds
 @pytest.mark.parametrize("idt", [torch.int32, torch.int64])
 def test_routing_lists(ops, oracle, T, k, E, idt):
     rng = np.random.default_rng(T + k)

@@ -21,5 +21,5 @@ def test_host_encoder_under_asan_ubsan(tmp_path):
     env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=1")
     r = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert "fallback format 2" in r.stdout
+    assert "fallback format 2, tiles 2 R 16" in r.stdout
     assert "thrown 6" in r.stdout and "encoded " in r.stdout
