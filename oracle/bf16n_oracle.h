@@ -14,6 +14,10 @@
  *       a case while cost, Kraft sum and decoded weights never do (tests state which comparison they use).
  *   orc_decode   against the reference encoder's output (decode(encode(w)) == w for every format/layout, special BF16
  *       classes included) and the golden fixtures.
+ *   orc_decode_w64 (this build's layout, no reference counterpart)   decode(encode(w)) == w, equality with orc_decode of
+ *       the reference layout of the same tensor, and — for the R = 32 tile form — the tile mapping restated in numpy from
+ *       its definition (tests/test_encoder_host.py: the permuted matrix encodes to the same plane and stream; a lane's 16
+ *       weights of a step are two runs of 8 consecutive columns of one row).
  *   orc_gemv_*   against numpy float64 on exact weights (bound 1e-5 * sum|w x|) and one-hot known answers.
  *   orc_route    against a brute-force stable sort of (expert, token) pairs.
  *   orc_router_topk   no counterpart in the reference core (engine op): pinned by closed forms only (softmax sums to 1,
