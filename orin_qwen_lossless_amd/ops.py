@@ -394,9 +394,10 @@ def mm_ids_route(topk_ids: torch.Tensor, n_experts: int, per_slot: bool):
 
 
 def moe_mm_ids(x: torch.Tensor, topk_ids: torch.Tensor, w: Weight, n_experts: int, up: Weight | None = None,
-               out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+               out_dtype: torch.dtype = torch.float32, routes=None) -> torch.Tensor:
     """Batched MUL_MAT_ID over routed tokens (core/torch/torch_bindings.cpp:307-345): x [T, K] (gate / up) or
-    [T, n_used, K] (down), BF16; out [T, n_used, N]; up given: fused gate/up + SwiGLU."""
+    [T, n_used, K] (down), BF16; out [T, n_used, N]; up given: fused gate/up + SwiGLU.  routes: the lists of
+    mm_ids_route(topk_ids, n_experts, x.dim() == 3) if the caller already has them (they are computed otherwise)."""
     cw = _cweight(w)
     cu = _cweight(up) if up is not None else None
     _check_ids(topk_ids)
@@ -416,7 +417,7 @@ def moe_mm_ids(x: torch.Tensor, topk_ids: torch.Tensor, w: Weight, n_experts: in
     L = _lib.lib()
     if not L.bf16n_mm_ids_supported(C.byref(cw), C.byref(cu) if cu is not None else None):
         raise ValueError("bf16n.moe_mm_ids: no batched kernel for this matrix (format/K/R/layout)")
-    src1, dst, bounds = mm_ids_route(topk_ids, n_experts, per_slot)
+    src1, dst, bounds = routes if routes is not None else mm_ids_route(topk_ids, n_experts, per_slot)
     with torch.cuda.device(x.device):
         _lib.check(L.bf16n_mm_ids(C.byref(cw), C.byref(cu) if cu is not None else None, x.data_ptr(), w.meta.K,
                                   src1.data_ptr(), dst.data_ptr(), bounds.data_ptr(), y.data_ptr(),
@@ -482,8 +483,11 @@ def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_we
     H = down.meta.rows // n_experts
     x = x.contiguous()
     if T > GEMV_MAX_TOKENS and mm_ids_supported(gate, up) and mm_ids_supported(down):
-        a = moe_mm_ids(x, topk_ids, gate, n_experts, up=up, out_dtype=torch.bfloat16)
-        ys = moe_mm_ids(a, topk_ids, down, n_experts, out_dtype=torch.float32)
+        # one routing pass for both products: with one activation row per (token, slot), as down takes them, the
+        # source row of a pair is its destination row
+        src1, dst, bounds = mm_ids_route(topk_ids, n_experts, False)
+        a = moe_mm_ids(x, topk_ids, gate, n_experts, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
+        ys = moe_mm_ids(a, topk_ids, down, n_experts, out_dtype=torch.float32, routes=(dst, dst, bounds))
     elif glu2_supported(gate, up):
         ys = mmv(mmv_glu2(x, gate, up, topk_ids, N), down, topk_ids, H)
     else:
