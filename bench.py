@@ -289,6 +289,43 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
     return out
 
 
+def prefill_only(T: int, steps: int) -> None:
+    """Only the batched MoE kernels of one 35B-A3B-shaped layer (256 experts x (gate, up 512 x 2048; down 2048 x 512),
+    top-8, experts in the mi355x policy's layout) on T tokens: routing lists once, then fused gate/up + SwiGLU (BF16)
+    and down, `steps` times.  For profiling these kernels alone; prints its own JSON line."""
+    import numpy as np
+    import torch
+
+    from orin_qwen_lossless_amd import ops
+
+    torch.cuda.set_device(0)
+    ops.init()
+    E, topk, N, K = 256, 8, 512, 2048
+    g = torch.Generator(device="cuda").manual_seed(3)
+
+    def randw(rows, k):
+        return (torch.randn((rows, k), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+
+    (gate,), _, gdesc = encode_to_device(ops, randw(E * N, K), n_matrices=E)
+    (up,), _, _ = encode_to_device(ops, randw(E * N, K), n_matrices=E)
+    (down,), _, ddesc = encode_to_device(ops, randw(E * K, N), n_matrices=E)
+    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
+    _, ids = ops.router_topk(torch.randn((T, E), generator=g, device="cuda"), topk)
+    src1, dst, bounds = ops.mm_ids_route(ids, E, False)
+
+    def gate_up(i):
+        return ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
+
+    a = gate_up(0)
+    t_gu = med_us(gate_up, steps, 2)
+    t_dn = med_us(lambda i: ops.moe_mm_ids(a, ids, down, E, routes=(dst, dst, bounds)), steps, 2)
+    flops_gu, flops_dn = 2.0 * T * topk * 2 * N * K, 2.0 * T * topk * K * N
+    print(json.dumps({"workload": f"MoE prefill, {T} tokens, top-{topk} of {E} experts", "gate_up": gdesc, "down": ddesc,
+                      "gate_up_us": round(t_gu, 1), "down_us": round(t_dn, 1),
+                      "gate_up_TFLOPs": round(flops_gu / t_gu / 1e6, 1), "down_TFLOPs": round(flops_dn / t_dn / 1e6, 1),
+                      "frac_of_bf16_mfma_peak": round((flops_gu + flops_dn) / (t_gu + t_dn) / 1e6 / 2500.0, 4)}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -300,9 +337,14 @@ def main() -> None:
     ap.add_argument("--cpu-rows", type=int, default=16384)
     ap.add_argument("--no-graph", action="store_true", help="time the steps as separate launches instead of one HIP graph replay")
     ap.add_argument("--suite", action="store_true", help="also time batch 4, the NIBBLE matrices, a MoE layer and the prefill")
+    ap.add_argument("--prefill", type=int, default=0, metavar="T",
+                    help="run only the batched MoE kernels of one layer on T tokens (for profiling) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path has no collective); run with --gpus 1")
+    if args.prefill > 0:
+        prefill_only(args.prefill, min(args.steps, 20))
+        return
 
     import numpy as np
     import torch
