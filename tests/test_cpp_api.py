@@ -43,3 +43,16 @@ def test_cpp_api_on_the_device(tmp_path):
     assert "encoded format 3 R 4 flags 4" in out       # 4096 x 2048 under the mi355x policy: wave64 units of 4 rows
     assert "dequant ok" in out and "mmv ok" in out
     assert "invalid_argument bf16n: dequant rows must be whole units" in out
+
+
+@pytest.mark.gpu
+def test_cpp_api_moe_layer_on_the_device(tmp_path):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    exe = str(tmp_path / "gpu_moe")
+    subprocess.run([hipcc, "-std=c++17", "-O2", "--offload-arch=gfx950", "-I" + os.path.join(ROOT, "include"),
+                    os.path.join(ROOT, "tests", "cpp", "gpu_moe.cpp"), "-o", exe, "-L" + LIBDIR, "-lbf16n_hip", "-Wl,-rpath," + LIBDIR],
+                   check=True, capture_output=True, timeout=300)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=120).stdout
+    assert "experts R 32 32 flags 4 4" in out          # the mi355x policy: 32 x 256 tiles for experts
+    assert "mm_ids_supported 1 1" in out
+    assert "batched ok" in out and "gemv ok" in out, out
