@@ -299,6 +299,10 @@ template <> struct x8<float> {
 };
 
 constexpr int TV_WAVES = 16;
+// wavefronts per block: 16 (128 registers each) where gate and up run on separate wavefronts with BF16 activations,
+// else 8 (FP32 activations take twice the registers)
+template <typename TX, bool GLU>
+constexpr int tv_max_waves() { return GLU && sizeof(TX) == 2 ? TV_WAVES : TV_WAVES / 2; }
 
 // A block covers `gpb` row groups of one column.  Each wavefront runs one decode chain — `upw` consecutive tiles of
 // one matrix (at decode a launch is a few hundred tiles and its time is the length of a chain: one short chain per
@@ -306,7 +310,7 @@ constexpr int TV_WAVES = 16;
 // are added in tile order.  GLU: the group has wpg wavefronts on the gate matrix and wpg on the up matrix, and the
 // block writes silu(gate x) * (up x).
 template <typename TX, bool GLU>
-__global__ void __launch_bounds__(GLU ? TV_WAVES * 64 : TV_WAVES * 32) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw) {
+__global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw) {
     constexpr int NM = GLU ? 2 : 1;
     __shared__ __align__(16) uint32_t lut[NM * LUT_WORDS];
     __shared__ float part[TV_WAVES][32];
@@ -341,12 +345,19 @@ __global__ void __launch_bounds__(GLU ? TV_WAVES * 64 : TV_WAVES * 32) k_tile_mm
 #pragma unroll
                 for (int s = 0; s < 4; s++) {
                     const int kk = k0 + 32 * (4 * hh + s);
+                    // BF16 activations (8 registers a step) are requested before the decode, FP32 ones (16) after it
                     x8<TX> xa, xb;
-                    xa.load(cv.x, kk);
-                    xb.load(cv.x, kk + 16);
+                    if (sizeof(TX) == 2) {
+                        xa.load(cv.x, kk);
+                        xb.load(cv.x, kk + 16);
+                    }
                     uint32_t wp[1][8];
                     tile_step<1>(ch, my_lut, 0, s, wp);
                     ch[0].reload(s, lane);
+                    if (sizeof(TX) != 2) {
+                        xa.load(cv.x, kk);
+                        xb.load(cv.x, kk + 16);
+                    }
                     acc = xb.dot(wp[0] + 4, xa.dot(wp[0], acc));
                 }
             }
@@ -480,8 +491,14 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
 // y = W x (up == nullptr) or silu(gate x) * (up x), one column per launch row
 void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols & p, int ncols, bool x_bf16, hipStream_t stream) {
     const int slabs = (int) (w.K / TILE_K);
-    // wavefronts per row group and matrix: one per tile up to 8 tiles (K <= 2048), two tiles each beyond
-    const int wpg = slabs <= 8 ? slabs : (slabs + 1) / 2, upw = slabs / wpg, wpgm = wpg * (up ? 2 : 1);
+    // wavefronts per row group and matrix: one per tile where the block has room for them, else the fewest tiles per
+    // wavefront that fit
+    const int nm = up ? 2 : 1, max_waves = up && x_bf16 ? TV_WAVES : TV_WAVES / 2;
+    int upw = 1;
+    while (slabs % upw != 0 || slabs / upw * nm > max_waves) {
+        upw++;
+    }
+    const int wpg = slabs / upw, wpgm = wpg * nm;
     // blocks of four wavefronts where a row group takes at most four: more, smaller blocks spread a routed GEMV (a
     // few hundred tiles) over more compute units
     const int waves = wpgm <= 4 ? 4 : wpgm <= 8 ? 8 : TV_WAVES, gpb = waves / wpgm;
