@@ -275,9 +275,10 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
         wts, ids = ops.router_topk(lg, topk)
         for engine, (gate, up, gdesc) in pairs.items():
 
-            def prefill(i):
-                a = ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16)
-                return ops.moe_mm_ids(a, ids, down, E)
+            def prefill(i):  # as ops.moe_experts does it: one routing pass, fused gate/up + SwiGLU (BF16), down
+                src1, dst, bounds = ops.mm_ids_route(ids, E, False)
+                a = ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
+                return ops.moe_mm_ids(a, ids, down, E, routes=(dst, dst, bounds))
 
             t = med_us(prefill, 10, 2)
             t_gu = med_us(lambda i: ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16), 10, 2)
