@@ -69,3 +69,63 @@ def test_full_size_product_within_fp64_bound(ops, head):
         assert bool((err[keep] <= 1e-5 * bound[keep]).all())
     # batch columns equal single-column launches bit for bit (compared as bits: one row is NaN)
     assert torch.equal(ops.mmv(x[1:2], enc)[0].view(torch.int32), y[1].view(torch.int32))
+
+
+# ---- one MoE layer of the 35B-A3B shape at its real size: 256 experts x (gate, up 512 x 2048; down 2048 x 512) -----------
+
+E, TOPK, N = 256, 8, 512
+
+
+@pytest.fixture(scope="module")
+def experts(ops):
+    g = torch.Generator(device="cuda").manual_seed(11)
+
+    def make(rows_per, k):
+        w = (torch.randn((E * rows_per, k), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+        fmt, R, cm, _, w64 = ops.choose(rows_per, k, E, engine="mi355x", expert=True)
+        assert (fmt, R, w64) == (3, 32, True)                # 32 x 256 tiles
+        plane, aux, _, _ = ops.encode_bits(w.cpu().view(torch.int16).numpy().view(np.uint16), fmt, R, cm, wave64=w64)
+        ta = torch.from_numpy(aux)
+        return w, ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
+
+    return make(N, K), make(N, K), make(K, N)
+
+
+def test_full_size_experts_round_trip(ops, experts):
+    for w, enc in experts:
+        assert ops.roundtrip_equal(enc, w)
+
+
+def test_full_size_batched_moe_against_exact_weights_and_the_gemv_path(ops, experts):
+    (wg, gate), (wu, up), (wd, down) = experts
+    T = 1024                                                   # 8192 routed pairs, about 32 per expert
+    g = torch.Generator(device="cuda").manual_seed(12)
+    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
+    wts, ids = ops.router_topk(torch.randn((T, E), generator=g, device="cuda"), TOPK)
+    src1, dst, bounds = ops.mm_ids_route(ids, E, False)
+    b = bounds.cpu().numpy()
+    assert b[0] == 0 and b[-1] == T * TOPK and np.all(np.diff(b) >= 0)
+    # routing lists: a permutation of the pairs, sorted by expert, tokens in order inside an expert
+    d = dst.cpu().numpy()
+    assert np.array_equal(np.sort(d), np.arange(T * TOPK))
+    flat = ids.cpu().numpy().reshape(-1)
+    assert np.all(np.diff(flat[d]) >= 0)
+    a = ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.float32, routes=(src1, dst, bounds))
+    # sampled tokens against FP64 products with the exact weights of their experts
+    for t in (0, 1, 511, T - 1):
+        for s in range(TOPK):
+            e = int(ids[t, s])
+            xe = x[t].double()
+            gg, uu = wg[e * N:(e + 1) * N].double() @ xe, wu[e * N:(e + 1) * N].double() @ xe
+            want = uu * (gg / (1.0 + torch.exp(-gg)))
+            assert torch.all((a[t, s].double() - want).abs() <= 1e-3 * want.abs() + 1e-5), (t, s)
+    # the batched kernel and the routed GEMV (decode path) agree on the first tokens; so do the down products
+    a8 = ops.mmv_glu2(x[:8], gate, up, ids[:8].contiguous(), N)
+    assert torch.all((a8 - a[:8]).abs() <= 1e-3 * a[:8].abs() + 1e-5)
+    a16 = a.to(torch.bfloat16)
+    ys = ops.moe_mm_ids(a16, ids, down, E, routes=(dst, dst, bounds))
+    y8 = ops.mmv(a16[:8].float(), down, ids[:8].contiguous(), K)
+    assert torch.all((y8 - ys[:8]).abs() <= 1e-3 * ys[:8].abs() + 1e-5)
+    # linearity in the activations: doubling them doubles every product exactly (powers of two commute with rounding)
+    ys2 = ops.moe_mm_ids((a16.float() * 2).to(torch.bfloat16), ids, down, E, routes=(dst, dst, bounds))
+    assert torch.equal(ys2, ys * 2)
