@@ -215,8 +215,16 @@ __device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uin
 
 // NCH = 2: a wave splits its units into two halves decoded as two interleaved chains (twice the independent work per
 // wave to cover LDS latency); NCH = 1 where a wave has a single unit.
+// activation registers per lane of an instance (BF16: 8 per 512-column chunk set and column, FP32: 16)
+template <typename TX, int C, int NC>
+constexpr int x_regs() { return NC * geom<C>::XS * (sizeof(TX) == 2 ? 8 : 16); }
+
+// instances that need more than 128 registers per lane: more than 64 of activations, or 64 with FP32 activations or
+// eight chunks per row (they spilled at 128); these run in blocks of at most eight wavefronts
+constexpr bool wide_regs(int xr, bool x_bf16, int C) { return xr > 64 || (xr == 64 && (!x_bf16 || C == 8)); }
+
 template <typename TX, int C, int NC, int NCH>
-__global__ void __launch_bounds__(1024) k_w64_mmv(const bf16n_weight w, const cols p, int units_per_wave) {
+__global__ void __launch_bounds__(wide_regs(x_regs<TX, C, NC>(), sizeof(TX) == 2, C) ? 512 : 1024) k_w64_mmv(const bf16n_weight w, const cols p, int units_per_wave) {
     using G = geom<C>;
     constexpr int K = C * CHUNK;
     __shared__ __align__(16) uint32_t lut[LUT_WORDS];          // static: sits at LDS address 0
@@ -388,15 +396,15 @@ size_t w64_shm(int waves) { return (size_t) waves * WAVE_LDS_WORDS * 4; } // dyn
 
 // waves per block and units per wave for `units` units per column: every wave gets the same number of units (but the
 // last), and a launch fills the device once when it can
-void w64_dims(int64_t units, int ncols, int cus, int & waves_per_block, int & blocks, int & units_per_wave) {
-    int64_t max_waves = (int64_t) cus * 16 / (ncols < 1 ? 1 : ncols);
+void w64_dims(int64_t units, int ncols, int cus, int & waves_per_block, int & blocks, int & units_per_wave, int waves_per_cu = 16) {
+    int64_t max_waves = (int64_t) cus * waves_per_cu / (ncols < 1 ? 1 : ncols);
     max_waves = max_waves < 16 ? 16 : max_waves;
     int64_t upw = (units + max_waves - 1) / max_waves;
     if (upw > 1 && (upw & 1)) {
         upw++; // two chains per wave: an even split
     }
     const int64_t waves = (units + upw - 1) / upw;
-    waves_per_block = waves >= 8 * (int64_t) cus ? 8 : 4;
+    waves_per_block = waves >= 8 * (int64_t) cus && waves_per_cu != 12 ? 8 : 4;
     if (waves < waves_per_block) {
         waves_per_block = (int) waves;
     }
@@ -404,25 +412,29 @@ void w64_dims(int64_t units, int ncols, int cus, int & waves_per_block, int & bl
     units_per_wave = (int) upw;
 }
 
-// columns that share one decode: as many (up to 4) as keep the activations within 64 registers per lane
+// columns that share one decode (reference launch.cu:174-193 groups four; its eight-column kernels are
+// kernels.cuh:2002-2104).  Up to 64 activation registers per lane an instance runs sixteen wavefronts per CU; up to 128
+// (five to eight BF16 columns at K <= 2048, three or four at K = 4096, ...) eight to twelve wavefronts of up to 256
+// registers: a lower decode rate, but one pass over the matrix instead of two.
 template <typename TX, int C>
 constexpr int max_group() {
-    constexpr int per_col = geom<C>::XS * (sizeof(TX) == 2 ? 8 : 16);
-    return 64 / per_col < 1 ? 1 : 64 / per_col > 4 ? 4 : 64 / per_col;
+    constexpr int per_col = x_regs<TX, C, 1>();
+    return 128 / per_col < 1 ? 1 : 128 / per_col > 8 ? 8 : 128 / per_col;
 }
-
 // two decode chains per wave only where the activations leave room for them in 128 registers (the instances with
 // more activation registers would spill; they run one chain per wave)
 template <typename TX, int C, int NC>
-constexpr bool two_chains() { return NC * geom<C>::XS * (sizeof(TX) == 2 ? 8 : 16) <= 16; }
+constexpr bool two_chains() { return x_regs<TX, C, NC>() <= 16; }
 
 template <typename TX, int C, int NC>
 void mmv_launch(dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
-    if (upw >= 2 && two_chains<TX, C, NC>()) {
-        hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 2>), grid, dim3(nt), w64_shm(2 * wpb), stream, w, p, upw);
-    } else {
-        hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 1>), grid, dim3(nt), w64_shm(wpb), stream, w, p, upw);
+    if constexpr (two_chains<TX, C, NC>()) {
+        if (upw >= 2) {
+            hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 2>), grid, dim3(nt), w64_shm(2 * wpb), stream, w, p, upw);
+            return;
+        }
     }
+    hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 1>), grid, dim3(nt), w64_shm(wpb), stream, w, p, upw);
 }
 
 template <typename TX, int C>
@@ -434,8 +446,16 @@ void mmv_nc(int nc, dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_
         if constexpr (G >= 2) mmv_launch<TX, C, 2>(grid, nt, wpb, stream, w, p, upw);
     } else if (nc == 3) {
         if constexpr (G >= 3) mmv_launch<TX, C, 3>(grid, nt, wpb, stream, w, p, upw);
-    } else {
+    } else if (nc == 4) {
         if constexpr (G >= 4) mmv_launch<TX, C, 4>(grid, nt, wpb, stream, w, p, upw);
+    } else if (nc == 5) {
+        if constexpr (G >= 8) mmv_launch<TX, C, 5>(grid, nt, wpb, stream, w, p, upw);
+    } else if (nc == 6) {
+        if constexpr (G >= 8) mmv_launch<TX, C, 6>(grid, nt, wpb, stream, w, p, upw);
+    } else if (nc == 7) {
+        if constexpr (G >= 8) mmv_launch<TX, C, 7>(grid, nt, wpb, stream, w, p, upw);
+    } else {
+        if constexpr (G >= 8) mmv_launch<TX, C, 8>(grid, nt, wpb, stream, w, p, upw);
     }
 }
 
@@ -458,11 +478,16 @@ template <typename TX, int C, int NC>
 void set_attr() {
     if constexpr (NC <= max_group<TX, C>()) {
         (void) hipFuncSetAttribute((const void *) k_w64_mmv<TX, C, NC, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(16));
-        (void) hipFuncSetAttribute((const void *) k_w64_mmv<TX, C, NC, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(32));
+        if constexpr (two_chains<TX, C, NC>()) {
+            (void) hipFuncSetAttribute((const void *) k_w64_mmv<TX, C, NC, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) w64_shm(32));
+        }
     }
 }
 template <typename TX, int C>
-void set_attr_nc() { set_attr<TX, C, 1>(); set_attr<TX, C, 2>(); set_attr<TX, C, 3>(); set_attr<TX, C, 4>(); }
+void set_attr_nc() {
+    set_attr<TX, C, 1>(); set_attr<TX, C, 2>(); set_attr<TX, C, 3>(); set_attr<TX, C, 4>();
+    set_attr<TX, C, 5>(); set_attr<TX, C, 6>(); set_attr<TX, C, 7>(); set_attr<TX, C, 8>();
+}
 template <typename TX>
 void set_attr_c() { set_attr_nc<TX, 1>(); set_attr_nc<TX, 2>(); set_attr_nc<TX, 4>(); set_attr_nc<TX, 8>(); }
 
@@ -496,8 +521,7 @@ bool w64_mmv_supported(const bf16n_weight & w, bool) {
 void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf16, bool multi_col, int cus, hipStream_t stream) {
     const int C = (int) (w.K / CHUNK);
     const int64_t units = p.nrows / w.R;
-    // dense batches: groups of up to 4 columns share one decode (reference launch.cu:174-193), fewer where the
-    // activations of 4 columns would not fit in 64 registers per lane
+    // dense batches: groups of columns share one decode (max_group)
     const int group_max = !multi_col || p.ids ? 1 : x_bf16 ? group_for<bf16_t>(C) : group_for<float>(C);
     for (int c0 = 0; c0 < (group_max == 1 ? 1 : ncols); c0 += group_max) {
         const int nc = group_max == 1 ? 1 : (ncols - c0 < group_max ? ncols - c0 : group_max);
@@ -508,7 +532,10 @@ void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf
             q.y += c0 * p.y_tok;
         }
         int wpb, blocks, upw;
-        w64_dims(units, ny, cus, wpb, blocks, upw);
+        // wavefronts per CU the instance is sized for, by its activation registers (x_regs): 16 up to 64 registers,
+        // then three per SIMD in blocks of four, two per SIMD beyond 112
+        const int xr = nc * (C >= 2 ? C / 2 : 1) * (x_bf16 ? 8 : 16);
+        w64_dims(units, ny, cus, wpb, blocks, upw, !wide_regs(xr, x_bf16, C) ? 16 : xr <= 112 ? 12 : 8);
         const dim3 grid(blocks, ny);
         if (x_bf16) {
             mmv_c<bf16_t>(C, nc, grid, wpb * 64, wpb, stream, w, q, upw);

@@ -59,6 +59,29 @@ def test_gemv_dense(ops, oracle, K, fmt, R, cm, w64):
     assert np.array_equal(y_sc, y_bf)
 
 
+@pytest.mark.parametrize("K", [512, 1024, 2048, 4096])
+@pytest.mark.parametrize("R", [1, 4, 16])
+def test_wave64_column_groups_equal_single_columns(ops, oracle, K, R):
+    # one decode serves a group of up to eight token columns (fewer when K is large or the activations are FP32);
+    # every batch size gives each column the bits of its single-column launch, which the oracle bounds
+    if R * K % (4096 if K == 4096 else 2048):
+        pytest.skip("the GEMV takes units of whole pairs (K = 4096: quadruples) of 1024-column steps")
+    rows = 16 * 37
+    wb = synth.weights(rows, K, 3 * K + R)
+    w = enc(ops, wb, HP, R, False, True)
+    xb = synth.activations(8, K, K + 11)
+    xf = synth.bf16_bits_to_f32(xb)
+    for x in (tbf16(xb), torch.from_numpy(xf).cuda()):
+        y1 = torch.cat([ops.mmv(x[t: t + 1], w) for t in range(8)])
+        check_gemv(oracle, y1.cpu().numpy(), wb, xf)
+        for T in range(2, 9):
+            assert torch.equal(ops.mmv(x[:T], w), y1[:T]), (T, x.dtype)
+        # strided activation rows (a view of a wider buffer)
+        wide = torch.zeros((8, K + 64), dtype=x.dtype, device="cuda")
+        wide[:, :K] = x
+        assert torch.equal(ops.mmv(wide[:, :K], w), y1)
+
+
 @pytest.mark.parametrize("fmt,R,cm,w64", LAYOUTS)
 def test_one_hot_activations_give_exact_weights(ops, fmt, R, cm, w64):
     K, rows = 2048, 64
