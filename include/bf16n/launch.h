@@ -63,6 +63,15 @@ inline void init() { detail::check(bf16n_init()); }
 inline int sm_count() { int n = 0; detail::check(bf16n_cu_count(&n)); return n; } // compute units of the device
 inline int cu_count() { return sm_count(); }
 
+// BF16 token columns up to which mmv is the faster dense path for this matrix; beyond it: dequant + a stock GEMM.
+// (8 in the reference, fixed: core/torch/torch_bindings.cpp:195.)
+inline int gemv_max_tokens(const weight & w) {
+    const bf16n_weight cw = detail::c_view(w);
+    int n = 0;
+    detail::check(bf16n_gemv_max_tokens(&cw, &n));
+    return n;
+}
+
 inline void mmv(const weight & w, const mmv_args & a, hipStream_t stream, bool multi_col = true) {
     const bf16n_weight cw = detail::c_view(w);
     const bf16n_mmv_args ca = detail::c_args(a);

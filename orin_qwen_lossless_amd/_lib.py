@@ -41,6 +41,7 @@ SYMBOLS = {
     "bf16n_init": (_i, []),
     "bf16n_cu_count": (_i, [C.POINTER(_i)]),
     "bf16n_mmv": (_i, [_WP, _AP, _vp, _i]),
+    "bf16n_gemv_max_tokens": (_i, [_WP, C.POINTER(_i)]),
     "bf16n_mmv_glu": (_i, [_WP, _AP, _vp]),
     "bf16n_mmv_glu2": (_i, [_WP, _WP, _AP, _vp]),
     "bf16n_dequant": (_i, [_WP, _i64, _i64, _vp, _vp]),

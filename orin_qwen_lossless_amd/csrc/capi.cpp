@@ -98,6 +98,16 @@ dev::cols make_cols(const bf16n_mmv_args & a) { // launch.cu:69-84
     return p;
 }
 
+// dense products of a tile-layout matrix that go through the matrix cores: BF16 activations, rows enough to fill the
+// GPU, and the 16-byte alignment of x rows and y columns that the kernel's vector accesses need
+bool tile_dense_mm(const bf16n_weight & w, const bf16n_mmv_args & a) {
+    if (a.ids || !a.x_bf16 || !dev::tile_mm_dense_pays(w, a.nrows, g_cus)) {
+        return false;
+    }
+    const int64_t ya = a.y_bf16 ? 8 : 16;
+    return ((uintptr_t) a.x & 15) == 0 && ((uintptr_t) a.y & 15) == 0 && (a.ncols == 1 || (a.x_tok % 16 == 0 && a.y_tok % ya == 0));
+}
+
 void launch_check(const char * what) { hip_check(hipGetLastError(), what); }
 
 } // namespace
@@ -175,7 +185,11 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
             return;
         }
         const dev::cols p = make_cols(*a);
-        if (dev::is_tile_layout(*w)) {
+        if (dev::is_tile_layout(*w) && tile_dense_mm(*w, *a)) {
+            // a large dense matrix, BF16 activations: any number of columns through the matrix cores
+            dev::launch_tile_mm_dense(*w, a->row0, a->nrows, a->x, a->x_tok / 2, a->ncols, a->y, a->y_bf16 != 0,
+                                      a->y_tok / (a->y_bf16 ? 2 : 4), g_cus, (hipStream_t) stream);
+        } else if (dev::is_tile_layout(*w)) {
             dev::launch_tile_mmv(*w, nullptr, p, a->ncols, a->x_bf16 != 0, (hipStream_t) stream);
         } else if (is_w64(*w)) {
             require(dev::w64_mmv_supported(*w, a->x_bf16 != 0), "no wave64 GEMV kernel for this K / R (K in {512, 1024, 2048, 4096})");
@@ -184,6 +198,18 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
             dev::launch_compat_mmv(*w, nullptr, 0, p, a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
         }
         launch_check("mmv");
+    });
+}
+
+// The number of BF16 token columns up to which bf16n_mmv is the faster dense path; beyond it dequant + a stock GEMM is.
+// 8 is the reference's fixed rule (core/torch/torch_bindings.cpp:195); matrices whose products run on the matrix cores
+// stay ahead for far longer (every pass of up to 128 columns decodes the matrix once).
+int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(out != nullptr, "null output");
+        *out = dev::is_tile_layout(*w) && dev::tile_mm_dense_pays(*w, w->rows, g_cus) ? 256 : 8;
     });
 }
 
@@ -315,8 +341,8 @@ int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x
         require(((uintptr_t) x_bf16 & 15) == 0 && x_row % 8 == 0, "activations must be 16-byte aligned with 16-byte row strides");
         require(((uintptr_t) dst & 15) == 0 && dst_col % 4 == 0, "dst must be 16-byte aligned with a column stride that is a multiple of 4");
         if (dev::is_tile_layout(*w)) {
-            dev::launch_tile_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, g_cus,
-                                    (hipStream_t) stream);
+            dev::launch_tile_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts,
+                                    (int64_t) n_tok * n_used, g_cus, (hipStream_t) stream);
         } else {
             dev::launch_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, n_tok, n_used,
                                g_cus, (hipStream_t) stream);

@@ -32,13 +32,13 @@ constexpr int STEP_BYTES = 1024;
 // column (inside the tile) of the first of the four weights that plane word j of a lane holds in step s
 __device__ __forceinline__ int tile_col(int s, int j, int half) { return 32 * s + 16 * (j >> 1) + 8 * half + 4 * (j & 1); }
 
-// One decode chain: the tiles [first unit, first unit + n) of one matrix, with the plane bytes of the next four steps
+// One decode chain: the tiles [first unit, first unit + n) of one matrix, with the plane bytes of the next D steps
 // in registers (reloaded as soon as a step is consumed).
-struct tchain {
+template <int D> struct tchain_t {
     w64_dec dec;
     const uint8_t * plane;
     uint32_t off, last;
-    uint4 sm[4];
+    uint4 sm[D];
     __device__ __forceinline__ uint4 load_step(int lane) const {
         const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
         return *((const uint4 *) (plane + o) + lane);
@@ -53,14 +53,15 @@ struct tchain {
         off = 0;
         last = (uint32_t) (n_units * T_BYTES - STEP_BYTES);
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
+        for (int s = 0; s < D; s++) {
             sm[s] = load_step(lane);
             off += STEP_BYTES;
         }
         dec.start(ring, q.stream, uniform(first), uniform(end), lane);
     }
+    // s: the step just consumed (a compile-time value at every call)
     __device__ __forceinline__ void reload(int s, int lane) {
-        sm[s] = load_step(lane);
+        sm[s % D] = load_step(lane);
         off += STEP_BYTES;
     }
     __device__ __forceinline__ void begin_tile() {
@@ -69,14 +70,15 @@ struct tchain {
         dec.keep_ahead();
     }
 };
+typedef tchain_t<4> tchain;
 
 // one step of N chains, instruction streams interleaved; lut of chain k at lut + k * lut_stride
-template <int N>
-__device__ __forceinline__ void tile_step(tchain * ch, const uint32_t * lut, int lut_stride, int s, uint32_t (&wp)[N][8]) {
+template <int N, int D>
+__device__ __forceinline__ void tile_step(tchain_t<D> * ch, const uint32_t * lut, int lut_stride, int s, uint32_t (&wp)[N][8]) {
     uint32_t smw[N][4];
 #pragma unroll
     for (int k = 0; k < N; k++) {
-        smw[k][0] = ch[k].sm[s].x; smw[k][1] = ch[k].sm[s].y; smw[k][2] = ch[k].sm[s].z; smw[k][3] = ch[k].sm[s].w;
+        smw[k][0] = ch[k].sm[s % D].x; smw[k][1] = ch[k].sm[s % D].y; smw[k][2] = ch[k].sm[s % D].z; smw[k][3] = ch[k].sm[s % D].w;
     }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -96,30 +98,58 @@ __device__ __forceinline__ void tile_step(tchain * ch, const uint32_t * lut, int
 
 // ---------------------------------------------------------------- batched MoE prefill
 
-constexpr int MT_WAVES = 8, MT_THREADS = MT_WAVES * 64;
-constexpr int MT_TOK = 128;        // tokens per pass: four 32-token blocks per wavefront
+constexpr int MT_SMALL_PAIRS = 16;  // routed pairs per expert up to which the 32-token shape is used
 constexpr int MT_HK = 128;         // activation columns staged at a time (half a tile)
 constexpr int MT_BSTRIDE = 136;    // BF16 elements per staged token row: 272 bytes spread 16 lanes over all banks
 
-struct mm_args {
-    const uint16_t * x; int64_t x_row;
-    const int32_t * ids_src1, * ids_dst, * bounds;
-    char * dst; int64_t dst_col; bool dst_bf16;
-    int64_t rows; // per expert
-    int n_experts;
+// Two shapes of the kernel.  NT = 4: passes of 128 tokens, eight wavefronts per block (the 2 x 4 accumulator blocks take
+// 128 registers: two wavefronts per SIMD).  NT = 1: passes of 32 tokens, sixteen wavefronts per block (32 accumulator
+// registers: four wavefronts per SIMD, twice the decode chains per CU) for experts, or dense matrices, with few tokens,
+// where the decode is all that counts.
+template <int NT> struct mt_shape {
+    static constexpr int WAVES = NT == 1 ? 16 : 8, THREADS = WAVES * 64, TOK = 32 * NT;
+    static constexpr int STAGERS = NT == 1 ? 512 : THREADS;        // threads that stage activations
+    static constexpr int TPT = STAGERS / TOK;                      // of them per token
+    static constexpr int CPT = MT_HK / TPT;                        // columns each: 32 (four uint4) or 8 (one)
+    static constexpr int VPT = CPT / 8;
+    static constexpr int DEPTH = NT == 1 ? 2 : 4;                  // steps of plane bytes held ahead per chain
 };
 
-// A work item is (expert, slab of row groups): every wavefront owns two decode chains — gate and up of one row group
-// (GLU), or two row groups of the matrix — and keeps their 2 x 4 accumulator blocks (32 rows x 32 tokens each) for
+// the uint4s a thread stages per block of activations (named members, not an array: under this kernel's register
+// pressure an array stays in scratch)
+template <int V> struct stage_regs;
+template <> struct stage_regs<4> {
+    uint4 a, b, c, d;
+    __device__ __forceinline__ void load(const uint4 * p) { a = p[0]; b = p[1]; c = p[2]; d = p[3]; }
+    __device__ __forceinline__ void store(uint4 * p) const { p[0] = a; p[1] = b; p[2] = c; p[3] = d; }
+};
+template <> struct stage_regs<1> {
+    uint4 a;
+    __device__ __forceinline__ void load(const uint4 * p) { a = p[0]; }
+    __device__ __forceinline__ void store(uint4 * p) const { p[0] = a; }
+};
+
+struct mm_args {
+    const uint16_t * x; int64_t x_row;
+    const int32_t * ids_src1, * ids_dst, * bounds; // all null: one dense matrix, token j reads row j of x and writes column j
+    char * dst; int64_t dst_col; bool dst_bf16;
+    int64_t rows;   // per expert
+    int64_t group0; // first row group of the product inside the matrix (dense products of a row range)
+    int n_experts, n_tok;
+};
+
+// A work item is (expert, slab of row groups): every wavefront owns two decode chains, gate and up of one row group
+// (GLU) or two row groups of the matrix, and keeps their 2 x NT accumulator blocks (32 rows x 32 tokens each) for
 // the whole pass over the expert's K columns.  Per step a chain yields two A operands (32 rows x 16 columns); the B
 // operands (16 columns x 32 tokens) come from the staged activations and are used by both chains.
-template <bool GLU>
-__global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+template <bool GLU, int NT>
+__global__ void __launch_bounds__(mt_shape<NT>::THREADS) k_mm_tile(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+    using S = mt_shape<NT>;
     constexpr int NM = GLU ? 2 : 1;
     extern __shared__ __align__(16) uint32_t shm[];
     uint32_t * lut = shm;
     uint32_t * rings = shm + NM * LUT_WORDS;
-    uint16_t * bbuf = (uint16_t *) (rings + MT_WAVES * 2 * WAVE_LDS_WORDS); // two buffers of MT_TOK x MT_BSTRIDE
+    uint16_t * bbuf = (uint16_t *) (rings + S::WAVES * 2 * WAVE_LDS_WORDS); // two buffers of TOK x MT_BSTRIDE
     const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
     stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
     if (GLU) {
@@ -127,58 +157,63 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
     }
     const int slabs = (int) (w.K / TILE_K), halves = 2 * slabs;
     const int groups = (int) (a.rows / TILE_R);               // row groups per expert
-    constexpr int GPI = GLU ? MT_WAVES : 2 * MT_WAVES;        // row groups per work item
+    constexpr int GPI = GLU ? S::WAVES : 2 * S::WAVES;        // row groups per work item
     const int slabs_per_expert = (groups + GPI - 1) / GPI;
     const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
-    const int b_tok = tid >> 2, b_part = tid & 3;             // this thread's share of a staged block: 32 columns of one token
+    // this thread's share of a staged block: CPT columns of one token (NT = 1: the upper wavefronts stage nothing)
+    const bool stager = S::STAGERS == S::THREADS || wave < S::STAGERS / 64;
+    const int b_tok = stager ? tid / S::TPT : 0, b_part = tid % S::TPT;
     __syncthreads();
     for (int item = blockIdx.x; item < a.n_experts * slabs_per_expert; item += gridDim.x) {
         const int e = item / slabs_per_expert, sl = item % slabs_per_expert;
-        const int j0 = a.bounds[e], n = a.bounds[e + 1] - j0;
+        const int j0 = a.bounds ? a.bounds[e] : 0, n = a.bounds ? a.bounds[e + 1] - j0 : a.n_tok;
         // this wavefront's row groups (inside the expert); a missing second group repeats the first and is dropped
         const int g0 = GLU ? sl * GPI + wave : sl * GPI + 2 * wave;
         const bool live = g0 < groups, has1 = GLU || g0 + 1 < groups;
         const int g1 = GLU ? g0 : (has1 ? g0 + 1 : g0);
-        for (int tp = 0; tp < n; tp += MT_TOK) {
-            const int left = n - tp, nt = left >= MT_TOK ? 4 : (left + 31) >> 5;
+        for (int tp = 0; tp < n; tp += S::TOK) {
+            const int left = n - tp, nt = NT == 1 ? 1 : left >= S::TOK ? NT : (left + 31) >> 5;
             const int btk = tp + b_tok;
-            const uint16_t * xsrc = a.x + (int64_t) a.ids_src1[j0 + (btk < n ? btk : 0)] * a.x_row + 32 * b_part;
-            uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + 32 * b_part;
-            // (four named registers, not an array: under this kernel's register pressure an array stays in scratch)
-            const uint4 f0 = *((const uint4 *) xsrc), f1 = *((const uint4 *) xsrc + 1), f2 = *((const uint4 *) xsrc + 2),
-                        f3 = *((const uint4 *) xsrc + 3);
-            tchain ch[2];
+            const int bj = j0 + (btk < n ? btk : 0);
+            const uint16_t * xsrc = a.x + (int64_t) (a.ids_src1 ? a.ids_src1[bj] : bj) * a.x_row + S::CPT * b_part;
+            uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + S::CPT * b_part;
+            stage_regs<S::VPT> f;
+            if (stager) {
+                f.load((const uint4 *) xsrc);
+            }
+            tchain_t<S::DEPTH> ch[2];
             if (live) {
                 uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * slabs, slabs, lane);
-                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * slabs, slabs, lane);
+                ch[0].start(ring, q0, (a.group0 + (int64_t) e * groups + g0) * slabs, slabs, lane);
+                ch[1].start(ring + WAVE_LDS_WORDS, q1, (a.group0 + (int64_t) e * groups + g1) * slabs, slabs, lane);
             }
-            f32x16_t acc[2][4];
+            f32x16_t acc[2][NT];
 #pragma unroll
             for (int c = 0; c < 2; c++) {
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
+                for (int t = 0; t < NT; t++) {
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
                         acc[c][t][i] = 0.f;
                     }
                 }
             }
-            *((uint4 *) bdst) = f0;
-            *((uint4 *) bdst + 1) = f1;
-            *((uint4 *) bdst + 2) = f2;
-            *((uint4 *) bdst + 3) = f3;
+            if (stager) {
+                f.store((uint4 *) bdst);
+            }
             __syncthreads();
 #pragma unroll 1
             for (int hs = 0; hs < halves; hs++) {
-                const uint16_t * bcur = bbuf + (hs & 1) * (MT_TOK * MT_BSTRIDE);
+                const uint16_t * bcur = bbuf + (hs & 1) * (S::TOK * MT_BSTRIDE);
                 // the next block of activations: requested now, staged after this block's steps.  Unconditional and
                 // local to the iteration (after the last block the same block goes into the buffer nobody reads any
                 // more): registers that are loaded under a condition and live around the loop are filled through a
                 // temporary with a full wait per load.
                 const int nxt = hs + 1 < halves ? hs + 1 : hs;
-                const uint4 * bsrc = (const uint4 *) (xsrc + nxt * MT_HK);
-                const uint4 b0 = bsrc[0], b1 = bsrc[1], b2 = bsrc[2], b3 = bsrc[3];
+                stage_regs<S::VPT> b;
+                if (stager) {
+                    b.load((const uint4 *) (xsrc + nxt * MT_HK));
+                }
                 if (live) {
                     if ((hs & 1) == 0) {
                         ch[0].begin_tile();
@@ -187,7 +222,7 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
 #pragma unroll
                     for (int s = 0; s < 4; s++) {
                         uint32_t wp[2][8];
-                        tile_step<2>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
+                        tile_step<2, S::DEPTH>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
                         ch[0].reload(s, lane);
                         ch[1].reload(s, lane);
                         const uint16_t * bp = bcur + l32 * MT_BSTRIDE + 32 * s + 8 * half;
@@ -203,7 +238,7 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
                         // token blocks beyond the first are there only for experts with that many tokens (one branch
                         // per block: both B operands are read together, then four matrix instructions)
 #pragma unroll
-                        for (int t = 0; t < 4; t++) {
+                        for (int t = 0; t < NT; t++) {
                             if (t == 0 || t < nt) {
                                 const bf16x8_t bv0 = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE);
                                 const bf16x8_t bv1 = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE + 16);
@@ -215,20 +250,18 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
                         }
                     }
                 }
-                uint4 * bn = (uint4 *) (bdst + ((hs + 1) & 1) * (MT_TOK * MT_BSTRIDE));
-                bn[0] = b0;
-                bn[1] = b1;
-                bn[2] = b2;
-                bn[3] = b3;
+                if (stager) {
+                    b.store((uint4 *) (bdst + ((hs + 1) & 1) * (S::TOK * MT_BSTRIDE)));
+                }
                 __syncthreads();
             }
             // accumulator element i of a lane: row 8 (i / 4) + 4 (lane / 32) + i % 4 of the group, token lane % 32
             if (live) {
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
+                for (int t = 0; t < NT; t++) {
                     const int tk = tp + 32 * t + l32;
                     if (t < nt && tk < n) {
-                        const int64_t col = (int64_t) a.ids_dst[j0 + tk] * a.dst_col;
+                        const int64_t col = (int64_t) (a.ids_dst ? a.ids_dst[j0 + tk] : tk) * a.dst_col;
 #pragma unroll
                         for (int c = 0; c < (GLU ? 1 : 2); c++) {
                             if (c == 1 && !has1) {
@@ -260,8 +293,9 @@ __global__ void __launch_bounds__(MT_THREADS) k_mm_tile(const bf16n_weight w, co
     }
 }
 
-size_t mt_shm(bool glu) {
-    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) MT_WAVES * 2 * WAVE_LDS_WORDS * 4 + (size_t) 2 * MT_TOK * MT_BSTRIDE * 2;
+template <int NT> size_t mt_shm(bool glu) {
+    using S = mt_shape<NT>;
+    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) S::WAVES * 2 * WAVE_LDS_WORDS * 4 + (size_t) 2 * S::TOK * MT_BSTRIDE * 2;
 }
 
 // ---------------------------------------------------------------- GEMV
@@ -352,7 +386,7 @@ __global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(con
                         xb.load(cv.x, kk + 16);
                     }
                     uint32_t wp[1][8];
-                    tile_step<1>(ch, my_lut, 0, s, wp);
+                    tile_step<1, 4>(ch, my_lut, 0, s, wp);
                     ch[0].reload(s, lane);
                     if (sizeof(TX) != 2) {
                         xa.load(cv.x, kk);
@@ -415,7 +449,7 @@ __device__ __forceinline__ void tile_run(const bf16n_weight & w, const uint32_t 
 #pragma unroll
             for (int s = 0; s < 4; s++) {
                 uint32_t wp[1][8];
-                tile_step<1>(ch, lut, 0, s, wp);
+                tile_step<1, 4>(ch, lut, 0, s, wp);
                 ch[0].reload(s, lane);
                 tile_store_step(wp[0], 4 * hh + s, lane & 31, lane >> 5, only_l, out + (int64_t) (t0 + u) * TILE_K * (f32 ? 4 : 2), row_bytes,
                                 f32);
@@ -462,29 +496,67 @@ bool is_tile_layout(const bf16n_weight & w) {
     return w.format == FMT_HUFPAIR && (w.flags & FLAG_WAVE64) && !(w.flags & FLAG_CHUNK_MAJOR) && w.R == TILE_R;
 }
 
+template <bool GLU, int NT> void mt_attr() {
+    (void) hipFuncSetAttribute((const void *) k_mm_tile<GLU, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<NT>(GLU));
+}
 void tile_init() {
-    (void) hipFuncSetAttribute((const void *) k_mm_tile<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm(true));
-    (void) hipFuncSetAttribute((const void *) k_mm_tile<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm(false));
+    mt_attr<true, 4>();
+    mt_attr<false, 4>();
+    mt_attr<true, 1>();
+    mt_attr<false, 1>();
 }
 
+template <int NT>
+void mt_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int cus, hipStream_t stream) {
+    using S = mt_shape<NT>;
+    const int groups = (int) (a.rows / TILE_R), gpi = up ? S::WAVES : 2 * S::WAVES;
+    const int64_t items = (int64_t) a.n_experts * ((groups + gpi - 1) / gpi);
+    const dim3 grid((unsigned) (items < (int64_t) cus ? items : (int64_t) cus));
+    if (up) {
+        hipLaunchKernelGGL((k_mm_tile<true, NT>), grid, dim3(S::THREADS), mt_shm<NT>(true), stream, w, *up, a);
+    } else {
+        hipLaunchKernelGGL((k_mm_tile<false, NT>), grid, dim3(S::THREADS), mt_shm<NT>(false), stream, w, w, a);
+    }
+}
+
+// n_pairs: routed (token, slot) pairs of the call
 void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
                         const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
-                        int cus, hipStream_t stream) {
+                        int64_t n_pairs, int cus, hipStream_t stream) {
     mm_args a;
     a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
     a.ids_src1 = ids_src1; a.ids_dst = ids_dst; a.bounds = bounds;
     a.dst = (char *) dst; a.dst_col = dst_col; a.dst_bf16 = dst_bf16;
-    a.rows = w.rows / n_experts; a.n_experts = n_experts;
+    a.rows = w.rows / n_experts; a.group0 = 0; a.n_experts = n_experts; a.n_tok = 0;
     if (a.rows % TILE_R != 0) {
         throw std::invalid_argument("bf16n: rows per expert must be a multiple of 32 for the tile layout");
     }
-    const int groups = (int) (a.rows / TILE_R), gpi = up ? MT_WAVES : 2 * MT_WAVES;
-    const int64_t items = (int64_t) n_experts * ((groups + gpi - 1) / gpi);
-    const dim3 grid((unsigned) (items < (int64_t) cus ? items : (int64_t) cus));
-    if (up) {
-        hipLaunchKernelGGL(k_mm_tile<true>, grid, dim3(MT_THREADS), mt_shm(true), stream, w, *up, a);
+    // passes of 32 tokens while few experts can hold more than 32 (every further pass decodes the expert again)
+    if (n_pairs <= (int64_t) MT_SMALL_PAIRS * n_experts) {
+        mt_launch<1>(w, up, a, cus, stream);
     } else {
-        hipLaunchKernelGGL(k_mm_tile<false>, grid, dim3(MT_THREADS), mt_shm(false), stream, w, w, a);
+        mt_launch<4>(w, up, a, cus, stream);
+    }
+}
+
+// Dense product through the matrix cores: y[j] = W[row0, row0 + nrows) x[j] for ncols BF16 columns (the products of BF16
+// values are exact in FP32, the accumulation is FP32).  Strides in elements of x (BF16) and of y.
+bool tile_mm_dense_pays(const bf16n_weight & w, int64_t nrows, int cus) {
+    // a block takes 32 row groups at a time: worth it when that gives at least half of the CUs a block
+    return nrows / (TILE_R * 2 * mt_shape<1>::WAVES) >= cus / 2 && w.K >= 1024;
+}
+
+void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x_bf16, int64_t x_row, int ncols, void * y,
+                          bool y_bf16, int64_t y_col, int cus, hipStream_t stream) {
+    mm_args a;
+    a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
+    a.ids_src1 = a.ids_dst = a.bounds = nullptr;
+    a.dst = (char *) y; a.dst_col = y_col; a.dst_bf16 = y_bf16;
+    a.rows = nrows; a.group0 = row0 / TILE_R; a.n_experts = 1; a.n_tok = ncols;
+    if (ncols <= mt_shape<1>::TOK) {
+        mt_launch<1>(w, nullptr, a, cus, stream);
+    } else {
+        mt_launch<4>(w, nullptr, a, cus, stream);
     }
 }
 

@@ -37,7 +37,11 @@ void launch_tile_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_
                           int64_t dst_s1, int64_t row0, hipStream_t stream);
 void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
                         const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
-                        int cus, hipStream_t stream);
+                        int64_t n_pairs, int cus, hipStream_t stream);
+
+bool tile_mm_dense_pays(const bf16n_weight & w, int64_t nrows, int cus);
+void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x_bf16, int64_t x_row, int ncols, void * y,
+                          bool y_bf16, int64_t y_col, int cus, hipStream_t stream);
 
 // MoE glue (kernels_moe.hip)
 void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int cus, hipStream_t stream);

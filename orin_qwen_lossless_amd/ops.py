@@ -318,8 +318,17 @@ def mmv_glu2(x: torch.Tensor, gate: Weight, up: Weight, ids: torch.Tensor | None
     return _mmv_common(x, gate, ids, rows_per_matrix, out_dtype == torch.bfloat16, False, True, up)
 
 
+def gemv_max_tokens(w: Weight) -> int:
+    """BF16 token columns up to which mmv is the faster dense path for this matrix: GEMV_MAX_TOKENS (the reference's
+    rule, ops.py:25-27), or more for matrices whose dense products run on the matrix cores."""
+    n = C.c_int(0)
+    cw = _cweight(w)
+    _lib.check(_lib.lib().bf16n_gemv_max_tokens(C.byref(cw), C.byref(n)))
+    return n.value
+
+
 def linear(x: torch.Tensor, w: Weight, bias: torch.Tensor | None = None) -> torch.Tensor:
-    """y = x W^T (+ bias) in BF16: up to GEMV_MAX_TOKENS tokens through the decode GEMV (FP32 accumulation, the bias
+    """y = x W^T (+ bias) in BF16: up to gemv_max_tokens(w) tokens through the decode GEMV (FP32 accumulation, the bias
     added in FP32 before the one rounding to BF16), more through exact dequant in row chunks + a stock BF16 GEMM
     (core/torch/torch_bindings.cpp:198-239)."""
     if x.dtype != torch.bfloat16:
@@ -330,7 +339,7 @@ def linear(x: torch.Tensor, w: Weight, bias: torch.Tensor | None = None) -> torc
     oshape = list(x.shape[:-1]) + [rows]
     x2 = x.reshape(-1, K)
     T = x2.shape[0]
-    if T <= GEMV_MAX_TOKENS:
+    if T <= GEMV_MAX_TOKENS or T <= gemv_max_tokens(w):
         ok = x2.stride(1) == 1 and (x2.stride(0) * 2) % 16 == 0 and x2.data_ptr() % 16 == 0
         xc = x2 if ok else x2.contiguous()
         if bias is not None:

@@ -71,6 +71,94 @@ def test_full_size_product_within_fp64_bound(ops, head):
     assert torch.equal(ops.mmv(x[1:2], enc)[0].view(torch.int32), y[1].view(torch.int32))
 
 
+# ---- the same matrix in the tile layout: dense products of BF16 activations run on the matrix cores, any batch size ------
+
+@pytest.fixture(scope="module")
+def head_tiles(ops, head):
+    w, _ = head
+    wbits = w.cpu().view(torch.int16).numpy().view(np.uint16)
+    plane, aux, fmt_out, R = ops.encode_bits(wbits, 3, 32, False, wave64=True)
+    assert (fmt_out, R) == (3, 32)
+    ta = torch.from_numpy(aux)
+    return w, ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
+
+
+def fp64_product(w, x):
+    """x [T, K] times the exact weights, and the bound sum |w x|, in FP64, in row chunks."""
+    ref = torch.empty((x.shape[0], ROWS), dtype=torch.float64, device="cuda")
+    bound = torch.empty_like(ref)
+    xd = x.double()
+    for r0 in range(0, ROWS, 1 << 15):
+        wd = w[r0: r0 + (1 << 15)].double()
+        ref[:, r0: r0 + wd.shape[0]] = xd @ wd.t()
+        bound[:, r0: r0 + wd.shape[0]] = xd.abs() @ wd.abs().t()
+    return ref, bound
+
+
+def test_full_size_tiles_round_trip_and_one_hot(ops, head_tiles):
+    w, enc = head_tiles
+    assert ops.roundtrip_equal(enc, w)
+    assert ops.gemv_max_tokens(enc) > 8
+    keep = torch.ones(ROWS, dtype=torch.bool, device="cuda")
+    keep[ROWS - 7] = False
+    for col in (0, 1033, K - 1):
+        x = torch.zeros((1, K), dtype=torch.bfloat16, device="cuda")
+        x[0, col] = 0.5
+        y = ops.mmv(x, enc)[0]
+        assert torch.equal(y[keep], (w[:, col].float() * 0.5)[keep])
+        assert bool(torch.isnan(y[ROWS - 7]))
+
+
+@pytest.mark.parametrize("T", [1, 7, 32, 33, 130])
+def test_full_size_tiles_dense_product_any_batch(ops, head_tiles, T):
+    w, enc = head_tiles
+    g = torch.Generator(device="cuda").manual_seed(20 + T)
+    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
+    y = ops.mmv(x, enc)
+    keep = torch.ones(ROWS, dtype=torch.bool, device="cuda")
+    keep[ROWS - 7] = False
+    ref, bound = fp64_product(w, x)
+    assert bool(((y.double() - ref).abs()[:, keep] <= 1e-5 * bound[:, keep]).all())
+    # every column has the bits of its single-column launch, whatever the batch (passes of 32 or of 128 tokens)
+    for t in {0, T // 2, T - 1}:
+        assert torch.equal(ops.mmv(x[t: t + 1], enc)[0].view(torch.int32), y[t].view(torch.int32))
+    # BF16 output: the round-to-nearest-even of the FP32 output; linear() takes the same path up to gemv_max_tokens
+    y16 = ops.mmv(x, enc, out_dtype=torch.bfloat16)
+    assert torch.equal(y16[:, keep], y[:, keep].to(torch.bfloat16))
+    assert T > ops.gemv_max_tokens(enc) or torch.equal(ops.linear(x, enc).view(torch.int16), y16.view(torch.int16))
+    # FP32 activations keep their precision: they go through the GEMV kernel, within the same bound
+    if T == 1:
+        xf = torch.randn((1, K), generator=g, device="cuda")
+        yf = ops.mmv(xf, enc)
+        rf, bf = fp64_product(w, xf)
+        assert bool(((yf.double() - rf).abs()[:, keep] <= 1e-5 * bf[:, keep]).all())
+
+
+def test_full_size_tiles_row_range_and_strides(ops, head_tiles):
+    """Through the C ABI: a product over a row range of the matrix, activations and outputs with padded row strides."""
+    import ctypes as C
+
+    from orin_qwen_lossless_amd import _lib
+    from orin_qwen_lossless_amd.ops import _cweight, _stream
+
+    w, enc = head_tiles
+    T, row0, nrows = 5, 32 * 100, 32 * 5000
+    g = torch.Generator(device="cuda").manual_seed(31)
+    xw = torch.randn((T, K + 8), generator=g, device="cuda").to(torch.bfloat16)
+    x = xw[:, :K]
+    full = ops.mmv(x.contiguous(), enc)
+    yw = torch.zeros((T, nrows + 4), dtype=torch.float32, device="cuda")
+    a = _lib.MmvArgs()
+    a.x, a.y, a.x_bf16, a.y_bf16 = x.data_ptr(), yw.data_ptr(), 1, 0
+    a.ncols, a.n_used, a.x_per_slot = T, 1, 1
+    a.x_tok, a.y_tok = x.stride(0) * 2, yw.stride(0) * 4
+    a.rows_per_matrix, a.row0, a.nrows = ROWS, row0, nrows
+    cw = _cweight(enc)
+    _lib.check(_lib.lib().bf16n_mmv(C.byref(cw), C.byref(a), _stream(), 1))
+    assert torch.equal(yw[:, :nrows], full[:, row0: row0 + nrows])
+    assert not bool(yw[:, nrows:].any())
+
+
 # ---- one MoE layer of the 35B-A3B shape at its real size: 256 experts x (gate, up 512 x 2048; down 2048 x 512) -----------
 
 E, TOPK, N = 256, 8, 512

@@ -122,6 +122,53 @@ def test_mm_ids_against_exact_weights(ops, K, N):
 
 
 @pytest.mark.parametrize("K,N", MM_SHAPES)
+def test_mm_ids_few_tokens_per_expert(ops, K, N):
+    # up to 16 routed pairs per expert the kernel runs passes of 32 tokens on blocks of sixteen wavefronts: experts with
+    # none, one, 32, 33 and 70 tokens (one to three passes), against FP64 products of the exact weights; the same
+    # tokens inside a larger call (passes of 128 tokens) give the same bits
+    E, k, T = 12, 2, 90
+    wb = synth.weights(E * N, K, 41 + K + N)
+    w = enc(ops, wb, HP, 32, False, True)
+    wf = synth.bf16_bits_to_f32(wb)
+    ids = routing(T, k, E, {0: 70, 1: 33, 2: 32, 3: 1, 4: 0}, 15)
+    per_slot = K == 512
+    xb = synth.activations(T * (k if per_slot else 1), K, 4).reshape((T, k, K) if per_slot else (T, K))
+    xf = synth.bf16_bits_to_f32(xb)
+    got = ops.moe_mm_ids(tbf16(xb), torch.from_numpy(ids).cuda(), w, E).cpu().numpy()
+    y, s = reference(wf, xf, ids, N, per_slot)
+    assert np.all(np.abs(got - y) <= GEMV_REL * s + 1e-30)
+    assert np.all(np.abs(got - y) <= 1e-3 * np.abs(y) + 1e-5)
+    got16 = ops.moe_mm_ids(tbf16(xb), torch.from_numpy(ids).cuda(), w, E, out_dtype=torch.bfloat16)
+    assert np.array_equal(bits(got16), rne_bf16(got))
+    more = 8 * E                                    # the same tokens followed by others: more than 16 pairs per expert
+    ids2 = np.concatenate([ids, routing(more, k, E, {}, 16)])
+    xb2 = np.concatenate([xb, synth.activations(more * (k if per_slot else 1), K, 5).reshape((more,) + xb.shape[1:])])
+    got2 = ops.moe_mm_ids(tbf16(xb2), torch.from_numpy(ids2).cuda(), w, E).cpu().numpy()
+    assert np.array_equal(got2[:T], got)
+
+
+@pytest.mark.parametrize("K,N", [(2048, 128), (2048, 512), (1024, 96)])
+def test_mm_ids_fused_gate_up_few_tokens_per_expert(ops, K, N):
+    E, k, T = 10, 2, 70
+    gb, ub = synth.weights(E * N, K, 51), synth.weights(E * N, K, 52)
+    g, u = enc(ops, gb, HP, 32, False, True), enc(ops, ub, HP, 32, False, True)
+    ids = routing(T, k, E, {0: 40, 1: 0}, 7)
+    xb = synth.activations(T, K, 9)
+    xt, it = tbf16(xb), torch.from_numpy(ids).cuda()
+    fused = ops.moe_mm_ids(xt, it, g, E, up=u).cpu().numpy()
+    xf = synth.bf16_bits_to_f32(xb)
+    y1, _ = reference(synth.bf16_bits_to_f32(gb), xf, ids, N, False)
+    y2, _ = reference(synth.bf16_bits_to_f32(ub), xf, ids, N, False)
+    ref = y2 * (y1 / (1.0 + np.exp(-y1)))
+    assert np.all(np.abs(fused - ref) <= 1e-3 * np.abs(ref) + 1e-5)
+    more = 9 * E
+    ids2 = np.concatenate([ids, routing(more, k, E, {}, 17)])
+    xb2 = np.concatenate([xb, synth.activations(more, K, 6)])
+    fused2 = ops.moe_mm_ids(tbf16(xb2), torch.from_numpy(ids2).cuda(), g, E, up=u).cpu().numpy()
+    assert np.array_equal(fused2[:T], fused)
+
+
+@pytest.mark.parametrize("K,N", MM_SHAPES)
 def test_mm_ids_one_hot_is_exact(ops, K, N):
     E, k, T = 4, 2, 70
     wb = synth.weights(E * N, K, 21 + K)
