@@ -99,20 +99,23 @@ __device__ __forceinline__ void tile_step(tchain_t<D> * ch, const uint32_t * lut
 // ---------------------------------------------------------------- batched MoE prefill
 
 constexpr int MT_SMALL_PAIRS = 16;  // routed pairs per expert up to which the 32-token shape is used
+constexpr int MT_MAX_LISTED = 1024; // experts up to which a block lists the active ones
 constexpr int MT_HK = 128;         // activation columns staged at a time (half a tile)
 constexpr int MT_BSTRIDE = 136;    // BF16 elements per staged token row: 272 bytes spread 16 lanes over all banks
 
-// Two shapes of the kernel.  NT = 4: passes of 128 tokens, eight wavefronts per block (the 2 x 4 accumulator blocks take
-// 128 registers: two wavefronts per SIMD).  NT = 1: passes of 32 tokens, sixteen wavefronts per block (32 accumulator
-// registers: four wavefronts per SIMD, twice the decode chains per CU) for experts, or dense matrices, with few tokens,
-// where the decode is all that counts.
-template <int NT> struct mt_shape {
-    static constexpr int WAVES = NT == 1 ? 16 : 8, THREADS = WAVES * 64, TOK = 32 * NT;
-    static constexpr int STAGERS = NT == 1 ? 512 : THREADS;        // threads that stage activations
+// Three shapes of the kernel.  NT = 4: passes of 128 tokens, eight wavefronts per block (the 2 x 4 accumulator blocks
+// take 128 registers: two wavefronts per SIMD).  NT = 1: passes of 32 tokens for experts, or dense matrices, with few
+// tokens, where the decode is all that counts: sixteen wavefronts per block (32 accumulator registers: four wavefronts
+// per SIMD, twice the decode chains per CU), or four per block, two blocks per CU, when so few experts are active that
+// whole experts per block would leave most of the CUs idle.
+template <int NT, int W> struct mt_shape {
+    static constexpr int WAVES = W, THREADS = WAVES * 64, TOK = 32 * NT;
+    static constexpr int STAGERS = TOK * MT_HK / 8 < THREADS ? TOK * MT_HK / 8 : THREADS; // threads that stage activations
     static constexpr int TPT = STAGERS / TOK;                      // of them per token
-    static constexpr int CPT = MT_HK / TPT;                        // columns each: 32 (four uint4) or 8 (one)
+    static constexpr int CPT = MT_HK / TPT;                        // columns each: 8 per uint4
     static constexpr int VPT = CPT / 8;
     static constexpr int DEPTH = NT == 1 ? 2 : 4;                  // steps of plane bytes held ahead per chain
+    static constexpr int BLOCKS_PER_CU = W == 4 ? 2 : 1;           // what the LDS of a CU holds
 };
 
 // the uint4s a thread stages per block of activations (named members, not an array: under this kernel's register
@@ -122,6 +125,11 @@ template <> struct stage_regs<4> {
     uint4 a, b, c, d;
     __device__ __forceinline__ void load(const uint4 * p) { a = p[0]; b = p[1]; c = p[2]; d = p[3]; }
     __device__ __forceinline__ void store(uint4 * p) const { p[0] = a; p[1] = b; p[2] = c; p[3] = d; }
+};
+template <> struct stage_regs<2> {
+    uint4 a, b;
+    __device__ __forceinline__ void load(const uint4 * p) { a = p[0]; b = p[1]; }
+    __device__ __forceinline__ void store(uint4 * p) const { p[0] = a; p[1] = b; }
 };
 template <> struct stage_regs<1> {
     uint4 a;
@@ -142,9 +150,9 @@ struct mm_args {
 // (GLU) or two row groups of the matrix, and keeps their 2 x NT accumulator blocks (32 rows x 32 tokens each) for
 // the whole pass over the expert's K columns.  Per step a chain yields two A operands (32 rows x 16 columns); the B
 // operands (16 columns x 32 tokens) come from the staged activations and are used by both chains.
-template <bool GLU, int NT>
-__global__ void __launch_bounds__(mt_shape<NT>::THREADS) k_mm_tile(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
-    using S = mt_shape<NT>;
+template <bool GLU, int NT, int W>
+__global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+    using S = mt_shape<NT, W>;
     constexpr int NM = GLU ? 2 : 1;
     extern __shared__ __align__(16) uint32_t shm[];
     uint32_t * lut = shm;
@@ -163,9 +171,34 @@ __global__ void __launch_bounds__(mt_shape<NT>::THREADS) k_mm_tile(const bf16n_w
     // this thread's share of a staged block: CPT columns of one token (NT = 1: the upper wavefronts stage nothing)
     const bool stager = S::STAGERS == S::THREADS || wave < S::STAGERS / 64;
     const int b_tok = stager ? tid / S::TPT : 0, b_part = tid % S::TPT;
+    // The experts that have tokens, in order, listed by the first wavefront: the blocks share out the work items of
+    // these only, so that a call with few active experts keeps one item per block instead of leaving some blocks
+    // with several and others with none.
+    uint16_t * act = (uint16_t *) (bbuf + 2 * S::TOK * MT_BSTRIDE);
+    const bool listed = a.bounds != nullptr && a.n_experts <= MT_MAX_LISTED;
+    int n_act = a.n_experts;
+    if (listed) {
+        if (wave == 0) {
+            int base = 0;
+            for (int e0 = 0; e0 < a.n_experts; e0 += 64) {
+                const int e = e0 + lane;
+                const bool on = e < a.n_experts && a.bounds[e + 1] > a.bounds[e];
+                const uint64_t m = __ballot(on);
+                if (on) {
+                    act[base + __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u))] = (uint16_t) e;
+                }
+                base += __builtin_popcountll(m);
+            }
+            if (lane == 0) {
+                act[MT_MAX_LISTED] = (uint16_t) base;
+            }
+        }
+        __syncthreads();
+        n_act = act[MT_MAX_LISTED];
+    }
     __syncthreads();
-    for (int item = blockIdx.x; item < a.n_experts * slabs_per_expert; item += gridDim.x) {
-        const int e = item / slabs_per_expert, sl = item % slabs_per_expert;
+    for (int item = blockIdx.x; item < n_act * slabs_per_expert; item += gridDim.x) {
+        const int e = listed ? act[item / slabs_per_expert] : item / slabs_per_expert, sl = item % slabs_per_expert;
         const int j0 = a.bounds ? a.bounds[e] : 0, n = a.bounds ? a.bounds[e + 1] - j0 : a.n_tok;
         // this wavefront's row groups (inside the expert); a missing second group repeats the first and is dropped
         const int g0 = GLU ? sl * GPI + wave : sl * GPI + 2 * wave;
@@ -293,9 +326,10 @@ __global__ void __launch_bounds__(mt_shape<NT>::THREADS) k_mm_tile(const bf16n_w
     }
 }
 
-template <int NT> size_t mt_shm(bool glu) {
-    using S = mt_shape<NT>;
-    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) S::WAVES * 2 * WAVE_LDS_WORDS * 4 + (size_t) 2 * S::TOK * MT_BSTRIDE * 2;
+template <int NT, int W> size_t mt_shm(bool glu) {
+    using S = mt_shape<NT, W>;
+    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) S::WAVES * 2 * WAVE_LDS_WORDS * 4 + (size_t) 2 * S::TOK * MT_BSTRIDE * 2 +
+           (MT_MAX_LISTED + 8) * 2;
 }
 
 // ---------------------------------------------------------------- GEMV
@@ -496,26 +530,43 @@ bool is_tile_layout(const bf16n_weight & w) {
     return w.format == FMT_HUFPAIR && (w.flags & FLAG_WAVE64) && !(w.flags & FLAG_CHUNK_MAJOR) && w.R == TILE_R;
 }
 
-template <bool GLU, int NT> void mt_attr() {
-    (void) hipFuncSetAttribute((const void *) k_mm_tile<GLU, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<NT>(GLU));
+template <bool GLU, int NT, int W> void mt_attr() {
+    (void) hipFuncSetAttribute((const void *) k_mm_tile<GLU, NT, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<NT, W>(GLU));
 }
 void tile_init() {
-    mt_attr<true, 4>();
-    mt_attr<false, 4>();
-    mt_attr<true, 1>();
-    mt_attr<false, 1>();
+    mt_attr<true, 4, 8>();
+    mt_attr<false, 4, 8>();
+    mt_attr<true, 1, 16>();
+    mt_attr<false, 1, 16>();
+    mt_attr<true, 1, 4>();
+    mt_attr<false, 1, 4>();
 }
 
-template <int NT>
+template <int W> int64_t mt_items(const mm_args & a, bool glu) {
+    const int groups = (int) (a.rows / TILE_R), gpi = glu ? W : 2 * W;
+    return (int64_t) a.n_experts * ((groups + gpi - 1) / gpi);
+}
+
+template <int NT, int W>
 void mt_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int cus, hipStream_t stream) {
-    using S = mt_shape<NT>;
-    const int groups = (int) (a.rows / TILE_R), gpi = up ? S::WAVES : 2 * S::WAVES;
-    const int64_t items = (int64_t) a.n_experts * ((groups + gpi - 1) / gpi);
-    const dim3 grid((unsigned) (items < (int64_t) cus ? items : (int64_t) cus));
+    using S = mt_shape<NT, W>;
+    const int64_t items = mt_items<W>(a, up != nullptr), slots = (int64_t) cus * S::BLOCKS_PER_CU;
+    const dim3 grid((unsigned) (items < slots ? items : slots));
     if (up) {
-        hipLaunchKernelGGL((k_mm_tile<true, NT>), grid, dim3(S::THREADS), mt_shm<NT>(true), stream, w, *up, a);
+        hipLaunchKernelGGL((k_mm_tile<true, NT, W>), grid, dim3(S::THREADS), (mt_shm<NT, W>(true)), stream, w, *up, a);
     } else {
-        hipLaunchKernelGGL((k_mm_tile<false, NT>), grid, dim3(S::THREADS), mt_shm<NT>(false), stream, w, w, a);
+        hipLaunchKernelGGL((k_mm_tile<false, NT, W>), grid, dim3(S::THREADS), (mt_shm<NT, W>(false)), stream, w, w, a);
+    }
+}
+
+// passes of 32 tokens: whole experts (or 32 row groups) per block of sixteen wavefronts, unless the experts that can be
+// active (one per routed pair at most) would then occupy less than half of the CUs: blocks of four wavefronts
+void mt_launch_small(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int64_t n_pairs, int cus, hipStream_t stream) {
+    const int64_t active = n_pairs < a.n_experts ? n_pairs : a.n_experts;
+    if (active * (mt_items<16>(a, up != nullptr) / a.n_experts) <= cus / 2) {
+        mt_launch<1, 4>(w, up, a, cus, stream);
+    } else {
+        mt_launch<1, 16>(w, up, a, cus, stream);
     }
 }
 
@@ -533,9 +584,9 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
     }
     // passes of 32 tokens while few experts can hold more than 32 (every further pass decodes the expert again)
     if (n_pairs <= (int64_t) MT_SMALL_PAIRS * n_experts) {
-        mt_launch<1>(w, up, a, cus, stream);
+        mt_launch_small(w, up, a, n_pairs, cus, stream);
     } else {
-        mt_launch<4>(w, up, a, cus, stream);
+        mt_launch<4, 8>(w, up, a, cus, stream);
     }
 }
 
@@ -543,7 +594,7 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
 // values are exact in FP32, the accumulation is FP32).  Strides in elements of x (BF16) and of y.
 bool tile_mm_dense_pays(const bf16n_weight & w, int64_t nrows, int cus) {
     // a block takes 32 row groups at a time: worth it when that gives at least half of the CUs a block
-    return nrows / (TILE_R * 2 * mt_shape<1>::WAVES) >= cus / 2 && w.K >= 1024;
+    return nrows / (TILE_R * 2 * 16) >= cus / 2 && w.K >= 1024;
 }
 
 void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x_bf16, int64_t x_row, int ncols, void * y,
@@ -553,10 +604,10 @@ void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, c
     a.ids_src1 = a.ids_dst = a.bounds = nullptr;
     a.dst = (char *) y; a.dst_col = y_col; a.dst_bf16 = y_bf16;
     a.rows = nrows; a.group0 = row0 / TILE_R; a.n_experts = 1; a.n_tok = ncols;
-    if (ncols <= mt_shape<1>::TOK) {
-        mt_launch<1>(w, nullptr, a, cus, stream);
+    if (ncols <= 32) {
+        mt_launch<1, 16>(w, nullptr, a, cus, stream);
     } else {
-        mt_launch<4>(w, nullptr, a, cus, stream);
+        mt_launch<4, 8>(w, nullptr, a, cus, stream);
     }
 }
 
