@@ -228,7 +228,7 @@ def test_moe_experts_in_both_token_regimes(ops, T):
 @pytest.mark.parametrize("T", [11, 12, 13, 30])
 def test_moe_experts_path_switch_by_routed_pairs_per_expert(ops, T, monkeypatch):
     # 128 experts, top-4: expert GEMVs up to 0.4 * 128 / 4 = 12 tokens, the batched kernels above; both within tolerance
-    E, k, Kd, N = 128, 4, 1024, 256
+    E, k, Kd, N = 128, 4, 512, 512
     gate = enc(ops, synth.weights(E * N, Kd, 81), HP, 32, False, True)
     up = enc(ops, synth.weights(E * N, Kd, 82), HP, 32, False, True)
     down = enc(ops, synth.weights(E * Kd, N, 83), HP, 32, False, True)
