@@ -104,14 +104,16 @@ def cpu_baseline(wbits, K: int, xf, sample_rows: int):
                       f"{nbytes} compressed bytes), mean of {reps} runs ({med * 1e3:.1f} ms each, best {best * 1e3:.1f} ms)"}
 
 
-def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: str = "mi355x"):
-    """Encode a [rows, K] BF16 device tensor under the mi355x policy (n_matrices stacked experts) and upload `copies`
-    copies; returns (list of weights, compressed bytes, description)."""
+def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: str = "mi355x", matrix_core_order: bool = False):
+    """Encode a [rows, K] BF16 device tensor under the mi355x policy (n_matrices stacked experts; matrix_core_order: the
+    policy's dense_frag_order option) and upload `copies` copies; returns (list of weights, compressed bytes,
+    description)."""
     import numpy as np
     import torch
 
     rows, K = w_dev.shape
-    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, K, n_matrices, engine=engine, expert=n_matrices > 1)
+    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, K, n_matrices, engine=engine, expert=n_matrices > 1,
+                                    dense_frag_order=matrix_core_order)
     wbits = w_dev.cpu().view(torch.int16).numpy().view(np.uint16)
     plane, aux, fmt_out, _ = ops.encode_bits(wbits, fmt, R, cm, wave64=w64)
     ta = torch.from_numpy(aux)
@@ -224,6 +226,18 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
     x4 = randx(4, K)
     t4 = med_us(lambda i: ops.mmv(x4, head_copies[i & 1]))
     out["lm_head_batch4_us"] = round(t4, 2)
+    # the output projection at other batch sizes: groups of up to eight columns per decode in the layout above, then
+    # dequant + a stock GEMM; and the same matrix as 32 x 256 tiles (the policy's matrix-core order for dense matrices),
+    # where BF16 activations go through the matrix cores at any batch size
+    batches = {}
+    tiles, tbytes, tdesc = encode_to_device(ops, w_head, copies=2, matrix_core_order=True)
+    for T in (1, 2, 4, 8, 16, 32, 128):
+        xT = randx(T, K)
+        base = graph_us(lambda i: ops.mmv(xT, head_copies[i & 1]), 4, 10) if T <= 8 else med_us(lambda i: ops.linear(xT, head_copies[i & 1]), 10, 2)
+        batches[str(T)] = {"units_of_16_rows_us": round(base, 1), "path": "gemv" if T <= 8 else "dequant + BF16 GEMM",
+                           "tiles_us": round(graph_us(lambda i: ops.mmv(xT, tiles[i & 1]), 4, 10), 1)}
+    out["lm_head_batches"] = {"tiles": tdesc, "tiles_bytes": tbytes, "by_batch": batches}
+    del tiles
     # small NIBBLE matrices
     for rows, k in ((512, 2048), (2048, 512)):
         ws, nbytes, desc = encode_to_device(ops, randw(rows, k), copies=2)

@@ -45,7 +45,8 @@ void bf16n_set_encode_threads(int n);
 /* ---- shape policy: bf16n::choose, core/include/bf16n/policy.h:12-38, core/src/policy.cpp:45-69 -------------------- */
 /* out[5] = {format, R, chunk_major, frag_order, wave64}.  Returns 1 if a choice was made, 0 if the shape stays BF16
  * (std::nullopt).  Never fails.  engine MI355X: the reference's llama rules with unit sizes chosen for 256 CUs of
- * wave64 and the wave64 stream layout where the shape allows it; experts with a multiple of 32 rows get R = 32 tiles. */
+ * wave64 and the wave64 stream layout where the shape allows it; experts with a multiple of 32 rows get R = 32 tiles,
+ * and so do, with dense_frag_order set, dense matrices of at least 131072 rows (a multiple of 32), K >= 1024. */
 int bf16n_choose(int64_t rows, int64_t K, int64_t n_matrices, int engine, int mode, int64_t dense_min, int expert,
                  int dense_frag_order, int * out);
 

@@ -118,31 +118,32 @@ template <int NT, int W> struct mt_shape {
     static constexpr int BLOCKS_PER_CU = W == 4 ? 2 : 1;           // what the LDS of a CU holds
 };
 
-// the uint4s a thread stages per block of activations (named members, not an array: under this kernel's register
-// pressure an array stays in scratch)
-template <int V> struct stage_regs;
-template <> struct stage_regs<4> {
-    uint4 a, b, c, d;
-    __device__ __forceinline__ void load(const uint4 * p) { a = p[0]; b = p[1]; c = p[2]; d = p[3]; }
-    __device__ __forceinline__ void store(uint4 * p) const { p[0] = a; p[1] = b; p[2] = c; p[3] = d; }
-};
-template <> struct stage_regs<2> {
-    uint4 a, b;
-    __device__ __forceinline__ void load(const uint4 * p) { a = p[0]; b = p[1]; }
-    __device__ __forceinline__ void store(uint4 * p) const { p[0] = a; p[1] = b; }
-};
-template <> struct stage_regs<1> {
-    uint4 a;
-    __device__ __forceinline__ void load(const uint4 * p) { a = p[0]; }
-    __device__ __forceinline__ void store(uint4 * p) const { p[0] = a; }
-};
+// the V uint4s a thread stages per block of activations, in named registers (under this kernel's register pressure
+// an array, or a struct of them, stays in scratch, and every load into it is waited for at once)
+#define MT_STAGE_LOAD(V, r0, r1, r2, r3, p)  \
+    do {                                      \
+        r0 = (p)[0];                          \
+        if constexpr ((V) >= 2) r1 = (p)[1];  \
+        if constexpr ((V) >= 4) {             \
+            r2 = (p)[2];                      \
+            r3 = (p)[3];                      \
+        }                                     \
+    } while (0)
+#define MT_STAGE_STORE(V, r0, r1, r2, r3, p) \
+    do {                                      \
+        (p)[0] = r0;                          \
+        if constexpr ((V) >= 2) (p)[1] = r1;  \
+        if constexpr ((V) >= 4) {             \
+            (p)[2] = r2;                      \
+            (p)[3] = r3;                      \
+        }                                     \
+    } while (0)
 
 struct mm_args {
     const uint16_t * x; int64_t x_row;
     const int32_t * ids_src1, * ids_dst, * bounds; // all null: one dense matrix, token j reads row j of x and writes column j
     char * dst; int64_t dst_col; bool dst_bf16;
     int64_t rows;   // per expert
-    int64_t group0; // first row group of the product inside the matrix (dense products of a row range)
     int n_experts, n_tok;
 };
 
@@ -175,7 +176,8 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
     // these only, so that a call with few active experts keeps one item per block instead of leaving some blocks
     // with several and others with none.
     uint16_t * act = (uint16_t *) (bbuf + 2 * S::TOK * MT_BSTRIDE);
-    const bool listed = a.bounds != nullptr && a.n_experts <= MT_MAX_LISTED;
+    // (passes of 128 tokens are for calls with many tokens per expert: every expert is active)
+    const bool listed = NT == 1 && a.bounds != nullptr && a.n_experts <= MT_MAX_LISTED;
     int n_act = a.n_experts;
     if (listed) {
         if (wave == 0) {
@@ -194,11 +196,12 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
             }
         }
         __syncthreads();
-        n_act = act[MT_MAX_LISTED];
+        n_act = (int) uniform(act[MT_MAX_LISTED]);
     }
     __syncthreads();
     for (int item = blockIdx.x; item < n_act * slabs_per_expert; item += gridDim.x) {
-        const int e = listed ? act[item / slabs_per_expert] : item / slabs_per_expert, sl = item % slabs_per_expert;
+        // (read from LDS: the same in every lane, and kept in a scalar register like the arithmetic form)
+        const int e = listed ? (int) uniform(act[item / slabs_per_expert]) : item / slabs_per_expert, sl = item % slabs_per_expert;
         const int j0 = a.bounds ? a.bounds[e] : 0, n = a.bounds ? a.bounds[e + 1] - j0 : a.n_tok;
         // this wavefront's row groups (inside the expert); a missing second group repeats the first and is dropped
         const int g0 = GLU ? sl * GPI + wave : sl * GPI + 2 * wave;
@@ -210,15 +213,15 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
             const int bj = j0 + (btk < n ? btk : 0);
             const uint16_t * xsrc = a.x + (int64_t) (a.ids_src1 ? a.ids_src1[bj] : bj) * a.x_row + S::CPT * b_part;
             uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + S::CPT * b_part;
-            stage_regs<S::VPT> f;
+            uint4 f0, f1, f2, f3;
             if (stager) {
-                f.load((const uint4 *) xsrc);
+                MT_STAGE_LOAD(S::VPT, f0, f1, f2, f3, (const uint4 *) xsrc);
             }
             tchain_t<S::DEPTH> ch[2];
             if (live) {
                 uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-                ch[0].start(ring, q0, (a.group0 + (int64_t) e * groups + g0) * slabs, slabs, lane);
-                ch[1].start(ring + WAVE_LDS_WORDS, q1, (a.group0 + (int64_t) e * groups + g1) * slabs, slabs, lane);
+                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * slabs, slabs, lane);
+                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * slabs, slabs, lane);
             }
             f32x16_t acc[2][NT];
 #pragma unroll
@@ -232,7 +235,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                 }
             }
             if (stager) {
-                f.store((uint4 *) bdst);
+                MT_STAGE_STORE(S::VPT, f0, f1, f2, f3, (uint4 *) bdst);
             }
             __syncthreads();
 #pragma unroll 1
@@ -243,9 +246,9 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                 // more): registers that are loaded under a condition and live around the loop are filled through a
                 // temporary with a full wait per load.
                 const int nxt = hs + 1 < halves ? hs + 1 : hs;
-                stage_regs<S::VPT> b;
+                uint4 b0, b1, b2, b3;
                 if (stager) {
-                    b.load((const uint4 *) (xsrc + nxt * MT_HK));
+                    MT_STAGE_LOAD(S::VPT, b0, b1, b2, b3, (const uint4 *) (xsrc + nxt * MT_HK));
                 }
                 if (live) {
                     if ((hs & 1) == 0) {
@@ -284,7 +287,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                     }
                 }
                 if (stager) {
-                    b.store((uint4 *) (bdst + ((hs + 1) & 1) * (S::TOK * MT_BSTRIDE)));
+                    MT_STAGE_STORE(S::VPT, b0, b1, b2, b3, (uint4 *) (bdst + ((hs + 1) & 1) * (S::TOK * MT_BSTRIDE)));
                 }
                 __syncthreads();
             }
@@ -578,7 +581,7 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
     a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
     a.ids_src1 = ids_src1; a.ids_dst = ids_dst; a.bounds = bounds;
     a.dst = (char *) dst; a.dst_col = dst_col; a.dst_bf16 = dst_bf16;
-    a.rows = w.rows / n_experts; a.group0 = 0; a.n_experts = n_experts; a.n_tok = 0;
+    a.rows = w.rows / n_experts; a.n_experts = n_experts; a.n_tok = 0;
     if (a.rows % TILE_R != 0) {
         throw std::invalid_argument("bf16n: rows per expert must be a multiple of 32 for the tile layout");
     }
@@ -603,11 +606,16 @@ void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, c
     a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
     a.ids_src1 = a.ids_dst = a.bounds = nullptr;
     a.dst = (char *) y; a.dst_col = y_col; a.dst_bf16 = y_bf16;
-    a.rows = nrows; a.group0 = row0 / TILE_R; a.n_experts = 1; a.n_tok = ncols;
+    a.rows = nrows; a.n_experts = 1; a.n_tok = ncols;
+    // a view of the row range: the plane bytes and the unit bases of its first tile onwards
+    bf16n_weight v = w;
+    const int64_t tile0 = row0 / TILE_R * (w.K / TILE_K);
+    v.plane += tile0 * T_BYTES;
+    v.off_b += (uint64_t) tile0 * 4;
     if (ncols <= 32) {
-        mt_launch<1, 16>(w, nullptr, a, cus, stream);
+        mt_launch<1, 16>(v, nullptr, a, cus, stream);
     } else {
-        mt_launch<4, 8>(w, nullptr, a, cus, stream);
+        mt_launch<4, 8>(v, nullptr, a, cus, stream);
     }
 }
 

@@ -174,6 +174,13 @@ def test_policy_mi355x():
     assert ops.choose(96, 1536, 8, expert=True) == (HP, 32, False, False, True)
     assert ops.choose(144, 2048, 8, expert=True) == (HP, 4, False, False, True)
     assert ops.choose(512, 2048)[0] == NIB and ops.choose(2048, 512)[0] == NIB and ops.choose(256, 2048)[0] == NIB
+    # dense matrices of at least 131072 rows take the tiles when the caller asks for the matrix-core order
+    assert ops.choose(248320, 2048, dense_frag_order=True) == (HP, 32, False, False, True)
+    assert ops.choose(131072, 1024, dense_frag_order=True) == (HP, 32, False, False, True)
+    assert ops.choose(131040, 2048, dense_frag_order=True) == (HP, 16, False, False, True)   # too few rows
+    assert ops.choose(248336, 2048, dense_frag_order=True) == (HP, 16, False, False, True)   # not a multiple of 32
+    assert ops.choose(248320, 512, dense_frag_order=True) == (HP, 16, False, False, True)    # K too short
+    assert ops.choose(5120, 2048, dense_frag_order=True) == (HP, 4, False, False, True)
     # shapes without a wave64 GEMV instance keep the reference layouts
     assert ops.choose(16384, 1536) == (HP, 4, False, False, False)
     assert ops.choose(520, 1536, 8, expert=True) == (HP, 8, True, False, False)
