@@ -341,6 +341,29 @@ def prefill_only(T: int, steps: int) -> None:
                       "frac_of_bf16_mfma_peak": round((flops_gu + flops_dn) / (t_gu + t_dn) / 1e6 / 2500.0, 4)}))
 
 
+def head_tiles_only(T: int, steps: int, rows: int, K: int) -> None:
+    """Only the output projection in the policy's matrix-core order (32 x 256 tiles) at batch T: bf16n_mmv with BF16
+    activations, which runs on the matrix cores, `steps` times on two alternated copies.  For profiling this kernel
+    alone; prints its own JSON line."""
+    import torch
+
+    from orin_qwen_lossless_amd import ops
+
+    torch.cuda.set_device(0)
+    ops.init()
+    w = gen_weights(rows, K, 1)
+    tiles, nbytes, desc = encode_to_device(ops, w, copies=2, matrix_core_order=True)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
+    y = ops.mmv(x, tiles[0])
+    err = float(((y.double() - x.double() @ w.double().t()).abs() / (x.double().abs() @ w.double().abs().t())).max())
+    t = med_us(lambda i: ops.mmv(x, tiles[i & 1]), steps, 5)
+    algo = nbytes + T * K * 2 + T * rows * 4
+    print(json.dumps({"workload": f"output projection {rows}x{K}, {desc}, batch {T} BF16 activations, FP32 out", "us": round(t, 2),
+                      "compressed_bytes": nbytes, "algorithmic_bytes": algo, "GBps": round(algo / t / 1e3, 1),
+                      "frac_of_hbm_peak": round(algo / t / 1e3 / HBM_PEAK_GBS, 4), "max_err_over_sum_abs": err}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -354,11 +377,16 @@ def main() -> None:
     ap.add_argument("--suite", action="store_true", help="also time batch 4, the NIBBLE matrices, a MoE layer and the prefill")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="run only the batched MoE kernels of one layer on T tokens (for profiling) and exit")
+    ap.add_argument("--head-tiles", type=int, default=0, metavar="T",
+                    help="run only the output projection as 32 x 256 tiles at batch T (for profiling) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path has no collective); run with --gpus 1")
     if args.prefill > 0:
         prefill_only(args.prefill, min(args.steps, 20))
+        return
+    if args.head_tiles > 0:
+        head_tiles_only(args.head_tiles, min(args.steps, 50), args.rows, args.K)
         return
 
     import numpy as np

@@ -209,7 +209,7 @@ int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
         ensure_init();
         check_weight(*w);
         require(out != nullptr, "null output");
-        *out = dev::is_tile_layout(*w) && dev::tile_mm_dense_pays(*w, w->rows, g_cus) ? 256 : 8;
+        *out = dev::is_tile_layout(*w) && dev::tile_mm_dense_pays(*w, w->rows, g_cus) ? 512 : 8;
     });
 }
 
