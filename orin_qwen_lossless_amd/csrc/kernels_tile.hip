@@ -115,7 +115,6 @@ template <int NT, int W> struct mt_shape {
     static constexpr int CPT = MT_HK / TPT;                        // columns each: 8 per uint4
     static constexpr int VPT = CPT / 8;
     static constexpr int DEPTH = NT == 1 ? 2 : 4;                  // steps of plane bytes held ahead per chain
-    static constexpr int BLOCKS_PER_CU = W == 4 ? 2 : 1;           // what the LDS of a CU holds
 };
 
 // the V uint4s a thread stages per block of activations, in named registers (under this kernel's register pressure
@@ -147,6 +146,29 @@ struct mm_args {
     int n_experts, n_tok;
 };
 
+// The experts that have tokens, in order, listed in LDS by the first wavefront (act[MT_MAX_LISTED]: their number, which
+// is returned): the blocks share out the work items of these only, so that a call with few active experts keeps its
+// blocks equally loaded instead of leaving some with several items and others with none.  Ends with a barrier.
+__device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, int wave, int lane) {
+    if (wave == 0) {
+        int base = 0;
+        for (int e0 = 0; e0 < a.n_experts; e0 += 64) {
+            const int e = e0 + lane;
+            const bool on = e < a.n_experts && a.bounds[e + 1] > a.bounds[e];
+            const uint64_t m = __ballot(on);
+            if (on) {
+                act[base + __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u))] = (uint16_t) e;
+            }
+            base += __builtin_popcountll(m);
+        }
+        if (lane == 0) {
+            act[MT_MAX_LISTED] = (uint16_t) base;
+        }
+    }
+    __syncthreads();
+    return (int) uniform(act[MT_MAX_LISTED]);
+}
+
 // A work item is (expert, slab of row groups): every wavefront owns two decode chains, gate and up of one row group
 // (GLU) or two row groups of the matrix, and keeps their 2 x NT accumulator blocks (32 rows x 32 tokens each) for
 // the whole pass over the expert's K columns.  Per step a chain yields two A operands (32 rows x 16 columns); the B
@@ -172,32 +194,10 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
     // this thread's share of a staged block: CPT columns of one token (NT = 1: the upper wavefronts stage nothing)
     const bool stager = S::STAGERS == S::THREADS || wave < S::STAGERS / 64;
     const int b_tok = stager ? tid / S::TPT : 0, b_part = tid % S::TPT;
-    // The experts that have tokens, in order, listed by the first wavefront: the blocks share out the work items of
-    // these only, so that a call with few active experts keeps one item per block instead of leaving some blocks
-    // with several and others with none.
     uint16_t * act = (uint16_t *) (bbuf + 2 * S::TOK * MT_BSTRIDE);
     // (passes of 128 tokens are for calls with many tokens per expert: every expert is active)
     const bool listed = NT == 1 && a.bounds != nullptr && a.n_experts <= MT_MAX_LISTED;
-    int n_act = a.n_experts;
-    if (listed) {
-        if (wave == 0) {
-            int base = 0;
-            for (int e0 = 0; e0 < a.n_experts; e0 += 64) {
-                const int e = e0 + lane;
-                const bool on = e < a.n_experts && a.bounds[e + 1] > a.bounds[e];
-                const uint64_t m = __ballot(on);
-                if (on) {
-                    act[base + __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u))] = (uint16_t) e;
-                }
-                base += __builtin_popcountll(m);
-            }
-            if (lane == 0) {
-                act[MT_MAX_LISTED] = (uint16_t) base;
-            }
-        }
-        __syncthreads();
-        n_act = (int) uniform(act[MT_MAX_LISTED]);
-    }
+    const int n_act = listed ? list_active(act, a, wave, lane) : a.n_experts;
     __syncthreads();
     for (int item = blockIdx.x; item < n_act * slabs_per_expert; item += gridDim.x) {
         // (read from LDS: the same in every lane, and kept in a scalar register like the arithmetic form)
@@ -327,6 +327,149 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
             }
         }
     }
+}
+
+// Few active experts (decode at small batch): a pass over an expert is one decode chain per wavefront, K / 32 steps
+// long, and nothing runs beside it, so the chain is cut instead: WPI = K / 256 wavefronts share a work item (expert,
+// pair of row groups, or gate and up of one group), each decodes one tile per chain (8 steps) against its 256 columns of
+// the activations, read straight from memory (16 bytes per lane and matrix instruction, one step ahead: no staging, no
+// barrier inside the chain), and the partial accumulators are added in K order through LDS (the rings, idle by then).
+// Sixteen wavefronts per block: 16 / WPI items.  Passes of 32 tokens; the block runs as many as its busiest item needs.
+constexpr int KS_WAVES = 16;
+
+template <bool GLU, int WPI>
+__global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight w, const bf16n_weight w_up, const mm_args a, const int spw) {
+    constexpr int NM = GLU ? 2 : 1, IPB = KS_WAVES / WPI, RPW = 16 / WPI; // items per block; accumulator registers a wavefront adds up
+    extern __shared__ __align__(16) uint32_t shm[];
+    uint32_t * lut = shm;
+    uint32_t * rings = shm + NM * LUT_WORDS;
+    float * part = (float *) rings;                           // [wavefront][register][lane], 6 KB apart
+    uint16_t * act = (uint16_t *) (rings + KS_WAVES * 2 * WAVE_LDS_WORDS);
+    const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
+    const int is = wave / WPI, kw = wave % WPI;               // item of the block, K part
+    stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
+    if (GLU) {
+        stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
+    }
+    const int groups = (int) (a.rows / TILE_R);
+    const int per_expert = GLU ? groups : (groups + 1) / 2;   // items per expert
+    const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
+    uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
+    const int n_items = list_active(act, a, wave, lane) * per_expert;
+    __syncthreads();
+    for (int base = blockIdx.x * IPB; base < n_items; base += gridDim.x * IPB) {
+        int maxn = 0;
+#pragma unroll
+        for (int k = 0; k < IPB; k++) {
+            if (base + k < n_items) {
+                const int ek = (int) uniform(act[(base + k) / per_expert]);
+                const int nk = a.bounds[ek + 1] - a.bounds[ek];
+                maxn = nk > maxn ? nk : maxn;
+            }
+        }
+        const int item = base + is;
+        const bool valid = item < n_items;
+        const int e = valid ? (int) uniform(act[item / per_expert]) : 0, p = valid ? item % per_expert : 0;
+        const int j0 = a.bounds[e], n = valid ? a.bounds[e + 1] - j0 : 0;
+        const int g0 = GLU ? p : 2 * p;
+        const bool has1 = GLU || g0 + 1 < groups;
+        const int g1 = has1 && !GLU ? g0 + 1 : g0;
+        for (int tp = 0; tp < maxn; tp += 32) {
+            const int tk = tp + l32;
+            f32x16_t acc[2];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    acc[c][i] = 0.f;
+                }
+            }
+            if (tp < n) {
+                // this lane's token (past the item's last: that one again, dropped at the store), its K part and half
+                const char * xr = (const char *) (a.x + (int64_t) a.ids_src1[j0 + (tk < n ? tk : n - 1)] * a.x_row + kw * spw * TILE_K) + 16 * half;
+                tchain_t<2> ch[2];
+                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * (WPI * spw) + kw * spw, spw, lane);
+                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * (WPI * spw) + kw * spw, spw, lane);
+                // B operands of a step: columns 32 s + 8 half + [0, 8) and 16 further on
+                bf16x8_t nb0 = *(const bf16x8_t *) xr, nb1 = *(const bf16x8_t *) (xr + 32);
+#pragma unroll 1
+                for (int t = 0; t < spw; t++) {
+                ch[0].begin_tile();
+                ch[1].begin_tile();
+#pragma unroll
+                for (int s = 0; s < T_STEPS; s++) {
+                    const bf16x8_t bv0 = nb0, bv1 = nb1;
+                    const int nq = t * T_STEPS + s + 1;
+                    const char * xn = xr + (nq < spw * T_STEPS ? nq : 0) * 64; // after the last step: the first again, unused
+                    nb0 = *(const bf16x8_t *) xn;
+                    nb1 = *(const bf16x8_t *) (xn + 32);
+                    uint32_t wp[2][8];
+                    tile_step<2, 2>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
+                    ch[0].reload(s, lane);
+                    ch[1].reload(s, lane);
+                    bf16x8_t av[2][2]; // [chain][16-column block]
+#pragma unroll
+                    for (int c = 0; c < 2; c++) {
+#pragma unroll
+                        for (int kb = 0; kb < 2; kb++) {
+                            const u32x4_t v = {wp[c][4 * kb], wp[c][4 * kb + 1], wp[c][4 * kb + 2], wp[c][4 * kb + 3]};
+                            av[c][kb] = __builtin_bit_cast(bf16x8_t, v);
+                        }
+                    }
+                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0][0], bv0, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][0], bv0, acc[1], 0, 0, 0);
+                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0][1], bv1, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][1], bv1, acc[1], 0, 0, 0);
+                }
+                }
+            }
+            __syncthreads(); // every ring is idle: they hold the partial sums now
+            float r[2][RPW];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    part[(wave * (2 * WAVE_LDS_WORDS)) + i * 64 + lane] = acc[c][i];
+                }
+                __syncthreads();
+#pragma unroll
+                for (int q = 0; q < RPW; q++) {
+                    float sum = 0.f;
+#pragma unroll
+                    for (int k = 0; k < WPI; k++) {
+                        sum += part[((is * WPI + k) * (2 * WAVE_LDS_WORDS)) + (kw * RPW + q) * 64 + lane];
+                    }
+                    r[c][q] = sum;
+                }
+                __syncthreads();
+            }
+            // accumulator element i of a lane: row 8 (i / 4) + 4 (lane / 32) + i % 4 of the group, token lane % 32
+            if (tk < n) {
+                const int64_t col = (int64_t) a.ids_dst[j0 + tk] * a.dst_col;
+#pragma unroll
+                for (int c = 0; c < (GLU ? 1 : 2); c++) {
+                    if (c == 1 && !has1) {
+                        continue;
+                    }
+#pragma unroll
+                    for (int q = 0; q < RPW; q++) {
+                        const int i = kw * RPW + q;
+                        const int64_t o = col + (int64_t) (c ? g1 : g0) * TILE_R + 8 * (i >> 2) + 4 * half + (i & 3);
+                        const float v = GLU ? r[1][q] * silu(r[0][q]) : r[c][q];
+                        if (a.dst_bf16) {
+                            ((uint16_t *) a.dst)[o] = f32_to_bf16_rne(v);
+                        } else {
+                            ((float *) a.dst)[o] = v;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+size_t ks_shm(bool glu) {
+    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_LISTED + 8) * 2;
 }
 
 template <int NT, int W> size_t mt_shm(bool glu) {
@@ -536,13 +679,17 @@ bool is_tile_layout(const bf16n_weight & w) {
 template <bool GLU, int NT, int W> void mt_attr() {
     (void) hipFuncSetAttribute((const void *) k_mm_tile<GLU, NT, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<NT, W>(GLU));
 }
+template <bool GLU, int WPI> void ks_attr() {
+    (void) hipFuncSetAttribute((const void *) k_mm_tile_ks<GLU, WPI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ks_shm(GLU));
+}
+
 void tile_init() {
     mt_attr<true, 4, 8>();
     mt_attr<false, 4, 8>();
     mt_attr<true, 1, 16>();
     mt_attr<false, 1, 16>();
-    mt_attr<true, 1, 4>();
-    mt_attr<false, 1, 4>();
+    ks_attr<true, 2>(); ks_attr<false, 2>(); ks_attr<true, 4>(); ks_attr<false, 4>();
+    ks_attr<true, 8>(); ks_attr<false, 8>(); ks_attr<true, 16>(); ks_attr<false, 16>();
 }
 
 template <int W> int64_t mt_items(const mm_args & a, bool glu) {
@@ -553,7 +700,7 @@ template <int W> int64_t mt_items(const mm_args & a, bool glu) {
 template <int NT, int W>
 void mt_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int cus, hipStream_t stream) {
     using S = mt_shape<NT, W>;
-    const int64_t items = mt_items<W>(a, up != nullptr), slots = (int64_t) cus * S::BLOCKS_PER_CU;
+    const int64_t items = mt_items<W>(a, up != nullptr), slots = cus; // the LDS of a CU holds one block
     const dim3 grid((unsigned) (items < slots ? items : slots));
     if (up) {
         hipLaunchKernelGGL((k_mm_tile<true, NT, W>), grid, dim3(S::THREADS), (mt_shm<NT, W>(true)), stream, w, *up, a);
@@ -562,12 +709,41 @@ void mt_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & 
     }
 }
 
+template <int WPI>
+void ks_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int64_t blocks, int spw, hipStream_t stream) {
+    if (up) {
+        hipLaunchKernelGGL((k_mm_tile_ks<true, WPI>), dim3((unsigned) blocks), dim3(KS_WAVES * 64), ks_shm(true), stream, w, *up, a, spw);
+    } else {
+        hipLaunchKernelGGL((k_mm_tile_ks<false, WPI>), dim3((unsigned) blocks), dim3(KS_WAVES * 64), ks_shm(false), stream, w, w, a, spw);
+    }
+}
+
 // passes of 32 tokens: whole experts (or 32 row groups) per block of sixteen wavefronts, unless the experts that can be
-// active (one per routed pair at most) would then occupy less than half of the CUs: blocks of four wavefronts
+// active (one per routed pair at most) are so few that K can be split over 2 to 16 wavefronts per item and the blocks
+// still fit the GPU at once: the most wavefronts per item (the shortest chains) for which they do
 void mt_launch_small(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int64_t n_pairs, int cus, hipStream_t stream) {
     const int64_t active = n_pairs < a.n_experts ? n_pairs : a.n_experts;
-    if (active * (mt_items<16>(a, up != nullptr) / a.n_experts) <= cus / 2) {
-        mt_launch<1, 4>(w, up, a, cus, stream);
+    const int slabs = (int) (w.K / TILE_K), groups = (int) (a.rows / TILE_R);
+    const int64_t items = active * (up ? groups : (groups + 1) / 2);
+    int wpi = 0;
+    if (a.bounds && a.n_experts <= MT_MAX_LISTED) {
+        for (int c = KS_WAVES; c >= 2; c /= 2) {
+            if (slabs % c == 0 && (items * c + KS_WAVES - 1) / KS_WAVES <= cus) {
+                wpi = c;
+                break;
+            }
+        }
+    }
+    if (wpi) {
+        int64_t blocks = (items * wpi + KS_WAVES - 1) / KS_WAVES;
+        blocks = blocks > 0 ? blocks : 1;
+        const int spw = slabs / wpi;
+        switch (wpi) {
+            case 2: ks_launch<2>(w, up, a, blocks, spw, stream); break;
+            case 4: ks_launch<4>(w, up, a, blocks, spw, stream); break;
+            case 8: ks_launch<8>(w, up, a, blocks, spw, stream); break;
+            default: ks_launch<16>(w, up, a, blocks, spw, stream); break;
+        }
     } else {
         mt_launch<1, 16>(w, up, a, cus, stream);
     }

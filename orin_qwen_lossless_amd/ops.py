@@ -25,7 +25,8 @@ FLAG_CHUNK_MAJOR, FLAG_FRAG_ORDER, FLAG_WAVE64 = 1, 2, 4
 # up to 8 tokens through the GEMV kernels, more through the batched MoE kernel / dequant + GEMM
 # (engines/vllm/vllm_bf16n/ops.py:25-27, core/torch/torch_bindings.cpp:195)
 GEMV_MAX_TOKENS = 8
-MOE_GEMV_PAIRS_PER_EXPERT = 0.4  # moe_experts: expert GEMVs up to this many routed (token, slot) pairs per expert
+# moe_experts: expert GEMVs up to this many routed (token, slot) pairs per expert (tile layout, other layouts)
+MOE_GEMV_PAIRS_PER_EXPERT = (0.2, 0.7)
 DEQUANT_CHUNK_BYTES = 64 << 20
 
 ENGINES = {"llama": 0, "vllm": 1, "mi355x": 2}
@@ -492,11 +493,14 @@ def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_we
     N = gate.meta.rows // n_experts
     H = down.meta.rows // n_experts
     x = x.contiguous()
-    # The reference switches to the batched kernels above 8 tokens.  On this part the expert GEMVs stay ahead while
-    # the routed pairs are fewer than about 0.4 x the experts (each pair decodes one expert matrix in its own GEMV
-    # column; the batched kernel decodes every active expert once, but a pass over an expert is one long decode chain
-    # per wavefront, which few active experts cannot hide): 12 tokens for top-8 of 256, where the two paths measure equal.
-    gemv_tokens = max(GEMV_MAX_TOKENS, int(MOE_GEMV_PAIRS_PER_EXPERT * n_experts) // max(topk_ids.shape[1], 1))
+    # The reference switches to the batched kernels above 8 tokens.  Here the expert GEMVs stay ahead while the routed
+    # pairs are few against the experts (each pair decodes one expert matrix in its own GEMV column; the batched kernel
+    # decodes every active expert once).  Tile layout: up to 0.2 pairs per expert (6 tokens for top-8 of 256; measured
+    # 57 / 97 us GEMV against 64 / 83 us batched at 4 / 8 tokens), its batched kernel splits K over wavefronts while
+    # few experts are active; other layouts: 0.7 and never below the reference's 8 tokens.
+    tiles = all(m.meta.wave64 and m.meta.R == 32 for m in (gate, up, down))
+    per_expert = MOE_GEMV_PAIRS_PER_EXPERT[0 if tiles else 1]
+    gemv_tokens = max(4 if tiles else GEMV_MAX_TOKENS, int(per_expert * n_experts) // max(topk_ids.shape[1], 1))
     if T > gemv_tokens and mm_ids_supported(gate, up) and mm_ids_supported(down):
         # one routing pass for both products: with one activation row per (token, slot), as down takes them, the
         # source row of a pair is its destination row

@@ -207,12 +207,12 @@ def test_full_size_batched_moe_against_exact_weights_and_the_gemv_path(ops, expe
             gg, uu = wg[e * N:(e + 1) * N].double() @ xe, wu[e * N:(e + 1) * N].double() @ xe
             want = uu * (gg / (1.0 + torch.exp(-gg)))
             assert torch.all((a[t, s].double() - want).abs() <= 1e-3 * want.abs() + 1e-5), (t, s)
-    # fewer tokens take other shapes of the kernel (passes of 32 tokens: blocks of sixteen wavefronts at 256 tokens, of
-    # four at 16 tokens, where few experts are active): the same bits for the same tokens
-    for n in (256, 16):
+    # fewer tokens take other shapes of the kernel: passes of 32 tokens at 256 tokens (the same bits for the same
+    # tokens), K split over the wavefronts at 16 and 2 tokens, where few experts are active (another summation order)
+    for n in (256, 16, 2):
         r = ops.mm_ids_route(ids[:n].contiguous(), E, False)
         an = ops.moe_mm_ids(x[:n], ids[:n].contiguous(), gate, E, up=up, out_dtype=torch.float32, routes=r)
-        assert torch.equal(an, a[:n]), n
+        assert torch.equal(an, a[:n]) if n == 256 else torch.all((an - a[:n]).abs() <= 1e-4 * a[:n].abs() + 1e-6), n
     # the batched kernel and the routed GEMV (decode path) agree on the first tokens; so do the down products
     a8 = ops.mmv_glu2(x[:8], gate, up, ids[:8].contiguous(), N)
     assert torch.all((a8 - a[:8]).abs() <= 1e-3 * a[:8].abs() + 1e-5)
@@ -220,9 +220,10 @@ def test_full_size_batched_moe_against_exact_weights_and_the_gemv_path(ops, expe
     ys = ops.moe_mm_ids(a16, ids, down, E, routes=(dst, dst, bounds))
     y8 = ops.mmv(a16[:8].float(), down, ids[:8].contiguous(), K)
     assert torch.all((y8 - ys[:8]).abs() <= 1e-3 * ys[:8].abs() + 1e-5)
-    for n in (256, 16):
+    for n in (256, 16, 2):
         r = ops.mm_ids_route(ids[:n].contiguous(), E, False)
-        assert torch.equal(ops.moe_mm_ids(a16[:n], ids[:n].contiguous(), down, E, routes=(r[1], r[1], r[2])), ys[:n]), n
+        yn = ops.moe_mm_ids(a16[:n], ids[:n].contiguous(), down, E, routes=(r[1], r[1], r[2]))
+        assert torch.equal(yn, ys[:n]) if n == 256 else torch.all((yn - ys[:n]).abs() <= 1e-4 * ys[:n].abs() + 1e-6), n
     # linearity in the activations: doubling them doubles every product exactly (powers of two commute with rounding)
     ys2 = ops.moe_mm_ids((a16.float() * 2).to(torch.bfloat16), ids, down, E, routes=(dst, dst, bounds))
     assert torch.equal(ys2, ys * 2)

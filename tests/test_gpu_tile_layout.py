@@ -123,9 +123,10 @@ def test_mm_ids_against_exact_weights(ops, K, N):
 
 @pytest.mark.parametrize("K,N", MM_SHAPES)
 def test_mm_ids_few_tokens_per_expert(ops, K, N):
-    # up to 16 routed pairs per expert the kernel runs passes of 32 tokens on blocks of sixteen wavefronts: experts with
-    # none, one, 32, 33 and 70 tokens (one to three passes), against FP64 products of the exact weights; the same
-    # tokens inside a larger call (passes of 128 tokens) give the same bits
+    # up to 16 routed pairs per expert the kernel runs passes of 32 tokens, here (few experts) with K split over the
+    # wavefronts of an item: experts with none, one, 32, 33 and 70 tokens (one to three passes), against FP64 products
+    # of the exact weights; the same tokens inside a larger call (passes of 128 tokens, another summation order) agree
+    # within the bound
     E, k, T = 12, 2, 90
     wb = synth.weights(E * N, K, 41 + K + N)
     w = enc(ops, wb, HP, 32, False, True)
@@ -144,7 +145,7 @@ def test_mm_ids_few_tokens_per_expert(ops, K, N):
     ids2 = np.concatenate([ids, routing(more, k, E, {}, 16)])
     xb2 = np.concatenate([xb, synth.activations(more * (k if per_slot else 1), K, 5).reshape((more,) + xb.shape[1:])])
     got2 = ops.moe_mm_ids(tbf16(xb2), torch.from_numpy(ids2).cuda(), w, E).cpu().numpy()
-    assert np.array_equal(got2[:T], got)
+    assert np.all(np.abs(got2[:T] - got) <= 2 * GEMV_REL * s + 1e-30)
 
 
 @pytest.mark.parametrize("K,N", [(2048, 128), (2048, 512), (1024, 96)])
@@ -165,7 +166,7 @@ def test_mm_ids_fused_gate_up_few_tokens_per_expert(ops, K, N):
     ids2 = np.concatenate([ids, routing(more, k, E, {}, 17)])
     xb2 = np.concatenate([xb, synth.activations(more, K, 6)])
     fused2 = ops.moe_mm_ids(tbf16(xb2), torch.from_numpy(ids2).cuda(), g, E, up=u).cpu().numpy()
-    assert np.array_equal(fused2[:T], fused)
+    assert np.all(np.abs(fused2[:T] - fused) <= 1e-4 * np.abs(fused) + 1e-6)
 
 
 @pytest.mark.parametrize("K,N", MM_SHAPES)
@@ -210,7 +211,7 @@ def test_mm_ids_fused_gate_up_swiglu(ops, K, N):
     assert np.array_equal(bits(f16), rne_bf16(fused))
 
 
-@pytest.mark.parametrize("T", [8, 9, 40])
+@pytest.mark.parametrize("T", [3, 8, 9, 40])
 def test_moe_experts_in_both_token_regimes(ops, T):
     E, k, Kd, N = 8, 2, 2048, 512
     gate = enc(ops, synth.weights(E * N, Kd, 51), HP, 32, False, True)
@@ -227,8 +228,8 @@ def test_moe_experts_in_both_token_regimes(ops, T):
 
 @pytest.mark.parametrize("T", [11, 12, 13, 30])
 def test_moe_experts_path_switch_by_routed_pairs_per_expert(ops, T, monkeypatch):
-    # 128 experts, top-4: expert GEMVs up to 0.4 * 128 / 4 = 12 tokens, the batched kernels above; both within tolerance
-    E, k, Kd, N = 128, 4, 512, 512
+    # 240 experts, top-4: expert GEMVs up to 0.2 * 240 / 4 = 12 tokens, the batched kernels above; both within tolerance
+    E, k, Kd, N = 240, 4, 512, 512
     gate = enc(ops, synth.weights(E * N, Kd, 81), HP, 32, False, True)
     up = enc(ops, synth.weights(E * N, Kd, 82), HP, 32, False, True)
     down = enc(ops, synth.weights(E * Kd, N, 83), HP, 32, False, True)
