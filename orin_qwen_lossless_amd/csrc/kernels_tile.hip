@@ -146,27 +146,34 @@ struct mm_args {
     int n_experts, n_tok;
 };
 
-// The experts that have tokens, in order, listed in LDS by the first wavefront (act[MT_MAX_LISTED]: their number, which
-// is returned): the blocks share out the work items of these only, so that a call with few active experts keeps its
-// blocks equally loaded instead of leaving some with several items and others with none.  Ends with a barrier.
-__device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, int wave, int lane) {
-    if (wave == 0) {
-        int base = 0;
-        for (int e0 = 0; e0 < a.n_experts; e0 += 64) {
-            const int e = e0 + lane;
-            const bool on = e < a.n_experts && a.bounds[e + 1] > a.bounds[e];
-            const uint64_t m = __ballot(on);
-            if (on) {
-                act[base + __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u))] = (uint16_t) e;
-            }
-            base += __builtin_popcountll(m);
-        }
+// The experts that have tokens, in order, listed in LDS (act[MT_MAX_LISTED]: their number, which is returned): the
+// blocks share out the work items of these only, so that a call with few active experts keeps its blocks equally loaded
+// instead of leaving some with several items and others with none.  Every wavefront of the block takes 64 experts at
+// a time (one read of their bounds for the whole block), the counts meet in LDS behind the list.  Ends with a barrier.
+__device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, int wave, int lane, int n_waves) {
+    int * cnt = (int *) (act + MT_MAX_LISTED + 8); // [n_waves], n_waves <= 16
+    int total = 0;
+    for (int e0 = 0; e0 < a.n_experts; e0 += 64 * n_waves) {
+        const int e = e0 + 64 * wave + lane;
+        const bool on = e < a.n_experts && a.bounds[e + 1] > a.bounds[e];
+        const uint64_t m = __ballot(on);
         if (lane == 0) {
-            act[MT_MAX_LISTED] = (uint16_t) base;
+            cnt[wave] = __builtin_popcountll(m);
         }
+        __syncthreads();
+        int before = total, all = 0;
+        for (int k = 0; k < n_waves; k++) {
+            const int c = cnt[k];
+            before += k < wave ? c : 0;
+            all += c;
+        }
+        if (on) {
+            act[before + __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u))] = (uint16_t) e;
+        }
+        total += all;
+        __syncthreads();
     }
-    __syncthreads();
-    return (int) uniform(act[MT_MAX_LISTED]);
+    return (int) uniform((uint32_t) total);
 }
 
 // A work item is (expert, slab of row groups): every wavefront owns two decode chains, gate and up of one row group
@@ -197,7 +204,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
     uint16_t * act = (uint16_t *) (bbuf + 2 * S::TOK * MT_BSTRIDE);
     // (passes of 128 tokens are for calls with many tokens per expert: every expert is active)
     const bool listed = NT == 1 && a.bounds != nullptr && a.n_experts <= MT_MAX_LISTED;
-    const int n_act = listed ? list_active(act, a, wave, lane) : a.n_experts;
+    const int n_act = listed ? list_active(act, a, wave, lane, S::WAVES) : a.n_experts;
     __syncthreads();
     for (int item = blockIdx.x; item < n_act * slabs_per_expert; item += gridDim.x) {
         // (read from LDS: the same in every lane, and kept in a scalar register like the arithmetic form)
@@ -355,7 +362,7 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     const int per_expert = GLU ? groups : (groups + 1) / 2;   // items per expert
     const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
     uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-    const int n_items = list_active(act, a, wave, lane) * per_expert;
+    const int n_items = list_active(act, a, wave, lane, KS_WAVES) * per_expert;
     __syncthreads();
     for (int base = blockIdx.x * IPB; base < n_items; base += gridDim.x * IPB) {
         int maxn = 0;
@@ -469,13 +476,13 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
 }
 
 size_t ks_shm(bool glu) {
-    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_LISTED + 8) * 2;
+    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_LISTED + 8) * 2 + 16 * 4;
 }
 
 template <int NT, int W> size_t mt_shm(bool glu) {
     using S = mt_shape<NT, W>;
     return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) S::WAVES * 2 * WAVE_LDS_WORDS * 4 + (size_t) 2 * S::TOK * MT_BSTRIDE * 2 +
-           (MT_MAX_LISTED + 8) * 2;
+           (MT_MAX_LISTED + 8) * 2 + 16 * 4;
 }
 
 // ---------------------------------------------------------------- GEMV
