@@ -146,7 +146,7 @@ def graph_us(fn, n: int = 16, reps: int = 30) -> float:
     return float(np.median(d)) * 1e3 / n
 
 
-def decode_step(ops, head, randw, randx, K: int, n_layers: int = 40, n_sets: int = 4) -> dict:
+def decode_step(ops, head, randw, randx, K: int, n_layers: int = 40, n_sets: int = 4, head_tiles=None) -> dict:
     """One decode step of the 35B-A3B shape as a single HIP graph: n_layers x (qkv 5120 x K, o K x 4096, router, top-8 of
     256 experts, fused gate/up, down, combine, shared expert) + the output projection.  n_sets distinct weight sets are
     used in turn and every layer's input is the previous layer's output (re-normalised), so that layers sharing a
@@ -167,9 +167,10 @@ def decode_step(ops, head, randw, randx, K: int, n_layers: int = 40, n_sets: int
         sets.append(d)
     touched = n_layers * (nbytes["qkv"] + nbytes["o"] + nbytes["router"] + nbytes["sh_gate_up"] + nbytes["sh_down"]
                           + (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * topk // E)
-    head_bytes = head.plane.numel() + head.aux.numel()
     res = {"layers": n_layers, "weight_sets": n_sets}
-    for T in (1, 4):
+    for T, hd, tag in ((1, head, ""), (4, head, ""), (16, head, ""), (16, head_tiles, "_head_as_tiles")):
+        if hd is None:
+            continue
         xin = [randx(T, K) for _ in range(4)]
         xbuf = xin[0].clone()
 
@@ -185,7 +186,7 @@ def decode_step(ops, head, randw, randx, K: int, n_layers: int = 40, n_sets: int
                 y = ops.moe_experts(h, w["gate"], w["up"], w["down"], wts, ids, E)
                 sh = ops.mmv(ops.mmv_glu(h, w["sh_gate_up"]), w["sh_down"], out_dtype=torch.bfloat16)
                 h = torch.nn.functional.rms_norm(h + y + sh, (K,))
-            return ops.linear(h, head)
+            return ops.linear(h, hd)
 
         step()
         torch.cuda.synchronize()
@@ -200,8 +201,8 @@ def decode_step(ops, head, randw, randx, K: int, n_layers: int = 40, n_sets: int
         d, _ = time_kernel(replay, 12, 3)
         t = float(np.median(d)) * 1e3
         # experts touched: at most T * top-k distinct ones per layer
-        tb = touched + (n_layers * (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * topk // E) * (T - 1) + head_bytes
-        res[f"batch{T}"] = {"graph_us": round(t, 1), "compressed_bytes_touched_upper_bound": int(tb),
+        tb = touched + (n_layers * (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * topk // E) * (min(T, E // topk) - 1) + hd.plane.numel() + hd.aux.numel()
+        res[f"batch{T}{tag}"] = {"graph_us": round(t, 1), "compressed_bytes_touched_upper_bound": int(tb),
                             "GBps": round(tb / t / 1e3, 1), "tokens_per_s": round(T / t * 1e6, 1)}
         del graph
     return res
@@ -237,6 +238,7 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
         batches[str(T)] = {"units_of_16_rows_us": round(base, 1), "path": "gemv" if T <= 8 else "dequant + BF16 GEMM",
                            "tiles_us": round(graph_us(lambda i: ops.mmv(xT, tiles[i & 1]), 4, 10), 1)}
     out["lm_head_batches"] = {"tiles": tdesc, "tiles_bytes": tbytes, "by_batch": batches}
+    head_tiles = tiles[0]
     del tiles
     # small NIBBLE matrices
     for rows, k in ((512, 2048), (2048, 512)):
@@ -300,7 +302,7 @@ def suite(ops, w_head, head_copies, x1, K: int) -> dict:
             out[f"moe_prefill_T{T}_gate_up_{engine}"] = {
                 "gate_up": gdesc, "us": round(t, 1), "gate_up_us": round(t_gu, 1), "TFLOPs": round(flops / t / 1e6, 2),
                 "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / 2500.0, 4), "tokens_per_s": round(T / t * 1e6, 0)}
-    out["decode_step"] = decode_step(ops, head_copies[0], randw, randx, K)
+    out["decode_step"] = decode_step(ops, head_copies[0], randw, randx, K, head_tiles=head_tiles)
     return out
 
 
