@@ -100,6 +100,31 @@ int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * 
 int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
                       int32_t * ids, float * weights, void * stream);
 
+/* ---- load-time conversion and the registry of resident tensors: the reference's llama.cpp adapter without ggml types
+ * (engines/llamacpp/patches/0002-ggml-cuda-thin-BF16N-adapter-over-the-shared-core.patch).  An engine stores a converted
+ * tensor as rows * K bytes of device memory (the plane); the aux buffer is allocated here and found again by the
+ * address of the tensor's data.  These calls allocate and synchronise: load time only, never under graph capture. ---- */
+/* ggml_backend_cuda_bf16n_choose, patch 0002:258-268: 0 = stay BF16, 1 = NIBBLE, 2 = Huffman family.  Never fails. */
+int bf16n_adapter_choose(int64_t rows, int64_t K, int64_t n_matrices, const char * mode, int64_t dense_min, int expert, int engine);
+/* ggml_backend_cuda_bf16n_convert, patch 0002:271-329: encode the host BF16 tensor (n_matrices x rows_per_matrix x K)
+ * with the layout the engine's policy picks for format_tag (1 NIBBLE, 2 Huffman family; matrix_core_order: the policy's
+ * dense_frag_order), copy the plane into tensor_data (device, rows * K bytes, 16-byte aligned), allocate and fill the
+ * aux buffer, register the tensor under `owner`, decode it on the device and compare every weight with the source.
+ * *roundtrip_ok = 1 when they are identical; verbose: one line per tensor on stderr as the reference prints. */
+int bf16n_adapter_convert(void * tensor_data, const void * bf16_host, int64_t rows_per_matrix, int64_t K, int64_t n_matrices,
+                          int format_tag, int engine, int matrix_core_order, const void * owner, const char * name, int verbose,
+                          int * roundtrip_ok);
+/* the verify step alone (patch 0002:309-322; roundtrip_equal of vllm_bf16n/ops.py): device decode against a host source */
+int bf16n_verify_roundtrip(const bf16n_weight * w, const uint16_t * bf16_host, int * ok);
+/* a tensor the caller encoded and uploaded itself joins the registry (its aux buffer stays the caller's) */
+int bf16n_adapter_register(const bf16n_weight * w, const void * owner);
+/* lookup, patch 0002:73-92: the registered tensor whose plane holds address p (any row start: views of whole rows);
+ * *found = 0 if none.  The weight is returned by value. */
+int bf16n_adapter_lookup(const void * p, bf16n_weight * out, int64_t * row0, int * found);
+/* ggml_cuda_bf16n_free, patch 0002:121-132: drop every tensor of `owner` (before its buffer is freed); *n: how many */
+int bf16n_adapter_release(const void * owner, int * n);
+int bf16n_adapter_count(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,7 +16,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libbf16n_hip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip"]
+SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "adapter.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall", "-Wno-unused-function"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -28,7 +28,7 @@ def _compile(src: str, force: bool) -> str:
         os.path.join(ROOT, "include", "bf16n_c.h"), os.path.join(ROOT, "include", "bf16n", "format.h")]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
         return obj
-    cmd = [HIPCC] + COMMON + (HIP_FLAGS if src.endswith(".hip") else ["-x", "hip", "--offload-arch=gfx950"] if src == "capi.cpp" else []) + ["-c", path, "-o", obj]
+    cmd = [HIPCC] + COMMON + (HIP_FLAGS if src.endswith(".hip") else ["-x", "hip"] + HIP_FLAGS if src == "adapter.cpp" else ["-x", "hip", "--offload-arch=gfx950"] if src == "capi.cpp" else []) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         sys.stderr.write(r.stdout + r.stderr)

@@ -10,6 +10,7 @@
 
 #include <climits>
 #include <cstdint>
+#include <functional>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -65,6 +66,17 @@ int guarded(F && f) {
         return BF16N_ERUNTIME;
     }
 }
+
+} // namespace
+
+namespace bf16n {
+namespace impl {
+// for the other translation units of the C ABI: run f, map exceptions to a status and the calling thread's message
+int report(const std::function<void()> & f) { return guarded(f); }
+} // namespace impl
+} // namespace bf16n
+
+namespace {
 
 // launch.cu:261-268
 void check_weight(const bf16n_weight & w) {
