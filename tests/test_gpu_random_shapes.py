@@ -88,3 +88,56 @@ def test_random_configuration(ops, K, fmt, R, cm, w64, rows_per, E, T, seed):
         err = np.abs(y - ref)
     assert np.all(err[np.broadcast_to(ok, err.shape)] <= (1e-5 * bound + 1e-30)[np.broadcast_to(ok, err.shape)])
     assert np.all(err[np.broadcast_to(ok, err.shape)] <= (1e-3 * np.abs(ref) + 1e-5)[np.broadcast_to(ok, err.shape)])
+
+
+def batched_cases(n: int):
+    """Batched products on the tile layout: K, rows per expert, experts, top-k and tokens drawn so that all shapes of the
+    kernel come up (K split over wavefronts for few active experts, 32-token passes, 128-token passes)."""
+    rng = np.random.default_rng(424242)
+    out = []
+    for _ in range(n):
+        K = int(rng.choice([512, 1024, 1536, 2048, 3072, 4096]))
+        N = 32 * int(rng.integers(1, 18))
+        E = int(rng.choice([1, 2, 7, 16, 40]))
+        k = int(rng.integers(1, min(E, 4) + 1))
+        T = int(rng.choice([1, 2, 5, 17, 33, 70, 150, 300]))
+        out.append((K, N, E, k, T, bool(rng.random() < 0.4), bool(rng.random() < 0.3), int(rng.integers(1 << 30))))
+    return out
+
+
+@pytest.mark.parametrize("K,N,E,k,T,glu,per_slot,seed", batched_cases(48))
+def test_random_batched_products_on_tiles(ops, K, N, E, k, T, glu, per_slot, seed):
+    from conftest import GEMV_REL
+    from test_gpu_mm_ids import reference
+
+    rng = np.random.default_rng(seed)
+    wb = synth.weights(E * N, K, seed)
+    w = enc(ops, wb, HP, 32, False, True)
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    if E > 2 and T > 40:
+        ids[:, 0] = np.where(rng.random(T) < 0.6, 0, ids[:, 0])       # one busy expert: several passes
+        for t in range(T):                                            # no repeats inside a token
+            if k > 1 and ids[t, 0] in ids[t, 1:]:
+                ids[t, 0] = next(e for e in range(E) if e not in ids[t, 1:])
+    per_slot = per_slot and not glu
+    xb = synth.activations(T * (k if per_slot else 1), K, seed + 1).reshape((T, k, K) if per_slot else (T, K))
+    xf = synth.bf16_bits_to_f32(xb)
+    xt, it = tbf16(xb), torch.from_numpy(ids).cuda()
+    y, s = reference(synth.bf16_bits_to_f32(wb), xf, ids, N, per_slot)
+    if not glu:
+        got = ops.moe_mm_ids(xt, it, w, E).cpu().numpy()
+        assert np.all(np.abs(got - y) <= GEMV_REL * s + 1e-30)
+        assert np.all(np.abs(got - y) <= 1e-3 * np.abs(y) + 1e-5)
+        got16 = ops.moe_mm_ids(xt, it, w, E, out_dtype=torch.bfloat16)
+        assert np.array_equal(bits(got16), synth.f32_to_bf16_bits(got))
+    else:
+        ub = synth.weights(E * N, K, seed + 2)
+        u = enc(ops, ub, HP, 32, False, True)
+        fused = ops.moe_mm_ids(xt, it, w, E, up=u).cpu().numpy()
+        y2, s2 = reference(synth.bf16_bits_to_f32(ub), xf, ids, N, False)
+        sg = 1.0 / (1.0 + np.exp(-y))
+        ref = y2 * y * sg
+        # first-order bound of silu(g) * u under |dg| <= eps sum|w x| (gate) and |du| <= eps sum|w x| (up), plus one rounding
+        dsilu = np.abs(sg * (1.0 + y * (1.0 - sg)))
+        tol = GEMV_REL * (np.abs(y2) * dsilu * s + np.abs(y * sg) * s2) * 1.5 + 2.0 ** -22 * np.abs(ref) + 1e-12
+        assert np.all(np.abs(fused - ref) <= tol)
