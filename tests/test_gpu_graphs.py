@@ -92,12 +92,16 @@ def test_moe_layer_graph(ops, T):
     assert float((out.float() - ref.float()).abs().max()) <= 2e-2 * scale
 
 
-def test_batched_moe_graph(ops):
-    # T = 64: routing lists, fused gate/up + SwiGLU and down run as batched kernels inside the graph
-    E, k, K, N, T = 8, 2, 2048, 512, 64
-    gate = enc(ops, synth.weights(E * N, K, 101), HP, 4, False, True)
-    up = enc(ops, synth.weights(E * N, K, 102), HP, 4, False, True)
-    down = enc(ops, synth.weights(E * K, N, 103), HP, 16, False, True)
+@pytest.mark.parametrize("layout,E,T", [("units", 8, 64), ("tiles", 8, 300), ("tiles", 8, 64), ("tiles", 40, 12)])
+def test_batched_moe_graph(ops, layout, E, T):
+    # routing lists, fused gate/up + SwiGLU and down run as batched kernels inside the graph: 4- and 16-row wave64 units
+    # (decode -> LDS tile -> MFMA) and the tile layout in its three shapes (128-token passes at 300 tokens, 32-token
+    # passes at 64, K split over wavefronts at 12 tokens of 40 experts); the routing changes from replay to replay
+    k, K, N = 2, 2048, 512
+    r_gu, r_dn = (4, 16) if layout == "units" else (32, 32)
+    gate = enc(ops, synth.weights(E * N, K, 101), HP, r_gu, False, True)
+    up = enc(ops, synth.weights(E * N, K, 102), HP, r_gu, False, True)
+    down = enc(ops, synth.weights(E * K, N, 103), HP, r_dn, False, True)
     assert ops.mm_ids_supported(gate, up) and ops.mm_ids_supported(down)
     x = tbf16(synth.activations(T, K, 104))
     logits = torch.randn((T, E), generator=torch.Generator().manual_seed(1)).cuda()
