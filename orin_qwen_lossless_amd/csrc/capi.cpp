@@ -110,10 +110,10 @@ dev::cols make_cols(const bf16n_mmv_args & a) { // launch.cu:69-84
     return p;
 }
 
-// dense products of a tile-layout matrix that go through the matrix cores: BF16 activations, rows enough to fill the
-// GPU, and the 16-byte alignment of x rows and y columns that the kernel's vector accesses need
+// dense products of a tile-layout matrix that go through the matrix cores: BF16 activations (or a few FP32 columns),
+// rows enough to fill the GPU, and the 16-byte alignment of x rows and y columns that the kernel's vector accesses need
 bool tile_dense_mm(const bf16n_weight & w, const bf16n_mmv_args & a) {
-    if (a.ids || !a.x_bf16 || !dev::tile_mm_dense_pays(w, a.nrows, g_cus)) {
+    if (a.ids || !dev::tile_mm_dense_pays(w, a.nrows, g_cus)) {
         return false;
     }
     const int64_t ya = a.y_bf16 ? 8 : 16;
@@ -198,9 +198,15 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
         }
         const dev::cols p = make_cols(*a);
         if (dev::is_tile_layout(*w) && tile_dense_mm(*w, *a)) {
-            // a large dense matrix, BF16 activations: any number of columns through the matrix cores
-            dev::launch_tile_mm_dense(*w, a->row0, a->nrows, a->x, a->x_tok / 2, a->ncols, a->y, a->y_bf16 != 0,
-                                      a->y_tok / (a->y_bf16 ? 2 : 4), g_cus, (hipStream_t) stream);
+            // a large dense matrix through the matrix cores: any number of BF16 columns, or up to ten FP32 columns as
+            // three BF16 components each
+            const int per_launch = a->x_bf16 ? a->ncols : dev::TILE_DENSE_F32_COLS;
+            for (int c0 = 0; c0 < a->ncols; c0 += per_launch) {
+                const int nc = a->ncols - c0 < per_launch ? a->ncols - c0 : per_launch;
+                dev::launch_tile_mm_dense(*w, a->row0, a->nrows, (const char *) a->x + c0 * a->x_tok, a->x_bf16 != 0,
+                                          a->x_tok / (a->x_bf16 ? 2 : 4), nc, (char *) a->y + c0 * a->y_tok, a->y_bf16 != 0,
+                                          a->y_tok / (a->y_bf16 ? 2 : 4), g_cus, (hipStream_t) stream);
+            }
         } else if (dev::is_tile_layout(*w)) {
             dev::launch_tile_mmv(*w, nullptr, p, a->ncols, a->x_bf16 != 0, (hipStream_t) stream);
         } else if (is_w64(*w)) {

@@ -138,6 +138,27 @@ template <int NT, int W> struct mt_shape {
         }                                     \
     } while (0)
 
+// Component c (0, 1, 2) of eight FP32 activations as BF16: x = hi + mid + lo exactly (three times eight significant
+// bits cover the 24 of an FP32 value), each the nearest BF16 of what the previous ones leave.  A product of FP32
+// activations becomes three columns of BF16 products, exact in FP32, added at the end.
+__device__ __forceinline__ uint4 split_bf16(const uint4 a, const uint4 b, int c) {
+    const uint32_t in[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t out[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float x = __uint_as_float(in[i]);
+        const uint32_t hi = f32_to_bf16_rne(x);
+        const float hf = __uint_as_float(hi << 16);
+        const bool fin = (hi & 0x7F80u) != 0x7F80u;               // infinities and NaNs stay in the first component alone
+        const float r1 = fin ? x - hf : 0.f;
+        const uint32_t mid = f32_to_bf16_rne(r1);
+        const float r2 = r1 - __uint_as_float(mid << 16);
+        const uint32_t lo = f32_to_bf16_rne(r2);
+        out[i] = c == 0 ? hi : c == 1 ? mid : lo;
+    }
+    return make_uint4(out[0] | (out[1] << 16), out[2] | (out[3] << 16), out[4] | (out[5] << 16), out[6] | (out[7] << 16));
+}
+
 struct mm_args {
     const uint16_t * x; int64_t x_row;
     const int32_t * ids_src1, * ids_dst, * bounds; // all null: one dense matrix, token j reads row j of x and writes column j
@@ -180,9 +201,13 @@ __device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, in
 // (GLU) or two row groups of the matrix, and keeps their 2 x NT accumulator blocks (32 rows x 32 tokens each) for
 // the whole pass over the expert's K columns.  Per step a chain yields two A operands (32 rows x 16 columns); the B
 // operands (16 columns x 32 tokens) come from the staged activations and are used by both chains.
-template <bool GLU, int NT, int W>
+// XF32 (dense products of up to ten FP32 activation columns, 32-token shape): a.x holds FP32 rows and token 3 j + c of
+// the pass is component c of column j (split_bf16); the three accumulator columns of a token are added before the store.
+template <bool GLU, int NT, int W, bool XF32 = false>
 __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
     using S = mt_shape<NT, W>;
+    static_assert(!XF32 || (NT == 1 && W == 16 && !GLU), "FP32 activations: the dense 32-token shape only");
+    constexpr int XB = XF32 ? 4 : 2;                          // bytes per activation
     constexpr int NM = GLU ? 2 : 1;
     extern __shared__ __align__(16) uint32_t shm[];
     uint32_t * lut = shm;
@@ -218,11 +243,13 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
             const int left = n - tp, nt = NT == 1 ? 1 : left >= S::TOK ? NT : (left + 31) >> 5;
             const int btk = tp + b_tok;
             const int bj = j0 + (btk < n ? btk : 0);
-            const uint16_t * xsrc = a.x + (int64_t) (a.ids_src1 ? a.ids_src1[bj] : bj) * a.x_row + S::CPT * b_part;
+            const int bcomp = XF32 ? bj % 3 : 0;
+            const char * xsrc = (const char *) a.x + ((int64_t) (XF32 ? bj / 3 : a.ids_src1 ? a.ids_src1[bj] : bj) * a.x_row + S::CPT * b_part) * XB;
             uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + S::CPT * b_part;
+            constexpr int VLD = XF32 ? 2 * S::VPT : S::VPT;       // uint4 loads per thread and block
             uint4 f0, f1, f2, f3;
             if (stager) {
-                MT_STAGE_LOAD(S::VPT, f0, f1, f2, f3, (const uint4 *) xsrc);
+                MT_STAGE_LOAD(VLD, f0, f1, f2, f3, (const uint4 *) xsrc);
             }
             tchain_t<S::DEPTH> ch[2];
             if (live) {
@@ -242,7 +269,11 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                 }
             }
             if (stager) {
-                MT_STAGE_STORE(S::VPT, f0, f1, f2, f3, (uint4 *) bdst);
+                if constexpr (XF32) {
+                    *(uint4 *) bdst = split_bf16(f0, f1, bcomp);
+                } else {
+                    MT_STAGE_STORE(S::VPT, f0, f1, f2, f3, (uint4 *) bdst);
+                }
             }
             __syncthreads();
 #pragma unroll 1
@@ -255,7 +286,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                 const int nxt = hs + 1 < halves ? hs + 1 : hs;
                 uint4 b0, b1, b2, b3;
                 if (stager) {
-                    MT_STAGE_LOAD(S::VPT, b0, b1, b2, b3, (const uint4 *) (xsrc + nxt * MT_HK));
+                    MT_STAGE_LOAD(VLD, b0, b1, b2, b3, (const uint4 *) (xsrc + nxt * MT_HK * XB));
                 }
                 if (live) {
                     if ((hs & 1) == 0) {
@@ -294,17 +325,33 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                     }
                 }
                 if (stager) {
-                    MT_STAGE_STORE(S::VPT, b0, b1, b2, b3, (uint4 *) (bdst + ((hs + 1) & 1) * (S::TOK * MT_BSTRIDE)));
+                    uint4 * bn = (uint4 *) (bdst + ((hs + 1) & 1) * (S::TOK * MT_BSTRIDE));
+                    if constexpr (XF32) {
+                        *bn = split_bf16(b0, b1, bcomp);
+                    } else {
+                        MT_STAGE_STORE(S::VPT, b0, b1, b2, b3, bn);
+                    }
                 }
                 __syncthreads();
+            }
+            if constexpr (XF32) {
+                // the three components of a token sit in adjacent lanes of a half: their sum lands in the first
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const float v = acc[c][0][i];
+                        acc[c][0][i] = (v + __shfl_down(v, 1, 32)) + __shfl_down(v, 2, 32);
+                    }
+                }
             }
             // accumulator element i of a lane: row 8 (i / 4) + 4 (lane / 32) + i % 4 of the group, token lane % 32
             if (live) {
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
                     const int tk = tp + 32 * t + l32;
-                    if (t < nt && tk < n) {
-                        const int64_t col = (int64_t) (a.ids_dst ? a.ids_dst[j0 + tk] : tk) * a.dst_col;
+                    if (t < nt && tk < n && (!XF32 || tk % 3 == 0)) {
+                        const int64_t col = (int64_t) (XF32 ? tk / 3 : a.ids_dst ? a.ids_dst[j0 + tk] : tk) * a.dst_col;
 #pragma unroll
                         for (int c = 0; c < (GLU ? 1 : 2); c++) {
                             if (c == 1 && !has1) {
@@ -695,6 +742,7 @@ void tile_init() {
     mt_attr<false, 4, 8>();
     mt_attr<true, 1, 16>();
     mt_attr<false, 1, 16>();
+    (void) hipFuncSetAttribute((const void *) k_mm_tile<false, 1, 16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<1, 16>(false));
     ks_attr<true, 2>(); ks_attr<false, 2>(); ks_attr<true, 4>(); ks_attr<false, 4>();
     ks_attr<true, 8>(); ks_attr<false, 8>(); ks_attr<true, 16>(); ks_attr<false, 16>();
 }
@@ -783,19 +831,27 @@ bool tile_mm_dense_pays(const bf16n_weight & w, int64_t nrows, int cus) {
     return nrows / (TILE_R * 2 * 16) >= cus / 2 && w.K >= 1024;
 }
 
-void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x_bf16, int64_t x_row, int ncols, void * y,
-                          bool y_bf16, int64_t y_col, int cus, hipStream_t stream) {
+void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x, bool x_bf16, int64_t x_row, int ncols,
+                          void * y, bool y_bf16, int64_t y_col, int cus, hipStream_t stream) {
     mm_args a;
-    a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
+    a.x = (const uint16_t *) x; a.x_row = x_row;
     a.ids_src1 = a.ids_dst = a.bounds = nullptr;
     a.dst = (char *) y; a.dst_col = y_col; a.dst_bf16 = y_bf16;
-    a.rows = nrows; a.n_experts = 1; a.n_tok = ncols;
+    a.rows = nrows; a.n_experts = 1; a.n_tok = x_bf16 ? ncols : 3 * ncols;
     // a view of the row range: the plane bytes and the unit bases of its first tile onwards
     bf16n_weight v = w;
     const int64_t tile0 = row0 / TILE_R * (w.K / TILE_K);
     v.plane += tile0 * T_BYTES;
     v.off_b += (uint64_t) tile0 * 4;
-    if (ncols <= 32) {
+    if (!x_bf16) {
+        if (ncols > TILE_DENSE_F32_COLS) {
+            throw std::invalid_argument("bf16n: at most 10 FP32 columns per dense tile product");
+        }
+        using S = mt_shape<1, 16>;
+        const int64_t items = mt_items<16>(a, false);
+        hipLaunchKernelGGL((k_mm_tile<false, 1, 16, true>), dim3((unsigned) (items < cus ? items : cus)), dim3(S::THREADS),
+                           (mt_shm<1, 16>(false)), stream, v, v, a);
+    } else if (ncols <= 32) {
         mt_launch<1, 16>(v, nullptr, a, cus, stream);
     } else {
         mt_launch<4, 8>(v, nullptr, a, cus, stream);

@@ -40,8 +40,9 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
                         int64_t n_pairs, int cus, hipStream_t stream);
 
 bool tile_mm_dense_pays(const bf16n_weight & w, int64_t nrows, int cus);
-void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x_bf16, int64_t x_row, int ncols, void * y,
-                          bool y_bf16, int64_t y_col, int cus, hipStream_t stream);
+constexpr int TILE_DENSE_F32_COLS = 10; // FP32 columns per dense tile product: three BF16 components each, 32 per pass
+void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x, bool x_bf16, int64_t x_row, int ncols,
+                          void * y, bool y_bf16, int64_t y_col, int cus, hipStream_t stream);
 
 // MoE glue (kernels_moe.hip)
 void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int cus, hipStream_t stream);

@@ -98,9 +98,9 @@ bool choose(int64_t rows, int64_t K, int64_t n, int engine, int mode, int64_t de
         } else if (dense_frag_order && rows % TILE_R == 0 && rows >= MI355X_DENSE_TILE_ROWS && K >= 2 * CHUNK) {
             // dense matrices with enough rows to give every CU whole blocks of row groups, when the caller asks for
             // the matrix-core order (the counterpart of the reference's fragment order for dense tensors): products
-            // with BF16 activations then run on the matrix cores for any batch, 1 to 32 tokens in the time of one
-            // decode of the matrix.  At batch 1 that is within a few per cent of the 16-row units below (the tiles
-            // are 4 % more bytes); FP32 activations take the slower tile GEMV, hence on request only.
+            // then run on the matrix cores for any batch, 1 to 32 BF16 tokens (10 FP32 tokens, as three BF16
+            // components each) in the time of one decode of the matrix.  At batch 1 that is a few per cent behind the
+            // 16-row units below with BF16 activations (the tiles are 4 % more bytes), hence on request.
             out = {FMT_HUFPAIR, TILE_R, false, false, true};
             return true;
         } else {

@@ -126,12 +126,17 @@ def test_full_size_tiles_dense_product_any_batch(ops, head_tiles, T):
     y16 = ops.mmv(x, enc, out_dtype=torch.bfloat16)
     assert torch.equal(y16[:, keep], y[:, keep].to(torch.bfloat16))
     assert T > ops.gemv_max_tokens(enc) or torch.equal(ops.linear(x, enc).view(torch.int16), y16.view(torch.int16))
-    # FP32 activations keep their precision: they go through the GEMV kernel, within the same bound
-    if T == 1:
-        xf = torch.randn((1, K), generator=g, device="cuda")
+    # FP32 activations keep their precision: each column goes in as three BF16 components whose products are exact
+    # (ten columns per launch); within the same bound, and every column equal to its single-column launch
+    if T <= 33:
+        xf = torch.randn((T, K), generator=g, device="cuda") * torch.exp(torch.randn((T, K), generator=g, device="cuda"))
         yf = ops.mmv(xf, enc)
         rf, bf = fp64_product(w, xf)
         assert bool(((yf.double() - rf).abs()[:, keep] <= 1e-5 * bf[:, keep]).all())
+        for t in {0, T // 2, T - 1}:
+            assert torch.equal(ops.mmv(xf[t: t + 1], enc)[0].view(torch.int32), yf[t].view(torch.int32))
+        # activations that are BF16 values give the BF16 path's bits (the other two components are zero)
+        assert torch.equal(ops.mmv(x.float(), enc)[:, keep], y[:, keep])
 
 
 def test_full_size_tiles_row_range_and_strides(ops, head_tiles):
