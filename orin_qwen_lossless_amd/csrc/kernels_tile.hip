@@ -244,7 +244,8 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
             const int btk = tp + b_tok;
             const int bj = j0 + (btk < n ? btk : 0);
             const int bcomp = XF32 ? bj % 3 : 0;
-            const char * xsrc = (const char *) a.x + ((int64_t) (XF32 ? bj / 3 : a.ids_src1 ? a.ids_src1[bj] : bj) * a.x_row + S::CPT * b_part) * XB;
+            // (element pointers, not bytes: the byte form costs the BF16 instances five more spilled registers)
+            const uint16_t * xsrc = a.x + ((int64_t) (XF32 ? bj / 3 : a.ids_src1 ? a.ids_src1[bj] : bj) * a.x_row + S::CPT * b_part) * (XB / 2);
             uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + S::CPT * b_part;
             constexpr int VLD = XF32 ? 2 * S::VPT : S::VPT;       // uint4 loads per thread and block
             uint4 f0, f1, f2, f3;
@@ -286,7 +287,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                 const int nxt = hs + 1 < halves ? hs + 1 : hs;
                 uint4 b0, b1, b2, b3;
                 if (stager) {
-                    MT_STAGE_LOAD(VLD, b0, b1, b2, b3, (const uint4 *) (xsrc + nxt * MT_HK * XB));
+                    MT_STAGE_LOAD(VLD, b0, b1, b2, b3, (const uint4 *) (xsrc + nxt * MT_HK * (XB / 2)));
                 }
                 if (live) {
                     if ((hs & 1) == 0) {
