@@ -45,19 +45,27 @@ bool reaches(int64_t rows, int64_t K, int64_t n, int64_t threshold) noexcept {
     return rows >= rows_needed;
 }
 
-// mi355x dense: one wave64 decodes one unit and a launch wants several thousand units in flight (256 CUs x 8-16
-// waves), so take the largest R in {16, 8, 4, 2} that still leaves at least 4096 units, else the largest that leaves
-// 1024, else 2 (the wave64 layout needs an even number of chunks per unit; R = 1 only when rows is odd).
+// mi355x dense: one wavefront decodes one unit, and 256 CUs hold 4096 wavefronts at once.  A matrix with more rows than
+// that streams: it takes the longest units (16 rows: fewest unit starts, fewest bytes).  A smaller one is a single
+// round of wavefronts whose time is the length of one unit's decode chain, so it takes the shortest units that still
+// fit the round, i.e. the smallest R with rows / R <= 4096 (measured, K = 2048: 5120 rows 7.9 us with R = 2 against
+// 9.2 with R = 4 and 8.9 with R = 1; 2048 x 4096: 6.7 us with R = 1 against 7.7 with R = 2), at 6 % more bytes per
+// halving.  Units of at least 4096 weights: every unit ends with about 512 bytes of stream words that were requested
+// and never used, one bit per weight at that size (units of 2048 weights compress to 0.82 of BF16 instead of 0.70-0.74).
+// The wave64 layout needs whole loop bodies per unit: R a multiple of 4 for K = 512, of 2 for K = 1024.
 int mi355x_dense_unit_rows(int64_t rows, int64_t K) noexcept {
-    const int candidates[] = {16, 8, 4, 2};
-    for (int64_t floor_units : {(int64_t) 4096, (int64_t) 1024, (int64_t) 1}) {
-        for (int r : candidates) {
-            if (rows % r == 0 && rows / r >= floor_units) {
-                return r;
-            }
+    const int64_t C = K / CHUNK;
+    const int step = C == 1 ? 4 : C == 2 ? 2 : 1;
+    for (int r : {1, 2, 4, 8, 16}) {
+        if (r % step == 0 && rows % r == 0 && rows / r <= 4096 && r * K >= 4096) {
+            return r;
         }
     }
-    (void) K;
+    for (int r : {16, 8, 4, 2}) {
+        if (rows % r == 0) {
+            return r;
+        }
+    }
     return 1;
 }
 

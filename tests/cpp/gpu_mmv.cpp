@@ -17,7 +17,7 @@ static float bf16_to_f32(uint16_t b) { uint32_t u = (uint32_t) b << 16; float f;
 static uint16_t f32_to_bf16(float f) { uint32_t u; std::memcpy(&u, &f, 4); return (uint16_t) ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16); }
 
 int main() {
-    const int64_t rows = 4096, K = 2048;
+    const int64_t rows = 8192, K = 2048;
     std::vector<uint16_t> w(rows * K), x(K);
     uint64_t s = 0x9E3779B97F4A7C15ull;
     auto rnd = [&]() { s ^= s << 13; s ^= s >> 7; s ^= s << 17; return (double) (s >> 11) / 9007199254740992.0; };

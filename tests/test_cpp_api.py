@@ -40,7 +40,7 @@ def test_cpp_api_on_the_device(tmp_path):
                     os.path.join(ROOT, "tests", "cpp", "gpu_mmv.cpp"), "-o", exe, "-L" + LIBDIR, "-lbf16n_hip", "-Wl,-rpath," + LIBDIR],
                    check=True, capture_output=True, timeout=300)
     out = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=120).stdout
-    assert "encoded format 3 R 4 flags 4" in out       # 4096 x 2048 under the mi355x policy: wave64 units of 4 rows
+    assert "encoded format 3 R 2 flags 4" in out       # 8192 x 2048 under the mi355x policy: one round of 4096 two-row wave64 units
     assert "dequant ok" in out and "mmv ok" in out
     assert "invalid_argument bf16n: dequant rows must be whole units" in out
 

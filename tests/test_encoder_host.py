@@ -164,10 +164,16 @@ def test_policy_contract_cases():
 
 
 def test_policy_mi355x():
-    # the benchmark shapes: wave64 row-major units, enough units for 256 CUs
+    # the benchmark shapes: wave64 row-major units; 16 rows for a matrix that streams (more than 4096 units), the
+    # shortest units that fit one round of 4096 wavefronts for a smaller one
     assert ops.choose(248320, 2048) == (HP, 16, False, False, True)
-    assert ops.choose(5120, 2048) == (HP, 4, False, False, True)
-    assert ops.choose(2048, 4096) == (HP, 2, False, False, True)
+    assert ops.choose(5120, 2048) == (HP, 2, False, False, True)
+    assert ops.choose(2048, 4096) == (HP, 1, False, False, True)
+    assert ops.choose(16384, 2048) == (HP, 4, False, False, True)
+    assert ops.choose(65536, 2048) == (HP, 16, False, False, True)
+    assert ops.choose(16384, 512) == (HP, 8, False, False, True)       # units of at least 4096 weights
+    assert ops.choose(4096, 2048) == (HP, 2, False, False, True)
+    assert ops.choose(8192, 1024) == (HP, 4, False, False, True)
     # experts: 32 x 256 tiles in matrix-core operand order where the rows per expert allow it, else units of 4 rows
     assert ops.choose(512, 2048, 256, expert=True) == (HP, 32, False, False, True)
     assert ops.choose(2048, 512, 256, expert=True) == (HP, 32, False, False, True)
@@ -180,7 +186,7 @@ def test_policy_mi355x():
     assert ops.choose(131040, 2048, dense_frag_order=True) == (HP, 16, False, False, True)   # too few rows
     assert ops.choose(248336, 2048, dense_frag_order=True) == (HP, 16, False, False, True)   # not a multiple of 32
     assert ops.choose(248320, 512, dense_frag_order=True) == (HP, 16, False, False, True)    # K too short
-    assert ops.choose(5120, 2048, dense_frag_order=True) == (HP, 4, False, False, True)
+    assert ops.choose(5120, 2048, dense_frag_order=True) == (HP, 2, False, False, True)
     # shapes without a wave64 GEMV instance keep the reference layouts
     assert ops.choose(16384, 1536) == (HP, 4, False, False, False)
     assert ops.choose(520, 1536, 8, expert=True) == (HP, 8, True, False, False)
