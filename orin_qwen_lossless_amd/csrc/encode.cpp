@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -692,15 +693,24 @@ int64_t tile32_index(int64_t vrow, int64_t vcol, int64_t K) {
 
 bool encode_tile32(const uint16_t * w, int64_t rows, int64_t K, encoded_buffers & out) {
     const int64_t vrows = rows * K / CHUNK;
-    std::vector<uint16_t> v((size_t) (rows * K));
+    const std::unique_ptr<uint16_t[]> v_mem(new uint16_t[(size_t) (rows * K)]); // not zeroed: every element is written below
+    uint16_t * const v = v_mem.get();
+    // tile32_index() row by row: the four weights of a (j, l) cell are adjacent in W
+    const int64_t slabs = K / TILE_K;
     parallel_blocks(vrows, 64, [&](int64_t r0, int64_t r1) {
         for (int64_t r = r0; r < r1; r++) {
-            for (int64_t c = 0; c < CHUNK; c++) {
-                v[(size_t) (r * CHUNK + c)] = w[tile32_index(r, c, K)];
+            const int64_t u = r / 16, s = (r % 16) / 2, h = r % 2, g = u / slabs, t = u % slabs;
+            const uint16_t * src = w + TILE_R * g * K + TILE_K * t + 32 * s + 8 * h;
+            uint16_t * dst = v + r * CHUNK;
+            for (int64_t j = 0; j < 4; j++) {
+                const uint16_t * sj = src + 16 * (j / 2) + 4 * (j % 2);
+                for (int64_t l = 0; l < 32; l++) {
+                    std::memcpy(dst + 128 * j + 4 * l, sj + l * K, 4 * sizeof(uint16_t));
+                }
             }
         }
     });
-    out.aux = encode_hufpair_w64(v.data(), vrows, CHUNK, 16, false);
+    out.aux = encode_hufpair_w64(v, vrows, CHUNK, 16, false);
     if (out.aux.empty()) {
         return false;
     }
@@ -708,7 +718,7 @@ bool encode_tile32(const uint16_t * w, int64_t rows, int64_t K, encoded_buffers 
     std::memcpy(&h, out.aux.data(), sizeof(h));
     h.K = (uint32_t) K; h.R = TILE_R; h.rows = (uint64_t) rows;
     std::memcpy(out.aux.data(), &h, sizeof(h));
-    write_plane(v.data(), vrows, CHUNK, 16, false, out.plane.data());
+    write_plane(v, vrows, CHUNK, 16, false, out.plane.data());
     out.format = FMT_HUFPAIR;
     out.R = TILE_R;
     return true;
