@@ -240,14 +240,17 @@ template <> __device__ __forceinline__ void x_chunk16<bf16_t>(const char * x, in
     }
 }
 
-// partial dot of (row gr, chunk c) with x; escaped weights read as +0 here.  The four per-position sums are combined
-// as in the reference (kernels.cuh:130-187), then over the 32 lanes; result in every lane of the half-wave.
-__device__ __forceinline__ float nib_chunk_dot(const nib_ptrs & w, int64_t gr, int C, int c, const uint4 T, const float (&xv)[16], int l32) {
+// the 16 weights of one lane in (row gr, chunk c) as 8 BF16 pairs; escaped weights read as +0 here
+__device__ __forceinline__ void nib_load_chunk(const nib_ptrs & w, int64_t gr, int C, int c, const uint4 T, int l32, uint32_t (&wp)[8]) {
     const int64_t K = (int64_t) C * CHUNK;
     const uint4 sm = *((const uint4 *) (w.plane + gr * K + c * CHUNK) + l32);
     const uint2 cd = *((const uint2 *) (w.codes + gr * (K / 2) + c * 256) + l32);
-    uint32_t wp[8];
     nib_chunk(sm, cd, T, wp);
+}
+
+// partial dot of a decoded chunk with x.  The four per-position sums are combined as in the reference
+// (kernels.cuh:130-187), then over the 32 lanes; result in every lane of the half-wave.
+__device__ __forceinline__ float nib_dot(const uint32_t (&wp)[8], const float (&xv)[16]) {
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -274,11 +277,18 @@ __device__ __forceinline__ float nib_escapes(const nib_ptrs & w, int64_t gr, con
 // NIBBLE GEMV; GLU 1: rows_per_matrix = [gate (nrows); up (nrows)] of one matrix; GLU 2: separate gate / up matrices.
 // These matrices are small (a few MB at most), so the launch is laid out for latency: one half-wave per (row, chunk)
 // pair, every load of a pair issued at once, the C chunk sums of a row combined through LDS in chunk order.
-template <typename TX, int GLU>
-__global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p) {
-    __shared__ float part[2][HALVES];
+// NC: columns per decode (dense batches: a (row, chunk) is decoded once for NC token columns, each of which gets the
+// bits of its single-column launch); columns past the last repeat it and are not stored.
+template <typename TX, int GLU, int NC>
+__global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, const int ncols) {
+    __shared__ float part[2][NC][HALVES];
     const int K = (int) w.K, C = K / CHUNK; // 1 .. 8
-    const col_view cv = col_setup(p, blockIdx.y);
+    col_view cv[NC];
+#pragma unroll
+    for (int j = 0; j < NC; j++) {
+        const int col = (int) blockIdx.y * NC + j;
+        cv[j] = col_setup(p, col < ncols ? col : ncols - 1);
+    }
     const nib_ptrs g = nibp(w, 0);
     const nib_ptrs u = GLU == 1 ? nibp(w, p.nrows) : nibp(w_up, 0);
     const int l32 = threadIdx.x & 31, half = threadIdx.x >> 5;
@@ -287,32 +297,36 @@ __global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16
     for (int64_t base = (int64_t) blockIdx.x * rpb; base < p.nrows; base += (int64_t) gridDim.x * rpb) {
         const bool live = lr < rpb && base + lr < p.nrows;
         const int64_t r = live ? base + lr : 0;
-        const int64_t gr = cv.rbase + r;
-        float xv[16];
-        x_chunk16<TX>(cv.x, c * CHUNK + 4 * l32, xv);
-        float v = nib_chunk_dot(g, gr, C, c, *(const uint4 *) (g.table + gr * 16), xv, l32);
-        float vu = 0.f;
+        const int64_t gr = cv[0].rbase + r; // dense batches share the rows; with expert ids NC is 1
+        uint32_t wg[8], wu[8];
+        nib_load_chunk(g, gr, C, c, *(const uint4 *) (g.table + gr * 16), l32, wg);
         if (GLU) {
-            vu = nib_chunk_dot(u, gr, C, c, *(const uint4 *) (u.table + gr * 16), xv, l32);
+            nib_load_chunk(u, gr, C, c, *(const uint4 *) (u.table + gr * 16), l32, wu);
         }
-        if (c == 0) {
-            v += nib_escapes<TX>(g, gr, cv.x, l32);
-            if (GLU) {
-                vu += nib_escapes<TX>(u, gr, cv.x, l32);
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            float xv[16];
+            x_chunk16<TX>(cv[j].x, c * CHUNK + 4 * l32, xv);
+            float v = nib_dot(wg, xv), vu = GLU ? nib_dot(wu, xv) : 0.f;
+            if (c == 0) {
+                v += nib_escapes<TX>(g, gr, cv[j].x, l32);
+                if (GLU) {
+                    vu += nib_escapes<TX>(u, gr, cv[j].x, l32);
+                }
             }
-        }
-        if (l32 == 0) {
-            part[0][half] = v;
-            part[1][half] = vu;
+            if (l32 == 0) {
+                part[0][j][half] = v;
+                part[1][j][half] = vu;
+            }
         }
         __syncthreads();
-        if (live && c == 0 && l32 == 0) {
-            float s = part[0][half], su = part[1][half];
+        if (live && c == 0 && l32 < NC && (int) blockIdx.y * NC + l32 < ncols) {
+            float s = part[0][l32][half], su = part[1][l32][half];
             for (int i = 1; i < C; i++) {
-                s += part[0][half + i];
-                su += part[1][half + i];
+                s += part[0][l32][half + i];
+                su += part[1][l32][half + i];
             }
-            store_y(cv.y, p.y_bf16, r, GLU ? su * silu(s) : s);
+            store_y(cv[0].y + l32 * p.y_tok, p.y_bf16, r, GLU ? su * silu(s) : s); // l32 > 0 only in dense batches
         }
         __syncthreads();
     }
@@ -375,11 +389,16 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
     const dim3 grid(grid_for(work, ncols, cus), ncols);
     if (w.format == FMT_NIBBLE) {
         const int rpb = HALVES / (int) (w.K / CHUNK);
-        const dim3 grid(grid_for((p.nrows + rpb - 1) / rpb * HALVES, ncols, cus), ncols);
-#define NIB(TX, G) hipLaunchKernelGGL((k_nib_mmv<TX, G>), grid, dim3(NT), 0, stream, w, wu, p)
+        // dense batches: four (two) columns share one decode of the matrix once there are columns enough to keep at
+        // least four groups of blocks (below that the columns run side by side on the idle CUs, which is faster)
+        const int nc = p.ids ? 1 : ncols >= 16 ? 4 : ncols >= 8 ? 2 : 1, ngroups = (ncols + nc - 1) / nc;
+        const dim3 grid(grid_for((p.nrows + rpb - 1) / rpb * HALVES, ngroups, cus), ngroups);
+#define NIBC(TX, G, N) hipLaunchKernelGGL((k_nib_mmv<TX, G, N>), grid, dim3(NT), 0, stream, w, wu, p, ncols)
+#define NIB(TX, G) do { if (nc == 4) NIBC(TX, G, 4); else if (nc == 2) NIBC(TX, G, 2); else NIBC(TX, G, 1); } while (0)
         if (x_bf16) { if (glu == 0) NIB(bf16_t, 0); else if (glu == 1) NIB(bf16_t, 1); else NIB(bf16_t, 2); }
         else        { if (glu == 0) NIB(float, 0);  else if (glu == 1) NIB(float, 1);  else NIB(float, 2); }
 #undef NIB
+#undef NIBC
         return;
     }
     const bool hp = w.format == FMT_HUFPAIR;

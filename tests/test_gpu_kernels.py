@@ -82,6 +82,25 @@ def test_wave64_column_groups_equal_single_columns(ops, oracle, K, R):
         assert torch.equal(ops.mmv(wide[:, :K], w), y1)
 
 
+@pytest.mark.parametrize("K", [512, 2048])
+def test_nibble_column_groups_equal_single_columns(ops, oracle, K):
+    # dense NIBBLE batches of 8 and more columns decode a (row, chunk) once for two or four columns; every column keeps
+    # the bits of its single-column launch, plain and with the fused SwiGLU, BF16 and FP32 activations, ragged tails
+    rows = 2 * 88
+    wb = synth.weights(rows, K, 5 * K)
+    wb[3, 7] = 0x4000                                          # 2.0: an exponent outside the row table, an escape
+    w = enc(ops, wb, NIB, 0, False, False)
+    xb = synth.activations(19, K, K + 3)
+    xf = synth.bf16_bits_to_f32(xb)
+    for x in (tbf16(xb), torch.from_numpy(xf).cuda()):
+        y1 = torch.cat([ops.mmv(x[t: t + 1], w) for t in range(19)])
+        g1 = torch.cat([ops.mmv_glu(x[t: t + 1], w) for t in range(19)])
+        check_gemv(oracle, y1[:4].cpu().numpy(), wb, xf[:4])
+        for T in (8, 9, 15, 16, 17, 19):
+            assert torch.equal(ops.mmv(x[:T], w), y1[:T]), (T, x.dtype)
+            assert torch.equal(ops.mmv_glu(x[:T], w), g1[:T]), (T, x.dtype)
+
+
 @pytest.mark.parametrize("fmt,R,cm,w64", LAYOUTS)
 def test_one_hot_activations_give_exact_weights(ops, fmt, R, cm, w64):
     K, rows = 2048, 64
