@@ -148,6 +148,20 @@ def test_mm_ids_few_tokens_per_expert(ops, K, N):
     assert np.all(np.abs(got2[:T] - got) <= 2 * GEMV_REL * s + 1e-30)
 
 
+def test_mm_ids_more_experts_than_a_block_lists(ops):
+    # above 1024 experts the blocks do not list the active ones (and K is not split): every expert's items are visited
+    E, k, T, K, N = 1500, 2, 40, 512, 32
+    wb = synth.weights(E * N, K, 77)
+    w = enc(ops, wb, HP, 32, False, True)
+    rng = np.random.default_rng(8)
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    ids[:, 0] = np.where(np.arange(T) % 2 == 0, 1499, ids[:, 0])     # the last expert takes half of the tokens
+    xb = synth.activations(T, K, 9)
+    got = ops.moe_mm_ids(tbf16(xb), torch.from_numpy(ids).cuda(), w, E).cpu().numpy()
+    y, s = reference(synth.bf16_bits_to_f32(wb), synth.bf16_bits_to_f32(xb), ids, N, False)
+    assert np.all(np.abs(got - y) <= GEMV_REL * s + 1e-30)
+
+
 @pytest.mark.parametrize("K,N", [(2048, 128), (2048, 512), (1024, 96)])
 def test_mm_ids_fused_gate_up_few_tokens_per_expert(ops, K, N):
     E, k, T = 10, 2, 70
