@@ -75,8 +75,8 @@ int bf16n_init(void);                 /* init(), launch.h:47, launch.cu:270-306:
 int bf16n_cu_count(int * out);        /* sm_count(), launch.h:48 */
 int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, int multi_col); /* mmv, launch.h:52, launch.cu:313-325 */
 /* the dense dispatch rule: BF16 token columns up to which bf16n_mmv beats dequant + GEMM for this matrix (8, the
- * reference's fixed rule, core/torch/torch_bindings.cpp:195 and ops.py:25-27, or more where the product runs on the
- * matrix cores) */
+ * reference's fixed rule, core/torch/torch_bindings.cpp:195 and ops.py:25-27; 16 for matrices of 128 Mi weights and more
+ * in wave64 units; 512 where the product runs on the matrix cores) */
 int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out);
 int bf16n_mmv_glu(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream);            /* mmv_glu merged [gate;up], launch.h:55, launch.cu:327-339 */
 int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf16n_mmv_args * a, void * stream); /* mmv_glu(gate, up), launch.h:61, launch.cu:341-365 */

@@ -227,7 +227,16 @@ int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
         ensure_init();
         check_weight(*w);
         require(out != nullptr, "null output");
-        *out = dev::is_tile_layout(*w) && dev::tile_mm_dense_pays(*w, w->rows, g_cus) ? 512 : 8;
+        if (dev::is_tile_layout(*w) && dev::tile_mm_dense_pays(*w, w->rows, g_cus)) {
+            *out = 512;
+        } else if (is_w64(*w) && !dev::is_tile_layout(*w) && dev::w64_mmv_supported(*w, true) && w->K <= 2048 &&
+                   w->rows * w->K >= ((int64_t) 1 << 27)) {
+            // a large matrix in wave64 units: two launches of eight columns per decode (2 x 302 us on 248320 x 2048)
+            // still beat writing and re-reading the whole matrix as BF16 (dequant + GEMM: 820 us)
+            *out = 16;
+        } else {
+            *out = 8;
+        }
     });
 }
 
