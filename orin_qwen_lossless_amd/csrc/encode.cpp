@@ -271,7 +271,7 @@ void write_plane(const uint16_t * w, int64_t rows, int64_t K, int R, bool cm, ui
 // per row: table entry 0 = exponent 0, then up to 15 exponents in (0, 128) by falling count, ties to the smaller
 // exponent; anything else is an escape record col | sm << 12 | exponent << 20 whose plane byte and code read as +0
 // (encode.cpp:94-180, 482-493)
-std::vector<uint8_t> encode_nibble(const uint16_t * w, int64_t rows, int64_t K, uint8_t * plane) {
+bytes encode_nibble(const uint16_t * w, int64_t rows, int64_t K, uint8_t * plane) {
     const int64_t C = K / CHUNK;
     aux_header h = {};
     h.magic = MAGIC; h.format = FMT_NIBBLE; h.K = (uint32_t) K; h.rows = (uint64_t) rows;
@@ -279,7 +279,7 @@ std::vector<uint8_t> encode_nibble(const uint16_t * w, int64_t rows, int64_t K, 
     h.off_b = h.off_a + (uint64_t) (rows * K / 2);
     h.off_c = h.off_b + (uint64_t) rows * 16;
     h.off_d = h.off_c + ((uint64_t) rows + 1) * 4;
-    std::vector<uint8_t> aux(h.off_d, 0);
+    bytes aux(h.off_d, 0);
     std::vector<uint32_t> n_esc(rows + 1, 0);
     auto row_table = [&](const uint16_t * row, uint8_t * table, int8_t * code_of) {
         int hist[256] = {0};
@@ -372,7 +372,7 @@ std::vector<uint8_t> encode_nibble(const uint16_t * w, int64_t rows, int64_t K, 
 // ---------------------------------------------------------------------------------------------- HUFFMAN (fallback)
 
 // single-exponent code, 16 symbols per (row, chunk, lane) in slot order, row-major units (encode.cpp:220-312)
-std::vector<uint8_t> encode_huffman(const uint16_t * w, int64_t rows, int64_t K, int R) {
+bytes encode_huffman(const uint16_t * w, int64_t rows, int64_t K, int R) {
     const int64_t C = K / CHUNK, units = rows / R;
     std::vector<uint64_t> freq(256, 0);
     {
@@ -421,7 +421,7 @@ std::vector<uint8_t> encode_huffman(const uint16_t * w, int64_t rows, int64_t K,
         invariant("n_words + 16 < 2^32");
     }
     h.n_a = (uint64_t) units; h.n_b = n_words;
-    std::vector<uint8_t> aux(h.off_c + (n_words + 16) * 4, 0); // 16 words of decoder lookahead
+    bytes aux(h.off_c + (n_words + 16) * 4, 0); // 16 words of decoder lookahead
     std::memcpy(aux.data(), &h, sizeof(h));
     uint32_t * lut = (uint32_t *) (aux.data() + h.off_a);
     for (int s = 0; s < 256; s++) {
@@ -456,7 +456,7 @@ std::vector<uint8_t> encode_huffman(const uint16_t * w, int64_t rows, int64_t K,
 
 // per unit and lane an MSB-first stream of pair codes, chunks in stream order, slots 0,2,..,14 (encode.cpp:321-439).
 // Empty result: too many distinct pairs.
-std::vector<uint8_t> encode_hufpair(const uint16_t * w, int64_t rows, int64_t K, int R, bool cm) {
+bytes encode_hufpair(const uint16_t * w, int64_t rows, int64_t K, int R, bool cm) {
     pair_code pc;
     if (!build_pair_code(w, rows, K, pc)) {
         return {};
@@ -506,7 +506,7 @@ std::vector<uint8_t> encode_hufpair(const uint16_t * w, int64_t rows, int64_t K,
         invariant("n_words + 32 < 2^32");
     }
     h.n_a = (uint64_t) units; h.n_b = n_words; h.flags = cm ? FLAG_CHUNK_MAJOR : 0;
-    std::vector<uint8_t> aux(h.off_d + (n_words + 32) * 4, 0); // 32 words of decoder lookahead
+    bytes aux(h.off_d + (n_words + 32) * 4, 0); // 32 words of decoder lookahead
     std::memcpy(aux.data(), &h, sizeof(h));
     std::memcpy(aux.data() + h.off_a, pc.lut.data(), 4u << HP_LP);
     uint32_t * unit_base = (uint32_t *) (aux.data() + h.off_b);
@@ -553,7 +553,7 @@ std::vector<uint8_t> encode_hufpair(const uint16_t * w, int64_t rows, int64_t K,
 // coalesced loads, and the lane of a refill word is its rank among the refilling lanes.  The table at off_a is
 // indexed by those 12 bits as they sit in the word (first code bit = index bit 0), i.e. the canonical table with
 // bit-reversed index.  unit_base has units + 1 entries (word index of each unit's first word and the end).
-std::vector<uint8_t> encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, bool cm) {
+bytes encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, bool cm) {
     pair_code pc;
     if (!build_pair_code(w, rows, K, pc)) {
         return {};
@@ -605,7 +605,11 @@ std::vector<uint8_t> encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_
     h.off_c = h.off_d;
     h.n_a = (uint64_t) units; h.n_b = n_words; h.flags = FLAG_WAVE64 | (cm ? FLAG_CHUNK_MAJOR : 0);
     // 1024 words of padding: a wave prefetches its stream in 1 KiB blocks and may run up to three blocks ahead
-    std::vector<uint8_t> aux(h.off_d + (n_words + 1024) * 4, 0);
+    // not zeroed as a whole: pass 2 writes every stream word; zero what it does not write (header padding, the gap
+    // before the stream, the padding behind it)
+    bytes aux(h.off_d + (n_words + 1024) * 4);
+    std::memset(aux.data(), 0, h.off_d);
+    std::memset(aux.data() + h.off_d + n_words * 4, 0, 1024 * 4);
     std::memcpy(aux.data(), &h, sizeof(h));
     uint32_t * lut = (uint32_t *) (aux.data() + h.off_a);
     for (uint32_t i = 0; i < (1u << HP_LP); i++) {

@@ -4,14 +4,27 @@
 #include "bf16n/format.h"
 
 #include <cstdint>
+#include <memory>
+#include <new>
+#include <utility>
 #include <vector>
 
 namespace bf16n {
 namespace impl {
 
+// std::allocator whose value-less construct leaves the bytes as they are: a vector of these can be sized without the
+// single-threaded zero fill (and page faults) of hundreds of megabytes that the encoder's threads overwrite anyway
+template <typename T>
+struct uninit_allocator : std::allocator<T> {
+    template <typename U> struct rebind { using other = uninit_allocator<U>; };
+    template <typename U> void construct(U * p) noexcept { ::new ((void *) p) U; }
+    template <typename U, typename... A> void construct(U * p, A &&... a) { ::new ((void *) p) U(std::forward<A>(a)...); }
+};
+using bytes = std::vector<uint8_t, uninit_allocator<uint8_t>>;
+
 struct encoded_buffers {
-    std::vector<uint8_t> plane; // rows * K sign|mantissa bytes
-    std::vector<uint8_t> aux;   // header + exponent data
+    bytes plane; // rows * K sign|mantissa bytes
+    bytes aux;   // header + exponent data
     int format = 0;             // format actually produced
     int R = 0;                  // rows per unit, 0 for NIBBLE
 };

@@ -169,15 +169,31 @@ def encode_bits(w_bits: np.ndarray, fmt: int, R: int, chunk_major: bool = False,
     L = _lib.lib()
     h = C.c_void_p()
     _lib.check(L.bf16n_encode(w_bits.ctypes.data, rows, K, fmt, R, flags, C.byref(h)))
-    try:
-        n = C.c_uint64()
-        p = L.bf16n_encoded_plane(h, C.byref(n))
-        plane = np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(n.value,)).copy().reshape(rows, K)
-        p = L.bf16n_encoded_aux(h, C.byref(n))
-        aux = np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(n.value,)).copy()
-        return plane, aux, L.bf16n_encoded_format(h), L.bf16n_encoded_R(h)
-    finally:
-        L.bf16n_encoded_free(h)
+    # the arrays are views of the encoder's buffers (no copy of hundreds of megabytes); the buffers are freed when the
+    # last view is gone
+    owner = _EncodedOwner(L, h)
+    n = C.c_uint64()
+    p = L.bf16n_encoded_plane(h, C.byref(n))
+    plane = _view(p, n.value, owner).reshape(rows, K)
+    p = L.bf16n_encoded_aux(h, C.byref(n))
+    aux = _view(p, n.value, owner)
+    return plane, aux, L.bf16n_encoded_format(h), L.bf16n_encoded_R(h)
+
+
+class _EncodedOwner:
+    """Keeps a bf16n_encoded handle alive for the numpy views of its buffers."""
+
+    def __init__(self, L, h):
+        self._free, self._h = L.bf16n_encoded_free, h
+
+    def __del__(self):
+        self._free(self._h)
+
+
+def _view(ptr: int, n: int, owner: _EncodedOwner) -> np.ndarray:
+    buf = (C.c_uint8 * n).from_address(ptr)
+    buf._bf16n_owner = owner  # numpy keeps `buf` as the base of the array, and `buf` keeps the handle
+    return np.frombuffer(buf, dtype=np.uint8)
 
 
 def encode(w: torch.Tensor, fmt: int, R: int, chunk_major: bool, frag_order: bool = False, wave64: bool = False
