@@ -621,23 +621,25 @@ bytes encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, boo
     }
     uint32_t * stream = (uint32_t *) (aux.data() + h.off_d);
     // pass 2: build each lane's words, then lay them out in the order the decoder takes them
+    // a lane takes at most 24 bits per pair of codes: steps * 4 * 24 bits and the two leading ones, + the zero words behind
+    const int64_t maxw = (steps * 4 * 24 + 2 + 31) / 32 + 5;
     parallel_blocks(units, 8, [&](int64_t u0, int64_t u1) {
-        std::vector<uint32_t> lane_bits[64];
+        std::vector<uint32_t> lane_words((size_t) (64 * maxw));
         std::vector<uint8_t> order; // lane of every refill, in decoder order
+        order.reserve((size_t) (steps * 4 * 64));
         for (int64_t u = u0; u < u1; u++) {
             order.clear();
             uint64_t acc[64];
-            int nb[64];
+            int nb[64], nw[64];
             uint32_t P[64];
             for (int l = 0; l < 64; l++) {
-                lane_bits[l].clear();
-                acc[l] = 0; nb[l] = 2; P[l] = 0; // two leading zero bits
+                acc[l] = 0; nb[l] = 2; nw[l] = 0; P[l] = 0; // two leading zero bits
             }
             auto put = [&](int l, uint32_t code, int len) { // first code bit lowest
                 acc[l] |= (uint64_t) bitrev(code, len) << nb[l];
                 nb[l] += len;
                 if (nb[l] >= 32) {
-                    lane_bits[l].push_back((uint32_t) acc[l]);
+                    lane_words[(size_t) (l * maxw + nw[l]++)] = (uint32_t) acc[l];
                     acc[l] >>= 32;
                     nb[l] -= 32;
                 }
@@ -660,15 +662,18 @@ bytes encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, boo
             uint32_t taken[64];
             uint32_t * out = stream + ubase[u];
             for (int l = 0; l < 64; l++) {
-                lane_bits[l].push_back((uint32_t) acc[l]); // partial last word, zero-filled
-                lane_bits[l].resize(lane_bits[l].size() + 4, 0);
-                *out++ = lane_bits[l][0];
-                *out++ = lane_bits[l][1];
-                *out++ = lane_bits[l][2];
+                uint32_t * lw = lane_words.data() + l * maxw;
+                lw[nw[l]++] = (uint32_t) acc[l]; // partial last word, zero-filled
+                for (int z = 0; z < 4; z++) {
+                    lw[nw[l]++] = 0;             // the words a lane requests past its last code
+                }
+                *out++ = lw[0];
+                *out++ = lw[1];
+                *out++ = lw[2];
                 taken[l] = 3;
             }
             for (uint8_t l : order) {
-                *out++ = lane_bits[l][taken[l]++];
+                *out++ = lane_words[(size_t) (l * maxw + taken[l]++)];
             }
             if ((uint64_t) (out - stream) != ubase[u + 1]) {
                 invariant("wave64 unit size");
