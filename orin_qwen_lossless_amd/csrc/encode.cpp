@@ -560,14 +560,23 @@ bytes encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, boo
     }
     const int64_t C = K / CHUNK, units = rows / R, steps = R * C / 2;
     auto sym_at = [&](int64_t i) { return exp_of(w[i]) | exp_of(w[i + 1]) << 8; };
-    // lens of lane l of unit u at step st, check t (pairs 2t, 2t+1)
-    auto pair_syms = [&](int64_t u, int64_t st, int l, int t, int & s0, int & s1) {
+    // first element of the chunk that half-wave `half` decodes in step st of unit u
+    auto chunk_base = [&](int64_t u, int64_t st, int half) {
         int rr; int64_t c;
-        chunk_of(2 * st + (l >> 5), R, C, cm, rr, c);
-        const int64_t base = (u * R + rr) * K + c * CHUNK;
+        chunk_of(2 * st + half, R, C, cm, rr, c);
+        return (u * R + rr) * K + c * CHUNK;
+    };
+    // the two pairs of lane l at check t (pairs 2t, 2t+1) of a chunk
+    auto pair_syms = [&](int64_t base, int l, int t, int & s0, int & s1) {
         s0 = sym_at(base + pos_of(l & 31, 4 * t));
         s1 = sym_at(base + pos_of(l & 31, 4 * t + 2));
     };
+    std::vector<uint16_t> rcode(65536, 0); // codes with their first bit lowest, as the stream holds them
+    for (int sidx = 0; sidx < 65536; sidx++) {
+        if (pc.len[sidx]) {
+            rcode[sidx] = (uint16_t) bitrev(pc.code[sidx], pc.len[sidx]);
+        }
+    }
     // pass 1: words per unit = 192 + number of refills
     std::vector<uint64_t> ubase(units + 1, 0);
     parallel_blocks(units, 8, [&](int64_t u0, int64_t u1) {
@@ -575,10 +584,11 @@ bytes encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, boo
             uint32_t P[64] = {0};
             uint64_t refills = 0;
             for (int64_t st = 0; st < steps; st++) {
+                const int64_t base[2] = {chunk_base(u, st, 0), chunk_base(u, st, 1)};
                 for (int t = 0; t < 4; t++) {
                     for (int l = 0; l < 64; l++) {
                         int s0, s1;
-                        pair_syms(u, st, l, t, s0, s1);
+                        pair_syms(base[l >> 5], l, t, s0, s1);
                         P[l] += pc.len[s0] + pc.len[s1];
                         if (P[l] >= 32) {
                             P[l] -= 32;
@@ -635,8 +645,8 @@ bytes encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, boo
             for (int l = 0; l < 64; l++) {
                 acc[l] = 0; nb[l] = 2; nw[l] = 0; P[l] = 0; // two leading zero bits
             }
-            auto put = [&](int l, uint32_t code, int len) { // first code bit lowest
-                acc[l] |= (uint64_t) bitrev(code, len) << nb[l];
+            auto put = [&](int l, uint32_t code, int len) { // code: first bit lowest
+                acc[l] |= (uint64_t) code << nb[l];
                 nb[l] += len;
                 if (nb[l] >= 32) {
                     lane_words[(size_t) (l * maxw + nw[l]++)] = (uint32_t) acc[l];
@@ -645,12 +655,13 @@ bytes encode_hufpair_w64(const uint16_t * w, int64_t rows, int64_t K, int R, boo
                 }
             };
             for (int64_t st = 0; st < steps; st++) {
+                const int64_t base[2] = {chunk_base(u, st, 0), chunk_base(u, st, 1)};
                 for (int t = 0; t < 4; t++) {
                     for (int l = 0; l < 64; l++) {
                         int s0, s1;
-                        pair_syms(u, st, l, t, s0, s1);
-                        put(l, pc.code[s0], pc.len[s0]);
-                        put(l, pc.code[s1], pc.len[s1]);
+                        pair_syms(base[l >> 5], l, t, s0, s1);
+                        put(l, rcode[s0], pc.len[s0]);
+                        put(l, rcode[s1], pc.len[s1]);
                         P[l] += pc.len[s0] + pc.len[s1];
                         if (P[l] >= 32) {
                             P[l] -= 32;
