@@ -192,7 +192,10 @@ bool build_pair_code(const uint16_t * w, int64_t rows, int64_t K, pair_code & pc
     std::vector<uint64_t> freq(65536, 0);
     {
         std::mutex mu;
-        parallel_blocks(rows, 256, [&](int64_t r0, int64_t r1) {
+        // at most 64 blocks: every block zeroes and merges a 65536-entry histogram of its own (a block holds fewer
+        // than 2^32 pairs: rows * K < 2^37 / 64)
+        const int64_t per_block = std::max<int64_t>(256, (rows + 63) / 64);
+        parallel_blocks(rows, per_block, [&](int64_t r0, int64_t r1) {
             std::vector<uint32_t> h(65536, 0);
             for (int64_t i = r0 * K; i < r1 * K; i += 2) {
                 h[exp_of(w[i]) | exp_of(w[i + 1]) << 8]++;
