@@ -164,6 +164,29 @@ def test_full_size_tiles_row_range_and_strides(ops, head_tiles):
     assert not bool(yw[:, nrows:].any())
 
 
+@pytest.mark.parametrize("K", [1024, 4096])
+def test_dense_tiles_other_row_lengths(ops, K):
+    # the smallest matrix that takes the dense matrix-core path (131072 rows), with 4 and 16 column slabs per row group
+    rows = 131072
+    g = torch.Generator(device="cuda").manual_seed(40 + K)
+    w = torch.empty((rows, K), dtype=torch.bfloat16, device="cuda")
+    for r0 in range(0, rows, 1 << 15):
+        w[r0: r0 + (1 << 15)] = (torch.randn((1 << 15, K), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    assert ops.choose(rows, K, engine="mi355x", dense_frag_order=True) == (3, 32, False, False, True)
+    plane, aux, _, _ = ops.encode_bits(w.cpu().view(torch.int16).numpy().view(np.uint16), 3, 32, False, wave64=True)
+    ta = torch.from_numpy(aux)
+    enc = ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
+    assert ops.roundtrip_equal(enc, w) and ops.gemv_max_tokens(enc) > 8
+    for T, dt in ((3, torch.bfloat16), (40, torch.bfloat16), (2, torch.float32)):
+        x = torch.randn((T, K), generator=g, device="cuda").to(dt)
+        y = ops.mmv(x, enc)
+        for r0 in range(0, rows, 1 << 15):
+            wd = w[r0: r0 + (1 << 15)].double()
+            ref, bound = x.double() @ wd.t(), x.double().abs() @ wd.abs().t()
+            assert bool(((y[:, r0: r0 + (1 << 15)].double() - ref).abs() <= 1e-5 * bound).all()), (K, T, dt, r0)
+        assert torch.equal(ops.mmv(x[T - 1:], enc)[0], y[T - 1])
+
+
 # ---- one MoE layer of the 35B-A3B shape at its real size: 256 experts x (gate, up 512 x 2048; down 2048 x 512) -----------
 
 E, TOPK, N = 256, 8, 512
