@@ -34,14 +34,16 @@ __device__ __forceinline__ int tile_col(int s, int j, int half) { return 32 * s 
 
 // One decode chain: the tiles [first unit, first unit + n) of one matrix, with the plane bytes of the next D steps
 // in registers (reloaded as soon as a step is consumed).
-template <int D> struct tchain_t {
+// ONCE: plane and stream are read by this launch only and are loaded with the non-temporal hint
+template <int D, bool ONCE = false> struct tchain_t {
     w64_dec dec;
     const uint8_t * plane;
     uint32_t off, last;
     uint4 sm[D];
     __device__ __forceinline__ uint4 load_step(int lane) const {
         const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
-        return *((const uint4 *) (plane + o) + lane);
+        const uint4 * src = (const uint4 *) (plane + o) + lane;
+        return ONCE ? load_once(src) : *src;
     }
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane) {
         start(ring, q, unit0, n_units, lane, q.ubase[unit0], q.ubase[unit0 + n_units]);
@@ -57,7 +59,7 @@ template <int D> struct tchain_t {
             sm[s] = load_step(lane);
             off += STEP_BYTES;
         }
-        dec.start(ring, q.stream, uniform(first), uniform(end), lane);
+        dec.start(ring, q.stream, uniform(first), uniform(end), lane, ONCE);
     }
     // s: the step just consumed (a compile-time value at every call)
     __device__ __forceinline__ void reload(int s, int lane) {
@@ -73,8 +75,8 @@ template <int D> struct tchain_t {
 typedef tchain_t<4> tchain;
 
 // one step of N chains, instruction streams interleaved; lut of chain k at lut + k * lut_stride
-template <int N, int D>
-__device__ __forceinline__ void tile_step(tchain_t<D> * ch, const uint32_t * lut, int lut_stride, int s, uint32_t (&wp)[N][8]) {
+template <int N, int D, bool ONCE = false>
+__device__ __forceinline__ void tile_step(tchain_t<D, ONCE> * ch, const uint32_t * lut, int lut_stride, int s, uint32_t (&wp)[N][8]) {
     uint32_t smw[N][4];
 #pragma unroll
     for (int k = 0; k < N; k++) {
@@ -252,7 +254,9 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
             if (stager) {
                 MT_STAGE_LOAD(VLD, f0, f1, f2, f3, (const uint4 *) xsrc);
             }
-            tchain_t<S::DEPTH> ch[2];
+            // 32-token shape: (nearly) every tile of a launch is decoded once, so its loads are read-once; the 128-token
+            // shape serves long token lists, whose passes share tiles
+            tchain_t<S::DEPTH, NT == 1> ch[2];
             if (live) {
                 uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
                 ch[0].start(ring, q0, ((int64_t) e * groups + g0) * slabs, slabs, lane);
@@ -297,7 +301,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
 #pragma unroll
                     for (int s = 0; s < 4; s++) {
                         uint32_t wp[2][8];
-                        tile_step<2, S::DEPTH>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
+                        tile_step<2, S::DEPTH, NT == 1>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
                         ch[0].reload(s, lane);
                         ch[1].reload(s, lane);
                         const uint16_t * bp = bcur + l32 * MT_BSTRIDE + 32 * s + 8 * half;
@@ -442,7 +446,7 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
             if (tp < n) {
                 // this lane's token (past the item's last: that one again, dropped at the store), its K part and half
                 const char * xr = (const char *) (a.x + (int64_t) a.ids_src1[j0 + (tk < n ? tk : n - 1)] * a.x_row + kw * spw * TILE_K) + 16 * half;
-                tchain_t<2> ch[2];
+                tchain_t<2, true> ch[2];
                 ch[0].start(ring, q0, ((int64_t) e * groups + g0) * (WPI * spw) + kw * spw, spw, lane);
                 ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * (WPI * spw) + kw * spw, spw, lane);
                 // B operands of a step: columns 32 s + 8 half + [0, 8) and 16 further on
@@ -459,7 +463,7 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
                     nb0 = *(const bf16x8_t *) xn;
                     nb1 = *(const bf16x8_t *) (xn + 32);
                     uint32_t wp[2][8];
-                    tile_step<2, 2>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
+                    tile_step<2, 2, true>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
                     ch[0].reload(s, lane);
                     ch[1].reload(s, lane);
                     bf16x8_t av[2][2]; // [chain][16-column block]
@@ -578,7 +582,7 @@ constexpr int tv_max_waves() { return GLU && sizeof(TX) == 2 ? TV_WAVES : TV_WAV
 // wavefront, many wavefronts) — and the partial sums (one per lane and row) of a group's `wpg` wavefronts per matrix
 // are added in tile order.  GLU: the group has wpg wavefronts on the gate matrix and wpg on the up matrix, and the
 // block writes silu(gate x) * (up x).
-template <typename TX, bool GLU>
+template <typename TX, bool GLU, bool ONCE>
 __global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw) {
     constexpr int NM = GLU ? 2 : 1;
     __shared__ __align__(16) uint32_t lut[NM * LUT_WORDS];
@@ -598,7 +602,7 @@ __global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(con
     if (GLU) {
         stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
     }
-    tchain ch[1];
+    tchain_t<4, ONCE> ch[1];
     if (live) {
         ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end);
     }
@@ -621,7 +625,7 @@ __global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(con
                         xb.load(cv.x, kk + 16);
                     }
                     uint32_t wp[1][8];
-                    tile_step<1, 4>(ch, my_lut, 0, s, wp);
+                    tile_step<1, 4, ONCE>(ch, my_lut, 0, s, wp);
                     ch[0].reload(s, lane);
                     if (sizeof(TX) != 2) {
                         xa.load(cv.x, kk);
@@ -878,17 +882,28 @@ void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols
     const int64_t groups = p.nrows / TILE_R;
     const dim3 grid((unsigned) ((groups + gpb - 1) / gpb), ncols);
     const size_t shm = (size_t) waves * WAVE_LDS_WORDS * 4;
+    // one token, or few routed pairs over many experts: (nearly) every tile is read once, by this launch only
+    const int64_t n_experts = p.rows_per_matrix > 0 ? w.rows / p.rows_per_matrix : 1;
+    const bool once = p.ids ? ncols <= p.n_used || (int64_t) ncols * 4 <= n_experts : ncols == 1;
+    const dim3 nt(waves * 64);
+#define TILE_MMV(TX, GLU, UP)                                                                                   \
+    if (once) {                                                                                                 \
+        hipLaunchKernelGGL((k_tile_mmv<TX, GLU, true>), grid, nt, shm, stream, w, UP, p, wpg, upw);             \
+    } else {                                                                                                    \
+        hipLaunchKernelGGL((k_tile_mmv<TX, GLU, false>), grid, nt, shm, stream, w, UP, p, wpg, upw);            \
+    }
     if (up) {
         if (x_bf16) {
-            hipLaunchKernelGGL((k_tile_mmv<bf16_t, true>), grid, dim3(waves * 64), shm, stream, w, *up, p, wpg, upw);
+            TILE_MMV(bf16_t, true, *up)
         } else {
-            hipLaunchKernelGGL((k_tile_mmv<float, true>), grid, dim3(waves * 64), shm, stream, w, *up, p, wpg, upw);
+            TILE_MMV(float, true, *up)
         }
     } else if (x_bf16) {
-        hipLaunchKernelGGL((k_tile_mmv<bf16_t, false>), grid, dim3(waves * 64), shm, stream, w, w, p, wpg, upw);
+        TILE_MMV(bf16_t, false, w)
     } else {
-        hipLaunchKernelGGL((k_tile_mmv<float, false>), grid, dim3(waves * 64), shm, stream, w, w, p, wpg, upw);
+        TILE_MMV(float, false, w)
     }
+#undef TILE_MMV
 }
 
 void launch_tile_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, hipStream_t stream) {
