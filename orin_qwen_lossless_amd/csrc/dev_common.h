@@ -23,7 +23,8 @@ struct cols {
     int n_used, x_per_slot;
     int64_t rows_per_matrix, row0, nrows;
     bool y_bf16;
-    bool stream_once; // the compressed stream is read by one launch only: load it with the non-temporal hint
+    bool stream_once; // stream blocks with the same hint (small matrices only)
+    bool plane_once; // the launch reads every plane byte once: load them with the non-temporal hint
 };
 
 struct col_view { const char * x; char * y; int64_t rbase; };

@@ -14,9 +14,12 @@ constexpr int AHEAD = 256;    // words kept ahead of the consumer: a unit start 
 constexpr int LUT_WORDS = 1 << HP_LP;
 constexpr int WAVE_LDS_WORDS = RING + RING_PAD;
 
-// 16 bytes of data that a launch reads once (plane bytes, stream blocks of a matrix that streams through): loaded with the
-// non-temporal hint, which measured 8 % faster on the 248320 x 2048 GEMV (124 against 135 us); data that other columns
-// or passes of the launch read again (routed experts, small matrices) keeps the default policy, which is faster there
+// 16 bytes that a launch reads once, loaded with the non-temporal hint: 8 % faster on the 248320 x 2048 GEMV (126
+// against 136 us). Planes that other columns or passes of the launch read again (routed experts with many tokens, small
+// matrices in a column loop) keep the default policy, which is faster there. Stream blocks start at any 16-byte
+// boundary, so consecutive blocks share a cache line, and with the hint that line is fetched twice (3 % more memory
+// traffic): the GEMVs and the routed batched kernels are still faster with it inside a decode step, a large dense matrix
+// in the batched tile kernel is 5 % slower, so the stream hint is a flag of its own (w64_dec::once)
 typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 load_once(const uint4 * p) {
     const u32x4_nt v = __builtin_nontemporal_load((const u32x4_nt *) p);
@@ -61,7 +64,7 @@ struct w64_dec {
     const uint32_t * src;   // 16-byte aligned
     uint4 pend;             // the block that starts at `filled`, in flight
     int lane;
-    bool once;              // the stream is read once by the whole launch: non-temporal loads (same in every lane)
+    bool once;              // stream blocks with the non-temporal hint (same in every lane)
 
     // Every load is unconditional (a block or step past the end re-reads the last one) so that the number of loads in
     // flight at any point of the loop is fixed and the waits for prefetched data never drain newer loads.

@@ -34,7 +34,8 @@ __device__ __forceinline__ int tile_col(int s, int j, int half) { return 32 * s 
 
 // One decode chain: the tiles [first unit, first unit + n) of one matrix, with the plane bytes of the next D steps
 // in registers (reloaded as soon as a step is consumed).
-// ONCE: plane and stream are read by this launch only and are loaded with the non-temporal hint
+// ONCE: the plane bytes are read by this launch only and are loaded with the non-temporal hint; stream_once (start)
+// asks the same for the stream blocks, which pays for routed experts and not for a large dense matrix
 template <int D, bool ONCE = false> struct tchain_t {
     w64_dec dec;
     const uint8_t * plane;
@@ -45,12 +46,12 @@ template <int D, bool ONCE = false> struct tchain_t {
         const uint4 * src = (const uint4 *) (plane + o) + lane;
         return ONCE ? load_once(src) : *src;
     }
-    __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane) {
-        start(ring, q, unit0, n_units, lane, q.ubase[unit0], q.ubase[unit0 + n_units]);
+    __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane, bool stream_once = false) {
+        start(ring, q, unit0, n_units, lane, q.ubase[unit0], q.ubase[unit0 + n_units], stream_once);
     }
     // first / end: the stream words of the units (their unit bases, read by the caller ahead of time)
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane, uint32_t first,
-                                          uint32_t end) {
+                                          uint32_t end, bool stream_once = false) {
         plane = q.plane + uniform64(unit0 * T_BYTES);
         off = 0;
         last = (uint32_t) (n_units * T_BYTES - STEP_BYTES);
@@ -59,7 +60,7 @@ template <int D, bool ONCE = false> struct tchain_t {
             sm[s] = load_step(lane);
             off += STEP_BYTES;
         }
-        dec.start(ring, q.stream, uniform(first), uniform(end), lane, ONCE);
+        dec.start(ring, q.stream, uniform(first), uniform(end), lane, stream_once);
     }
     // s: the step just consumed (a compile-time value at every call)
     __device__ __forceinline__ void reload(int s, int lane) {
@@ -259,8 +260,8 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
             tchain_t<S::DEPTH, NT == 1> ch[2];
             if (live) {
                 uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * slabs, slabs, lane);
-                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * slabs, slabs, lane);
+                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * slabs, slabs, lane, NT == 1 && a.bounds != nullptr);
+                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * slabs, slabs, lane, NT == 1 && a.bounds != nullptr);
             }
             f32x16_t acc[2][NT];
 #pragma unroll
@@ -447,8 +448,8 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
                 // this lane's token (past the item's last: that one again, dropped at the store), its K part and half
                 const char * xr = (const char *) (a.x + (int64_t) a.ids_src1[j0 + (tk < n ? tk : n - 1)] * a.x_row + kw * spw * TILE_K) + 16 * half;
                 tchain_t<2, true> ch[2];
-                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * (WPI * spw) + kw * spw, spw, lane);
-                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * (WPI * spw) + kw * spw, spw, lane);
+                ch[0].start(ring, q0, ((int64_t) e * groups + g0) * (WPI * spw) + kw * spw, spw, lane, true);
+                ch[1].start(ring + WAVE_LDS_WORDS, q1, ((int64_t) e * groups + g1) * (WPI * spw) + kw * spw, spw, lane, true);
                 // B operands of a step: columns 32 s + 8 half + [0, 8) and 16 further on
                 bf16x8_t nb0 = *(const bf16x8_t *) xr, nb1 = *(const bf16x8_t *) (xr + 32);
 #pragma unroll 1
@@ -604,7 +605,7 @@ __global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(con
     }
     tchain_t<4, ONCE> ch[1];
     if (live) {
-        ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end);
+        ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end, ONCE);
     }
     __syncthreads();
     if (live) {

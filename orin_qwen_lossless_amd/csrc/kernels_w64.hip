@@ -83,14 +83,14 @@ struct chain {
     uint32_t last;         // byte offset of the chain's last step
     uint4 sm[NB];          // plane bytes of the body's steps
     int64_t row;           // output row of the next body, relative to the product
-    bool once;             // plane and stream are read once by the launch (see load_once)
+    bool once;             // the launch reads the plane bytes once (see load_once)
     __device__ __forceinline__ uint4 load_step(int lane) const {
         const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
         return once ? load_once((const uint4 *) (plane + o) + lane) : *((const uint4 *) (plane + o) + lane);
     }
     // first / end: the stream words of units [gu0, gu0 + n_units) (unit bases, read by the caller ahead of time)
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t gu0, int64_t n_units, int64_t row0, int R, int K,
-                                          int lane, uint32_t first, uint32_t end, bool once_ = false) {
+                                          int lane, uint32_t first, uint32_t end, bool once_ = false, bool stream_once = false) {
         once = once_;
         plane = q.plane + uniform64(gu0 * R * K);
         off = 0;
@@ -101,7 +101,7 @@ struct chain {
             sm[s] = load_step(lane);
             off += 1024;
         }
-        dec.start(ring, q.stream, uniform(first), uniform(end), lane, once);
+        dec.start(ring, q.stream, uniform(first), uniform(end), lane, stream_once);
     }
     // plane bytes of step s of the next body, once step s of this body is consumed
     __device__ __forceinline__ void reload(int s, int lane) {
@@ -260,9 +260,9 @@ __global__ void __launch_bounds__(wide_regs(x_regs<TX, C, NC>(), sizeof(TX) == 2
     }
     chain<G::NB> ch[2];
     uint32_t * ring = rings + wave * (NCH * WAVE_LDS_WORDS);
-    ch[0].start(ring, q, gu0, nA, u_begin * R, R, K, lane, b0, b1, p.stream_once);
+    ch[0].start(ring, q, gu0, nA, u_begin * R, R, K, lane, b0, b1, p.plane_once, p.stream_once);
     if (NCH == 2 && nB > 0) {
-        ch[1].start(ring + WAVE_LDS_WORDS, q, gu0 + nA, nB, (u_begin + nA) * R, R, K, lane, b1, b2, p.stream_once);
+        ch[1].start(ring + WAVE_LDS_WORDS, q, gu0 + nA, nB, (u_begin + nA) * R, R, K, lane, b1, b2, p.plane_once, p.stream_once);
     }
     for (int64_t i = 0; i < nA; i++) {
         if (NCH == 2 && i < nB) {
@@ -306,8 +306,8 @@ __global__ void __launch_bounds__(1024) k_w64_glu(const bf16n_weight wg, const b
     }
     chain<G::NB> ch[2];
     uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-    ch[0].start(ring, qg, gu0, n, u_begin * R, R, K, lane, g0, g1, p.stream_once);
-    ch[1].start(ring + WAVE_LDS_WORDS, qu, gu0, n, u_begin * R, R, K, lane, u0, u1, p.stream_once);
+    ch[0].start(ring, qg, gu0, n, u_begin * R, R, K, lane, g0, g1, p.plane_once, p.stream_once);
+    ch[1].start(ring + WAVE_LDS_WORDS, qu, gu0, n, u_begin * R, R, K, lane, u0, u1, p.plane_once, p.stream_once);
     for (int64_t i = 0; i < n; i++) {
         unit_pass<TX, C, 1, 2, true>(ch, lut, xr, p, cv, R, lane);
     }
@@ -529,12 +529,13 @@ void launch_w64_mmv(const bf16n_weight & w, const cols & p, int ncols, bool x_bf
         const int nc = group_max == 1 ? 1 : (ncols - c0 < group_max ? ncols - c0 : group_max);
         const int ny = group_max == 1 ? ncols : 1;
         cols q = p;
-        // a dense product whose columns all fit one launch reads each stream word once, and a matrix of 2^27 weights
-        // or more outlasts the caches between two launches: keep such streams out of the way of the activations.
+        // a dense product whose columns all fit one launch reads each plane byte once, and a matrix of 2^27 weights
+        // or more outlasts the caches between two launches: keep such planes out of the way of the activations.
         // One routed token names each of its experts once. Routed batches and column loops over smaller matrices read
         // words again and keep the default policy.
-        q.stream_once = p.ids ? ncols <= p.n_used
+        q.plane_once = p.ids ? ncols <= p.n_used
                               : (group_max == 1 ? ncols == 1 : ncols <= group_max) || p.nrows * w.K >= ((int64_t) 1 << 27);
+        q.stream_once = q.plane_once;
         if (group_max > 1) {
             q.x += c0 * p.x_tok;
             q.y += c0 * p.y_tok;
@@ -575,7 +576,8 @@ void launch_w64_glu(const bf16n_weight & gate, const bf16n_weight & up, const co
     const int wpb = (int) (waves < 4 ? waves : 4);
     const dim3 grid((unsigned) ((waves + wpb - 1) / wpb), ncols);
     cols q = p;
-    q.stream_once = p.ids ? ncols <= p.n_used : ncols == 1; // one token: every stream word is read once
+    q.plane_once = p.ids ? ncols <= p.n_used : ncols == 1; // one token: every plane byte is read once
+    q.stream_once = q.plane_once;
     if (x_bf16) {
         glu_c<bf16_t>(C, grid, wpb * 64, wpb, stream, gate, up, q, (int) upw);
     } else {
