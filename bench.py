@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0
 SETTLE_MS = 40.0  # untimed load before the timed region of the headline kernel (see time_kernel)
 # HBM bytes per GEMV launch from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, each factor calibrated
 # on a copy of known size in the same profiler run), for the workloads that were profiled; not measurable in-process.
-MEASURED_TRAFFIC = {(248320, 2048): 729_300_000}
+MEASURED_TRAFFIC = {(248320, 2048): 711_400_000}
 
 
 def gen_weights(rows: int, K: int, seed: int):

@@ -84,10 +84,14 @@ struct w64_dec {
         ring = ring_;
         lane = lane_;
         once = once_;
-        const uint32_t a = first & ~3u;
-        src = stream + uniform(a); // kernel-argument pointer + scalar offset: stays a global, scalar address
-        cons = first - a;
-        last_block = (end - a - 1) / BLK * BLK; // the stream is padded: a block may run past `end`
+        // blocks start on 128-byte lines (a block is then eight whole cache lines, and no line belongs to two blocks):
+        // up to 31 words before `first`, which are skipped; before the first unit of a matrix these are the last words
+        // of the section that precedes the stream in the same buffer (the header and the table come first)
+        const uint32_t a4 = first & ~3u;
+        const int32_t a = (int32_t) a4 - (int32_t) (((uintptr_t) (stream + a4) & 127u) >> 2);
+        src = stream + (int32_t) uniform((uint32_t) a); // kernel-argument pointer + scalar offset: stays a global, scalar address
+        cons = (uint32_t) ((int32_t) first - a);
+        last_block = (uint32_t) ((int32_t) end - a - 1) / BLK * BLK; // the stream is padded: a block may run past `end`
         const uint4 b0 = load_block(0);
         pend = load_block(BLK);
         store_block(0, b0);
