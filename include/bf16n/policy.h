@@ -18,7 +18,8 @@ struct policy_options {
     policy_engine engine = policy_engine::vllm;
     policy_mode mode = policy_mode::hybrid;
     int64_t dense_min = 8ll << 20;  // dense tensors below this many weights take NIBBLE in hybrid mode
-    bool expert = false;            // llama: the loader's "_exps" classification; vllm and mi355x use n_matrices > 1
+    bool expert = false;            // llama: the loader's "_exps" classification; vllm uses n_matrices > 1 instead;
+                                    // mi355x: experts are n_matrices > 1 or this flag
     bool dense_frag_order = false;  // vllm: fragment order for dense tensors; mi355x: matrix-core tiles (R = 32) for
                                     // dense matrices of at least 131072 rows (BF16-activation callers)
 };

@@ -25,6 +25,7 @@ using namespace bf16n;
 namespace bf16n {
 namespace impl {
 int report(const std::function<void()> & f); // capi.cpp: runs f, maps exceptions to a status and the thread's message
+void check_weight(const bf16n_weight & w);   // capi.cpp: the launchers' contract on a weight (throws std::invalid_argument)
 }
 } // namespace bf16n
 
@@ -52,19 +53,25 @@ void hip_check(hipError_t e, const char * what) {
     }
 }
 
-void insert(const entry & e) {
-    std::lock_guard<std::mutex> lock(g_mutex);
+// where [plane, plane + nbytes) goes in the sorted registry; throws when the range overlaps a registered tensor.
+// The caller holds g_mutex.
+std::vector<entry>::iterator free_slot(const uint8_t * plane, size_t nbytes) {
     const auto less = std::less<const uint8_t *>{};
-    auto it = std::upper_bound(g_entries.begin(), g_entries.end(), e.w.plane,
+    auto it = std::upper_bound(g_entries.begin(), g_entries.end(), plane,
                                [&](const uint8_t * p, const entry & v) { return less(p, v.w.plane); });
     if (it != g_entries.begin()) {
         const entry & prev = *(it - 1);
-        require(!less(e.w.plane, prev.w.plane + prev.nbytes), "adapter: the tensor overlaps a registered one");
+        require(!less(plane, prev.w.plane + prev.nbytes), "adapter: the tensor overlaps a registered one");
     }
     if (it != g_entries.end()) {
-        require(!less(it->w.plane, e.w.plane + e.nbytes), "adapter: the tensor overlaps a registered one");
+        require(!less(it->w.plane, plane + nbytes), "adapter: the tensor overlaps a registered one");
     }
-    g_entries.insert(it, e);
+    return it;
+}
+
+void insert(const entry & e) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_entries.insert(free_slot(e.w.plane, e.nbytes), e);
 }
 
 // one flag for the whole comparison: any differing 16-byte piece sets it (plain stores of the same value)
@@ -89,6 +96,8 @@ struct device_buffer {
 // decode(encoded) == source for every weight: the tensor is decoded on the device in pieces of at most 64 MiB of BF16
 // (whole units), each piece compared there with the same rows of the source
 bool verify_on_device(const bf16n_weight & w, const uint16_t * host) {
+    impl::check_weight(w); // K, format and R are divisors below
+    require(w.rows > 0, "verify: empty tensor");
     const int64_t unit = w.format == FMT_NIBBLE ? 1 : w.R;
     int64_t chunk_rows = std::max<int64_t>((64ll << 20) / (w.K * 2) / unit * unit, unit);
     chunk_rows = std::min<int64_t>(chunk_rows, w.rows);
@@ -159,6 +168,11 @@ int bf16n_adapter_convert(void * tensor_data, const void * bf16_host, int64_t ro
                              n_matrices > 1, matrix_core_order, c) != 0,
                 "adapter: K must be a multiple of 512 in [512, 4096]");
         const int64_t rows = rows_per_matrix * n_matrices;
+        {
+            // a tensor that overlaps a registered one is refused before anything is written into it
+            std::lock_guard<std::mutex> lock(g_mutex);
+            (void) free_slot((const uint8_t *) tensor_data, (size_t) (rows * K));
+        }
         const uint32_t flags = (c[2] ? FLAG_CHUNK_MAJOR : 0) | (c[3] ? FLAG_FRAG_ORDER : 0) | (c[4] ? FLAG_WAVE64 : 0);
         bf16n_encoded * enc = nullptr;
         if (bf16n_encode((const uint16_t *) bf16_host, rows, K, c[0], c[1], flags, &enc) != BF16N_OK) {

@@ -78,10 +78,23 @@ int report(const std::function<void()> & f) { return guarded(f); }
 
 namespace {
 
+void check_weight(const bf16n_weight & w);
+
+} // namespace
+
+namespace bf16n {
+namespace impl {
+void check_weight(const bf16n_weight & w) { ::check_weight(w); }
+} // namespace impl
+} // namespace bf16n
+
+namespace {
+
 // launch.cu:261-268
 void check_weight(const bf16n_weight & w) {
     require(w.K % 512 == 0 && w.K >= 512 && w.K <= K_MAX, "K must be a multiple of 512 in [512, 4096]");
     require(w.format == FMT_NIBBLE || w.format == FMT_HUFFMAN || w.format == FMT_HUFPAIR, "unknown format");
+    require(w.rows >= 0, "rows must be nonnegative");
     require(w.format == FMT_NIBBLE || (w.R > 0 && w.rows % w.R == 0), "rows must be a multiple of R");
     require(!(w.flags & FLAG_CHUNK_MAJOR) || w.format == FMT_HUFPAIR, "chunk-major units exist only for HUFPAIR");
     require(!(w.flags & FLAG_FRAG_ORDER), "fragment-order weights are not supported by the MI355X build");

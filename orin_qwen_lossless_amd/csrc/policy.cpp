@@ -79,7 +79,9 @@ bool choose(int64_t rows, int64_t K, int64_t n, int engine, int mode, int64_t de
         return false;
     }
     const bool vllm = engine == 1, mi355x = engine == 2;
-    const bool expert = vllm ? n > 1 : expert_flag; // llama (and mi355x) classify by the caller's flag (policy.cpp:49)
+    // llama classifies by the caller's flag, vllm by the stack size (policy.cpp:49); mi355x takes either: a stack of
+    // several matrices is an expert stack whatever the caller says, as in every later decision of its branch
+    const bool expert = vllm ? n > 1 : mi355x ? (expert_flag || n > 1) : expert_flag;
     if (mode == 2 || (mode == 0 && !expert && !reaches(rows, K, n, dense_min))) {
         out = {FMT_NIBBLE, 0, false, false, false};
         return true;

@@ -33,9 +33,16 @@ ENGINES = {"llama": 0, "vllm": 1, "mi355x": 2}
 MODES = {"hybrid": 0, "huffman": 1, "nibble": 2}
 
 
+_HEADER_FIELDS = ("magic", "format", "K", "R", "rows", "off_a", "off_b", "off_c", "off_d", "n_a", "n_b", "flags", "reserved")
+_KNOWN_FLAGS = FLAG_CHUNK_MAJOR | FLAG_FRAG_ORDER | FLAG_WAVE64
+
+
 @dataclass(frozen=True)
 class Meta:
-    """Host-side metadata of one encoded matrix, parsed once from its aux header."""
+    """What the launchers need to know about one encoded matrix (the fields of bf16n_weight that are not pointers).
+
+    Field names and order are those of the reference's Meta (engines/vllm/vllm_bf16n/ops.py:33-50) so that code
+    written against it keeps working; wave64 is this build's layout bit and comes last."""
 
     format: int
     K: int
@@ -51,29 +58,40 @@ class Meta:
 
     @property
     def flags(self) -> int:
-        return ((FLAG_CHUNK_MAJOR if self.chunk_major else 0) | (FLAG_FRAG_ORDER if self.frag_order else 0)
-                | (FLAG_WAVE64 if self.wave64 else 0))
+        bits = 0
+        for on, bit in ((self.chunk_major, FLAG_CHUNK_MAJOR), (self.frag_order, FLAG_FRAG_ORDER), (self.wave64, FLAG_WAVE64)):
+            bits |= bit if on else 0
+        return bits
 
     def as_list(self) -> list[int]:
+        """The nine integers of the torch.ops.bf16n `meta` argument: format, K, rows, R, flags, off_a .. off_d."""
         return [self.format, self.K, self.rows, self.R, self.flags, self.off_a, self.off_b, self.off_c, self.off_d]
 
 
 def parse_header(aux: torch.Tensor) -> Meta:
-    """Metadata from the first 256 bytes of a CPU aux tensor; raises on a malformed header."""
-    if aux.device.type != "cpu" or aux.dtype != torch.uint8 or aux.numel() < 256:
+    """Meta of an encoded matrix from the aux_header at the start of its host aux buffer (include/bf16n/format.h).
+
+    ValueError when the buffer is not host uint8 memory holding a whole 256-byte header block, when the magic or the
+    format number is wrong, or when a layout flag is set that this build does not know."""
+    on_host = aux.device.type == "cpu"
+    if not on_host or aux.dtype != torch.uint8 or aux.numel() < 256:
         raise ValueError("bf16n: aux must be a CPU uint8 tensor of at least 256 bytes")
-    (magic, fmt, K, R, rows, a, b, c, d, _na, _nb, flags, _pad) = HEADER.unpack(bytes(aux[: HEADER.size].tolist()))
-    if magic != MAGIC or fmt not in FORMAT_NAMES:
-        raise ValueError(f"bf16n: bad aux header (magic {magic:#x}, format {fmt})")
-    if flags & ~(FLAG_CHUNK_MAJOR | FLAG_FRAG_ORDER | FLAG_WAVE64):
+    raw = aux.reshape(-1)[: HEADER.size].contiguous().numpy().tobytes()
+    h = dict(zip(_HEADER_FIELDS, HEADER.unpack(raw)))
+    if h["magic"] != MAGIC or h["format"] not in FORMAT_NAMES:
+        raise ValueError(f"bf16n: bad aux header (magic {h['magic']:#x}, format {h['format']})")
+    flags = h["flags"]
+    if flags & ~_KNOWN_FLAGS:
         raise ValueError(f"bf16n: unknown layout flags {flags:#x}")
-    return Meta(fmt, K, rows, R, bool(flags & FLAG_CHUNK_MAJOR), bool(flags & FLAG_FRAG_ORDER), a, b, c, d,
-                bool(flags & FLAG_WAVE64))
+    return Meta(format=h["format"], K=h["K"], rows=h["rows"], R=h["R"], chunk_major=bool(flags & FLAG_CHUNK_MAJOR),
+                frag_order=bool(flags & FLAG_FRAG_ORDER), off_a=h["off_a"], off_b=h["off_b"], off_c=h["off_c"],
+                off_d=h["off_d"], wave64=bool(flags & FLAG_WAVE64))
 
 
 @dataclass
 class Weight:
-    """One encoded matrix on the device: plane (rows x K sign|mantissa bytes) + aux, and its metadata."""
+    """An encoded matrix resident on a device: the two uint8 buffers the encoder produced (plane: one sign|mantissa byte
+    per weight; aux: header, tables and exponent streams) and the Meta parsed from the aux header on the host."""
 
     plane: torch.Tensor
     aux: torch.Tensor
@@ -85,7 +103,8 @@ class Weight:
 
     @property
     def nbytes(self) -> int:
-        return self.plane.numel() + self.aux.numel()
+        """Bytes the matrix occupies in device memory."""
+        return int(self.plane.numel()) + int(self.aux.numel())
 
 
 def _stream() -> C.c_void_p:
@@ -228,17 +247,26 @@ def dequant(w: Weight, row0: int = 0, nrows: int | None = None) -> torch.Tensor:
 
 
 def roundtrip_equal(w: Weight, src: torch.Tensor, chunk_bytes: int = 64 << 20) -> bool:
-    """Bitwise check of the GPU decode against the BF16 source (any device), in row chunks of whole units."""
-    K, rows = w.meta.K, w.meta.rows
-    unit = max(w.meta.R, 1)
-    src2 = src.reshape(rows, K)
-    step = max(chunk_bytes // (2 * K) // unit * unit, unit)
-    for r0 in range(0, rows, step):
-        nr = min(step, rows - r0)
-        got = dequant(w, r0, nr).view(torch.int16)
-        ref = src2[r0: r0 + nr].to(got.device).view(torch.int16)
-        if not torch.equal(got, ref):
+    """True when the device decode of w reproduces every BF16 bit pattern of src (rows x K values on any device).
+
+    The matrix is decoded in pieces of at most chunk_bytes of BF16 output, each a whole number of units, and each piece
+    is compared on the device; the first differing piece ends the check (engines/vllm/vllm_bf16n/ops.py:104-116)."""
+    meta = w.meta
+    want = src.reshape(meta.rows, meta.K)
+    if want.element_size() != 2:
+        raise ValueError("bf16n.roundtrip_equal: the source must hold 16-bit values (bfloat16)")
+    rows_per_unit = meta.R if meta.R > 0 else 1
+    piece = chunk_bytes // (2 * meta.K) // rows_per_unit * rows_per_unit
+    piece = piece if piece >= rows_per_unit else rows_per_unit
+    first = 0
+    while first < meta.rows:
+        n = piece if first + piece <= meta.rows else meta.rows - first
+        decoded = dequant(w, first, n)
+        expect = want.narrow(0, first, n).to(decoded.device, non_blocking=False)
+        # compare bit patterns, not values: NaN payloads and signed zeros count
+        if not bool((decoded.view(torch.int16) == expect.view(torch.int16)).all()):
             return False
+        first += n
     return True
 
 
@@ -364,16 +392,21 @@ def linear(x: torch.Tensor, w: Weight, bias: torch.Tensor | None = None) -> torc
         else:
             y = _mmv_common(xc, w, None, 0, True, False)
     else:
-        y = torch.empty((T, rows), dtype=x.dtype, device=x.device)
         unit = 1 if w.meta.format == FMT_NIBBLE else w.meta.R
         chunk = min(max(DEQUANT_CHUNK_BYTES // (K * 2) // unit * unit, unit), rows)
-        for r0 in range(0, rows, chunk):
-            nr = min(chunk, rows - r0)
-            wc = dequant(w, r0, nr)
-            ys = y.narrow(1, r0, nr)
-            torch.mm(x2, wc.t(), out=ys) if nr != rows else ys.copy_(torch.mm(x2, wc.t()))
-            if bias is not None:
-                ys.add_(bias.narrow(0, r0, nr))
+        if chunk == rows:
+            # one piece: the stock linear adds the bias before its single rounding to BF16, as the reference's does
+            y = torch.nn.functional.linear(x2, dequant(w, 0, rows), bias)
+        else:
+            y = torch.empty((T, rows), dtype=x.dtype, device=x.device)
+            for r0 in range(0, rows, chunk):
+                nr = min(chunk, rows - r0)
+                wc = dequant(w, r0, nr)
+                ys = y.narrow(1, r0, nr)
+                if bias is None:
+                    torch.mm(x2, wc.t(), out=ys)
+                else:
+                    torch.addmm(bias.narrow(0, r0, nr), x2, wc.t(), out=ys)
     return y.view(oshape)
 
 
@@ -499,51 +532,41 @@ def glu2_supported(gate: Weight, up: Weight) -> bool:
             and (not g.wave64 or g.K in (512, 1024, 2048, 4096)))
 
 
+def _experts_batched(x, gate, up, down, topk_ids, n_experts):
+    """Per-pair FP32 outputs of the routed experts through the batched kernels: one routing pass serves both products
+    (with one activation row per (token, slot), as down takes them, the source row of a pair is its destination row)."""
+    src1, dst, bounds = mm_ids_route(topk_ids, n_experts, False)
+    hidden = moe_mm_ids(x, topk_ids, gate, n_experts, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
+    return moe_mm_ids(hidden, topk_ids, down, n_experts, out_dtype=torch.float32, routes=(dst, dst, bounds))
+
+
+def _experts_gemv(x, gate, up, down, topk_ids, n_mid, n_out):
+    """The same through one GEMV column per (token, slot): FP32 between the products, gate/up fused where a kernel is."""
+    if glu2_supported(gate, up):
+        hidden = mmv_glu2(x, gate, up, topk_ids, n_mid)
+    else:
+        hidden = swiglu(mmv(x, gate, topk_ids, n_mid), mmv(x, up, topk_ids, n_mid))
+    return mmv(hidden, down, topk_ids, n_out)
+
+
 def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_weights: torch.Tensor,
                 topk_ids: torch.Tensor, n_experts: int) -> torch.Tensor:
-    """Routed experts of one MoE layer: sum_k w_k * down(silu(gate x) * up x) over the top-k experts, BF16 out.
-    Few tokens (see below; or shapes without a batched kernel): expert GEMVs with FP32 activations between
-    them; more: the batched kernels (fused gate/up + SwiGLU written as BF16, then down)
-    (engines/vllm/vllm_bf16n/ops.py:251-271)."""
-    T = x.shape[0]
-    N = gate.meta.rows // n_experts
-    H = down.meta.rows // n_experts
+    """Routed experts of one MoE layer, BF16 out: for every token the weighted sum over its top-k experts of
+    down_e(silu(gate_e x) * (up_e x)) (engines/vllm/vllm_bf16n/ops.py:251-271).
+
+    The reference switches from expert GEMVs to the batched kernels above 8 tokens.  Here the GEMVs stay ahead only
+    while the routed pairs are few against the experts (each pair decodes one expert matrix in its own GEMV column; the
+    batched kernel decodes every active expert once).  Tile layout: up to 0.2 pairs per expert (6 tokens for top-8 of
+    256; measured 57 / 97 us GEMV against 64 / 83 us batched at 4 / 8 tokens), its batched kernel splits K over
+    wavefronts while few experts are active; other layouts: 0.7 and never below the reference's 8 tokens."""
+    n_tokens, n_used = x.shape[0], max(int(topk_ids.shape[1]), 1)
+    n_mid, n_out = gate.meta.rows // n_experts, down.meta.rows // n_experts
     x = x.contiguous()
-    # The reference switches to the batched kernels above 8 tokens.  Here the expert GEMVs stay ahead while the routed
-    # pairs are few against the experts (each pair decodes one expert matrix in its own GEMV column; the batched kernel
-    # decodes every active expert once).  Tile layout: up to 0.2 pairs per expert (6 tokens for top-8 of 256; measured
-    # 57 / 97 us GEMV against 64 / 83 us batched at 4 / 8 tokens), its batched kernel splits K over wavefronts while
-    # few experts are active; other layouts: 0.7 and never below the reference's 8 tokens.
     tiles = all(m.meta.wave64 and m.meta.R == 32 for m in (gate, up, down))
     per_expert = MOE_GEMV_PAIRS_PER_EXPERT[0 if tiles else 1]
-    gemv_tokens = max(4 if tiles else GEMV_MAX_TOKENS, int(per_expert * n_experts) // max(topk_ids.shape[1], 1))
-    if T > gemv_tokens and mm_ids_supported(gate, up) and mm_ids_supported(down):
-        # one routing pass for both products: with one activation row per (token, slot), as down takes them, the
-        # source row of a pair is its destination row
-        src1, dst, bounds = mm_ids_route(topk_ids, n_experts, False)
-        a = moe_mm_ids(x, topk_ids, gate, n_experts, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
-        ys = moe_mm_ids(a, topk_ids, down, n_experts, out_dtype=torch.float32, routes=(dst, dst, bounds))
-    elif glu2_supported(gate, up):
-        ys = mmv(mmv_glu2(x, gate, up, topk_ids, N), down, topk_ids, H)
+    gemv_tokens = max(4 if tiles else GEMV_MAX_TOKENS, int(per_expert * n_experts) // n_used)
+    if n_tokens > gemv_tokens and mm_ids_supported(gate, up) and mm_ids_supported(down):
+        per_pair = _experts_batched(x, gate, up, down, topk_ids, n_experts)
     else:
-        g = mmv(x, gate, topk_ids, N)
-        u = mmv(x, up, topk_ids, N)
-        ys = mmv(swiglu(g, u), down, topk_ids, H)
-    return moe_combine(ys, topk_weights, torch.bfloat16)
-
-
-def moe_experts_reference(x, gate, up, down, topk_weights, topk_ids, n_experts):
-    """Exact-weight reference in FP32 (dequant per used expert): slow, for tests
-    (engines/vllm/vllm_bf16n/ops.py:274-287)."""
-    N = gate.meta.rows // n_experts
-    H = down.meta.rows // n_experts
-    xf = x.float()
-    out = torch.zeros(x.shape[0], H, dtype=torch.float32, device=x.device)
-    for e in torch.unique(topk_ids).tolist():
-        tok, slot = (topk_ids == e).nonzero(as_tuple=True)
-        g = dequant(gate, e * N, N).float()
-        u = dequant(up, e * N, N).float()
-        d = dequant(down, e * H, H).float()
-        a = torch.nn.functional.silu(xf[tok] @ g.t()) * (xf[tok] @ u.t())
-        out.index_add_(0, tok, (a @ d.t()) * topk_weights[tok, slot].float()[:, None])
-    return out.to(torch.bfloat16)
+        per_pair = _experts_gemv(x, gate, up, down, topk_ids, n_mid, n_out)
+    return moe_combine(per_pair, topk_weights, torch.bfloat16)

@@ -61,9 +61,11 @@ int main() {
     } catch (const std::invalid_argument & ex) {
         std::printf("invalid_argument %s\n", ex.what());
     }
-    // a tensor must not be converted twice into the same storage
+    // a tensor must not be converted twice into the same storage, and the refused call leaves the resident tensor as
+    // it was (the source here is another one: the verify step below would notice its plane bytes)
     try {
-        ad::convert(ts[2].data, ts[2].host.data(), 2048, 512, 1, ad::tag::nibble, &owner_b, "again", bf16n::policy_engine::mi355x, false, false);
+        const std::vector<uint16_t> other(ts[2].host.size(), (uint16_t) 0x3F80);
+        ad::convert(ts[2].data, other.data(), 2048, 512, 1, ad::tag::nibble, &owner_b, "again", bf16n::policy_engine::mi355x, false, false);
         std::printf("no throw\n");
     } catch (const std::invalid_argument & ex) {
         std::printf("invalid_argument %s\n", ex.what());

@@ -126,3 +126,19 @@ def test_adapter_registry_on_the_host():
         assert L.bf16n_adapter_choose(512, 2048, 1, b"huffman", 8 << 20, 0, engine) == 2
         assert L.bf16n_adapter_choose(248320, 2048, 1, b"nibble", 8 << 20, 0, engine) == 1
         assert L.bf16n_adapter_choose(512, 1000, 1, b"hybrid", 8 << 20, 0, engine) == 0
+
+
+def test_verify_roundtrip_rejects_a_malformed_weight():
+    """K = 0 or R = 0 are divisors in the verify step: they must come back as EINVAL, not as a signal."""
+    import ctypes as C
+
+    from orin_qwen_lossless_amd import _lib
+
+    L = _lib.lib()
+    src = (C.c_uint16 * 1024)()
+    ok = C.c_int(-1)
+    for K, R, fmt in ((0, 4, 3), (1024, 0, 3), (1024, 0, 2), (1000, 4, 3), (1024, 4, 7)):
+        w = _lib.Weight()
+        w.plane, w.aux, w.format, w.R, w.K, w.rows = 0x1000, 0x2000, fmt, R, K, 64
+        with pytest.raises(ValueError, match="bf16n:"):
+            _lib.check(L.bf16n_verify_roundtrip(C.byref(w), src, C.byref(ok)))

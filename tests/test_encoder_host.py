@@ -179,6 +179,10 @@ def test_policy_mi355x():
     assert ops.choose(2048, 512, 256, expert=True) == (HP, 32, False, False, True)
     assert ops.choose(96, 1536, 8, expert=True) == (HP, 32, False, False, True)
     assert ops.choose(144, 2048, 8, expert=True) == (HP, 4, False, False, True)
+    # a stack of several matrices is an expert stack with or without the caller's flag (a C++ caller that leaves
+    # policy_options::expert at its default gets the same layout as one that sets it)
+    for shape in ((512, 2048, 256), (2048, 512, 256), (144, 2048, 8), (64, 512, 4)):
+        assert ops.choose(*shape, expert=False) == ops.choose(*shape, expert=True) and ops.choose(*shape)[0] == HP
     assert ops.choose(512, 2048)[0] == NIB and ops.choose(2048, 512)[0] == NIB and ops.choose(256, 2048)[0] == NIB
     # dense matrices of at least 131072 rows take the tiles when the caller asks for the matrix-core order
     assert ops.choose(248320, 2048, dense_frag_order=True) == (HP, 32, False, False, True)

@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 import torch
 
+from moe_exact import moe_layer_exact
 from orin_qwen_lossless_amd import synth
 from test_gpu_kernels import tbf16
 from test_gpu_roundtrip import enc
@@ -87,7 +88,7 @@ def test_moe_layer_graph(ops, T):
         assert torch.equal(out, want), rep
         seen.add(tuple(np.sort(ids.cpu().numpy(), axis=None).tolist()))
     assert len(seen) > 1  # the routing changed between replays: it is computed inside the graph
-    ref = ops.moe_experts_reference(x, gate, up, down, *ops.router_topk(ops.mmv(x, router)[:, :E].contiguous(), k), E)
+    ref = moe_layer_exact(ops, x, gate, up, down, *ops.router_topk(ops.mmv(x, router)[:, :E].contiguous(), k), E)
     scale = float(ref.float().abs().max())
     assert float((out.float() - ref.float()).abs().max()) <= 2e-2 * scale
 

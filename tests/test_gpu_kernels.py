@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from conftest import GEMV_REL
+from moe_exact import moe_layer_exact
 from orin_qwen_lossless_amd import synth
 from test_gpu_roundtrip import bits, enc
 
@@ -297,11 +298,8 @@ def test_router_topk(ops, oracle):
 @pytest.mark.parametrize("w64", [False, True])
 def test_moe_layer_decode(ops, oracle, T, w64):
     # the MoE decode layer at reduced expert count: router top-k on the GPU, gate/up GEMVs, SwiGLU, down, combine
-    E, N, H, K, k = 16, 64, 128, 1024, 4
-    gate_b, up_b, down_b = synth.weights(E * N, K, 41), synth.weights(E * N, K, 42), synth.weights(E * H, 512, 43)[:, :N] if False else synth.weights(E * H, 512, 43)
-    # down consumes N = 512 activations in the real layer; here N = 64 would not be a multiple of 512, so use N = 512
-    N = 512
-    gate_b, up_b = synth.weights(E * N, K, 41), synth.weights(E * N, K, 42)
+    E, N, H, K, k = 16, 512, 128, 1024, 4  # down consumes N activations: N must be a multiple of 512
+    gate_b, up_b, down_b = synth.weights(E * N, K, 41), synth.weights(E * N, K, 42), synth.weights(E * H, N, 43)
     gate = enc(ops, gate_b, HP, 8, not w64, w64)
     up_ = enc(ops, up_b, HP, 8, not w64, w64)
     down = enc(ops, down_b, HP, 16, False, w64)
@@ -311,7 +309,7 @@ def test_moe_layer_decode(ops, oracle, T, w64):
     logits = x.float() @ router.t()
     wts, ids = ops.router_topk(logits, k)
     y = ops.moe_experts(x, gate, up_, down, wts, ids, E)
-    ref = ops.moe_experts_reference(x, gate, up_, down, wts, ids.long(), E)
+    ref = moe_layer_exact(ops, x, gate, up_, down, wts, ids.long(), E)
     err = (y.float() - ref.float()).abs()
     tol = 2.0 ** -7 * ref.float().abs() + 1e-4
     assert bool((err <= tol).all()), float(err.max())

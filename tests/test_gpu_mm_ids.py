@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 import torch
 
+from moe_exact import moe_layer_exact
 from orin_qwen_lossless_amd import synth
 from test_gpu_kernels import rne_bf16, tbf16
 from test_gpu_roundtrip import bits, enc
@@ -160,7 +161,7 @@ def test_moe_experts_switches_to_batched_kernels(ops, T, cm, w64):
     wts = torch.softmax(torch.randn((T, k), generator=torch.Generator().manual_seed(T)), dim=-1).cuda()
     x = tbf16(synth.activations(T, Kd, 54))
     got = ops.moe_experts(x, gate, up, down, wts, ids, E).float().cpu().numpy()
-    ref = ops.moe_experts_reference(x, gate, up, down, wts, ids, E).float().cpu().numpy()
+    ref = moe_layer_exact(ops, x, gate, up, down, wts, ids, E).float().cpu().numpy()
     scale = np.abs(ref).max()
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
 

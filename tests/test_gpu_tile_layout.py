@@ -9,6 +9,7 @@ import pytest
 import torch
 
 from conftest import GEMV_REL
+from moe_exact import moe_layer_exact
 from orin_qwen_lossless_amd import synth
 from test_gpu_kernels import check_gemv, rne_bf16, tbf16
 from test_gpu_mm_ids import reference, routing
@@ -235,7 +236,7 @@ def test_moe_experts_in_both_token_regimes(ops, T):
     wts = torch.softmax(torch.randn((T, k), generator=torch.Generator().manual_seed(T)), dim=-1).cuda()
     x = tbf16(synth.activations(T, Kd, 54))
     got = ops.moe_experts(x, gate, up, down, wts, ids, E).float().cpu().numpy()
-    ref = ops.moe_experts_reference(x, gate, up, down, wts, ids, E).float().cpu().numpy()
+    ref = moe_layer_exact(ops, x, gate, up, down, wts, ids, E).float().cpu().numpy()
     scale = np.abs(ref).max()
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
 
@@ -256,6 +257,6 @@ def test_moe_experts_path_switch_by_routed_pairs_per_expert(ops, T, monkeypatch)
     x = tbf16(synth.activations(T, Kd, 84))
     got = ops.moe_experts(x, gate, up, down, wts, ids, E).float().cpu().numpy()
     assert len(batched_calls) == (0 if T <= 12 else 2)
-    ref = ops.moe_experts_reference(x, gate, up, down, wts, ids, E).float().cpu().numpy()
+    ref = moe_layer_exact(ops, x, gate, up, down, wts, ids, E).float().cpu().numpy()
     scale = np.abs(ref).max()
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
