@@ -255,3 +255,165 @@ def test_full_size_batched_moe_against_exact_weights_and_the_gemv_path(ops, expe
     # linearity in the activations: doubling them doubles every product exactly (powers of two commute with rounding)
     ys2 = ops.moe_mm_ids((a16.float() * 2).to(torch.bfloat16), ids, down, E, routes=(dst, dst, bounds))
     assert torch.equal(ys2, ys * 2)
+
+
+# ---- the benchmark configurations at their stated sizes ---------------------------------------------------------------
+
+def upload_policy(ops, w, n_matrices=1):
+    """Encode a [rows, K] BF16 device tensor in the layout the mi355x policy picks and upload it."""
+    rows, k = w.shape
+    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, k, n_matrices, engine="mi355x", expert=n_matrices > 1)
+    plane, aux, _, _ = ops.encode_bits(w.cpu().view(torch.int16).numpy().view(np.uint16), fmt, R, cm, wave64=w64)
+    ta = torch.from_numpy(aux)
+    return ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
+
+
+def silu64(g):
+    return g / (1.0 + torch.exp(-g))
+
+
+@pytest.mark.parametrize("T", [2048, 8192])
+def test_prefill_at_the_benchmark_token_counts(ops, oracle, experts, T):
+    """Batched MoE prefill of the 256-expert layer at 2048 and 8192 tokens: routing lists equal to the oracle's, and
+    sampled (token, slot) outputs of the fused gate/up product and of the down product against FP64 products of the
+    exact weights (1e-3 relative / 1e-5 absolute; and the reassociation bound 1e-5 * sum |w x| where the output is not
+    a product of rounded intermediates)."""
+    (wg, gate), (wu, up), (wd, down) = experts
+    g = torch.Generator(device="cuda").manual_seed(100 + T)
+    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
+    wts, ids = ops.router_topk(torch.randn((T, E), generator=g, device="cuda"), TOPK)
+    src1, dst, bounds = ops.mm_ids_route(ids, E, False)
+    o_src1, o_dst, o_bounds = oracle.route(ids.cpu().numpy(), E, 1, 1)
+    assert np.array_equal(bounds.cpu().numpy(), o_bounds)
+    assert np.array_equal(dst.cpu().numpy(), o_dst) and np.array_equal(src1.cpu().numpy(), o_src1)
+    load = np.diff(o_bounds)
+    assert load.min() > 0 and load.max() < 2 * T * TOPK // E    # near-uniform expert load, as the configuration states
+    a = ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.float32, routes=(src1, dst, bounds))
+    a16 = ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
+    assert torch.equal(a16, a.to(torch.bfloat16))                # BF16 out is the rounding of the FP32 accumulators
+    ys = ops.moe_mm_ids(a16, ids, down, E, routes=(dst, dst, bounds))
+    rng = np.random.default_rng(T)
+    tokens = [0, T - 1] + rng.integers(1, T - 1, 30).tolist()
+    for t in tokens:
+        xe = x[t].double()
+        for s in range(TOPK):
+            e = int(ids[t, s])
+            gg, uu = wg[e * N:(e + 1) * N].double() @ xe, wu[e * N:(e + 1) * N].double() @ xe
+            want = uu * silu64(gg)
+            assert torch.all((a[t, s].double() - want).abs() <= 1e-3 * want.abs() + 1e-5), (t, s)
+            h = a16[t, s].double()
+            wde = wd[e * K:(e + 1) * K].double()
+            want_y, bound = wde @ h, wde.abs() @ h.abs()
+            err = (ys[t, s].double() - want_y).abs()
+            assert torch.all(err <= 1e-5 * bound), (t, s)
+            assert torch.all(err <= 1e-3 * want_y.abs() + 1e-5), (t, s)
+    # the layer through moe_experts (routing lists, both products, weighted sum) for the sampled tokens
+    y = ops.moe_experts(x, gate, up, down, wts, ids, E)
+    comb = (ys[tokens].double() * wts[tokens].double().unsqueeze(-1)).sum(1)
+    assert torch.all((y[tokens].double() - comb).abs() <= 2.0 ** -8 * comb.abs() + 1e-6)
+
+
+@pytest.fixture(scope="module")
+def moe_small_parts(ops):
+    """Router 256 x 2048 and the shared expert ([gate; up] 1024 x 2048, down 2048 x 512) under the mi355x policy."""
+    g = torch.Generator(device="cuda").manual_seed(21)
+    ws = {name: (torch.randn(shape, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+          for name, shape in (("router", (E, K)), ("sh_gate_up", (2 * N, K)), ("sh_down", (K, N)))}
+    return {name: (w, upload_policy(ops, w)) for name, w in ws.items()}
+
+
+def graph_of(fn):
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = fn()
+    return g, out
+
+
+@pytest.mark.parametrize("T", [1, 4])
+def test_moe_decode_layer_256_experts_as_one_graph(ops, experts, moe_small_parts, T):
+    """The MoE decode layer at its stated size (256 experts as 32 x 256 tiles, top-8 chosen on the device from the
+    router's logits, shared expert) captured as one HIP graph: every replay on new activations equals the eager result
+    bit for bit, the routing changes between replays, and the result agrees with FP64 on the exact weights."""
+    (wg, gate), (wu, up), (wd, down) = experts
+    (wr, router), (wsg, sh_gu), (wsd, sh_dn) = (moe_small_parts[k] for k in ("router", "sh_gate_up", "sh_down"))
+    assert all(m.meta.format == 1 for m in (router, sh_gu, sh_dn))   # small matrices: the fixed 4-bit code
+    g = torch.Generator(device="cuda").manual_seed(30 + T)
+    xs = [torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16) for _ in range(4)]
+    x = xs[0].clone()
+
+    def layer():
+        wts, ids = ops.router_topk(ops.mmv(x, router), TOPK)
+        routed = ops.moe_experts(x, gate, up, down, wts, ids, E)
+        shared = ops.mmv(ops.mmv_glu(x, sh_gu), sh_dn, out_dtype=torch.bfloat16)
+        return routed, shared, ids, wts
+
+    graph, outs = graph_of(layer)
+    seen = set()
+    for rep in range(4):
+        x.copy_(xs[rep])
+        want = [t.clone() for t in layer()]
+        torch.cuda.synchronize()
+        for t in outs:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip(outs, want):
+            assert torch.equal(got, ref), rep
+        seen.add(tuple(outs[2].cpu().numpy().reshape(-1).tolist()))
+    assert len(seen) == 4
+    routed, shared, ids, wts = outs
+    xd = x.double()
+    # the router: logits of the exact weights, the same top-8 (no ties in random data), softmax weights renormalised
+    logits = xd @ wr.double().t()
+    top = torch.topk(logits, TOPK, dim=-1)
+    assert torch.equal(top.indices.int(), ids)
+    p = torch.softmax(logits, -1).gather(1, top.indices)
+    assert torch.allclose(wts.double(), p / p.sum(-1, keepdim=True), rtol=1e-4, atol=1e-7)
+    for t in range(T):
+        acc = torch.zeros(K, dtype=torch.float64, device="cuda")
+        for s in range(TOPK):
+            e = int(ids[t, s])
+            h = silu64(wg[e * N:(e + 1) * N].double() @ xd[t]) * (wu[e * N:(e + 1) * N].double() @ xd[t])
+            acc += float(wts[t, s]) * (wd[e * K:(e + 1) * K].double() @ h)
+        assert torch.all((routed[t].double() - acc).abs() <= 2.0 ** -7 * acc.abs() + 1e-5), t
+        h = silu64(wsg[:N].double() @ xd[t]) * (wsg[N:].double() @ xd[t])
+        want_sh = wsd.double() @ h
+        assert torch.all((shared[t].double() - want_sh).abs() <= 2.0 ** -7 * want_sh.abs() + 1e-5), t
+
+
+@pytest.mark.parametrize("name,rows,k,R", [("qkv", 5120, 2048, 2), ("o", 2048, 4096, 1), ("cfg1", 2048, 2048, 2)])
+def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, R):
+    """The per-layer dense projections in the layouts the mi355x policy gives them (short wave64 units), and the
+    2048 x 2048 matrix of the CPU reference configuration, at batch 1 and 4 against the oracle's FP32-accumulated GEMV
+    and its FP64 bound; the decode is bit-exact and the pair table equals the oracle encoder's."""
+    from orin_qwen_lossless_amd import synth
+
+    wb = synth.weights(rows, k, 500 + rows % 97)
+    # 2048 x 2048 is below the policy's dense minimum (it would take the 4-bit code); its configuration names the pair
+    # code, so the policy is asked for the Huffman family there
+    fmt, r, cm, _, w64 = ops.choose(rows, k, engine="mi355x", mode="huffman" if name == "cfg1" else "hybrid")
+    assert (fmt, r, cm, w64) == (3, R, False, True)
+    plane, aux, _, _ = ops.encode_bits(wb, fmt, r, cm, wave64=w64)
+    assert np.array_equal(oracle.decode(plane, aux), wb)
+    ta = torch.from_numpy(aux)
+    enc = ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
+    assert ops.roundtrip_equal(enc, torch.from_numpy(wb.view(np.int16)).view(torch.bfloat16))
+    xb = synth.activations(4, k, 77)
+    x = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16).cuda()
+    y4 = ops.mmv(x, enc).cpu().numpy()
+    for t in range(4):
+        xf = synth.bf16_bits_to_f32(xb[t])
+        ref32 = oracle.gemv_f32(wb, xf)
+        y64, bound = oracle.gemv_f64(wb, xf)
+        y1 = ops.mmv(x[t: t + 1], enc).cpu().numpy()[0]
+        assert np.array_equal(y1, y4[t])                       # batch 4 = four batch-1 products, bit for bit
+        assert np.all(np.abs(y1 - ref32) <= 1e-3 * np.abs(ref32) + 1e-5)
+        assert np.all(np.abs(y1 - y64) <= 1e-5 * bound)
+    y16 = ops.linear(x, enc)
+    assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y4))
