@@ -89,6 +89,18 @@ int bf16n_mm_ids_route(const void * ids, int ids_i64, int64_t ids_row_stride, in
 int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row,
                  const int32_t * ids_src1, const int32_t * ids_dst, const int32_t * bounds, void * dst, int dst_bf16,
                  int64_t dst_col, int n_experts, int n_tok, int n_used, void * stream);          /* launch.h:77-79, launch.cu:473-535 */
+/* No counterpart in the reference.  bf16n_mm_ids_route + bf16n_mm_ids in one call that allocates nothing, for callers
+ * that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid it): the
+ * routing lists are kept in a device array that belongs to the library (about 516 KiB per GPU, held until the process
+ * ends) instead of buffers of the caller.  ids: n_tok x n_used expert ids (int32, or int64 with ids_i64; row stride in
+ * elements); per_slot: x holds one activation row per (token, slot) (the down product) instead of one per token.  At
+ * most 65536 routed pairs (n_tok * n_used) and 1024 experts per call, EINVAL beyond.  dst gets the bits that
+ * bf16n_mm_ids writes for the same arguments.  All calls on one GPU share the array: calls that can overlap on one GPU
+ * (different streams, different threads) race; calls on one stream are ordered.  Call bf16n_init() on every GPU before
+ * the first capture. */
+int bf16n_moe_mm_ids_static(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const void * ids,
+                            int ids_i64, int64_t ids_row_stride, int per_slot, void * dst, int dst_bf16, int64_t dst_col,
+                            int n_experts, int n_tok, int n_used, void * stream);
 int bf16n_moe_combine(const float * ys, const void * w, int w_bf16, void * y, int y_bf16, int n_tok, int n_used,
                       int64_t n, void * stream);                                                /* launch.h:82-83, launch.cu:562-572 */
 int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * stream);       /* launch.h:85, launch.cu:574-582 */

@@ -29,6 +29,23 @@ int g_cus = 0;
 int g_lds_max = 0;
 std::once_flag g_once;
 
+// Routing lists of bf16n_moe_mm_ids_static: device memory that belongs to the library, so that the call allocates
+// nothing.  Every GPU holds its own copy of the array for the life of the process (about 516 KiB).  In host code the
+// array's name is not a device address; the address on a device comes from hipGetSymbolAddress with that device
+// current, once per device (route_lists_of_current_device), and only that pointer is handed to kernels.
+constexpr int STATIC_MAX_PAIRS = 1 << 16;   // routed (token, slot) pairs per call: 8192 tokens of top-8
+constexpr int STATIC_MAX_EXPERTS = 1024;
+struct route_lists {
+    int32_t src1[STATIC_MAX_PAIRS];
+    int32_t dst[STATIC_MAX_PAIRS];
+    int32_t bounds[STATIC_MAX_EXPERTS + 64];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(route_lists)];
+
+constexpr int MAX_DEVICES = 64;
+route_lists * g_route_lists[MAX_DEVICES] = {};
+std::mutex g_route_lists_mutex;
+
 void require(bool cond, const char * msg) {
     if (!cond) {
         throw std::invalid_argument(std::string("bf16n: ") + msg);
@@ -41,6 +58,21 @@ void hip_check(hipError_t e, const char * what) {
     }
 }
 
+route_lists * route_lists_of_current_device() {
+    int dev = 0;
+    hip_check(hipGetDevice(&dev), "hipGetDevice");
+    if (dev < 0 || dev >= MAX_DEVICES) {
+        throw std::runtime_error("bf16n: device ordinal beyond the library's per-device tables");
+    }
+    std::lock_guard<std::mutex> lock(g_route_lists_mutex);
+    if (!g_route_lists[dev]) {
+        void * p = nullptr;
+        hip_check(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress (routing lists)");
+        g_route_lists[dev] = static_cast<route_lists *>(p);
+    }
+    return g_route_lists[dev];
+}
+
 void ensure_init() {
     std::call_once(g_once, [] {
         int dev = 0;
@@ -51,6 +83,7 @@ void ensure_init() {
         dev::mm_ids_init();
         dev::tile_init();
     });
+    (void) route_lists_of_current_device(); // per device; after the first call on a device this is a table lookup
 }
 
 template <typename F>
@@ -385,6 +418,43 @@ int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x
                                     (int64_t) n_tok * n_used, g_cus, (hipStream_t) stream);
         } else {
             dev::launch_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, n_tok, n_used,
+                               g_cus, (hipStream_t) stream);
+        }
+        launch_check("mm_ids");
+    });
+}
+
+// Routing lists + batched product in one call that allocates nothing: the lists live in the library's own device array
+// (see `scratch` above).  No counterpart in the reference, whose callers allocate the lists per call.
+int bf16n_moe_mm_ids_static(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const void * ids,
+                            int ids_i64, int64_t ids_row_stride, int per_slot, void * dst, int dst_bf16, int64_t dst_col,
+                            int n_experts, int n_tok, int n_used, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(dev::mm_ids_shape_ok(*w, up), "no batched kernel for this matrix");
+        require(n_experts > 0 && w->rows % n_experts == 0, "rows must split evenly into experts");
+        if (up) {
+            check_weight(*up);
+        }
+        require(x_bf16 && dst && ids, "null pointer");
+        require(n_tok > 0 && n_used > 0 && n_used < (1 << 10), "routing sizes out of range");
+        require(n_experts <= STATIC_MAX_EXPERTS && (int64_t) n_tok * n_used <= STATIC_MAX_PAIRS,
+                "moe_mm_ids_static: at most 65536 routed pairs and 1024 experts per call (use mm_ids_route + mm_ids beyond)");
+        require((int64_t) n_tok * ids_row_stride < INT32_MAX, "routing ids too large for 32-bit indexing");
+        require(((uintptr_t) x_bf16 & 15) == 0 && x_row % 8 == 0, "activations must be 16-byte aligned with 16-byte row strides");
+        require(((uintptr_t) dst & 15) == 0 && dst_col % 4 == 0, "dst must be 16-byte aligned with a column stride that is a multiple of 4");
+        route_lists * r = route_lists_of_current_device();
+        const int nch = per_slot ? n_used : 1; // activations per (token, slot), as the down product takes them, or per token
+        // every list entry and every bound the product reads is rewritten by the routing kernel: nothing to clear
+        dev::launch_route(ids, ids_i64 != 0, ids_row_stride, r->src1, r->dst, r->bounds, n_experts, n_tok, n_used, nch, nch,
+                          (hipStream_t) stream);
+        launch_check("mm_ids_route");
+        if (dev::is_tile_layout(*w)) {
+            dev::launch_tile_mm_ids(*w, up, x_bf16, x_row, r->src1, r->dst, r->bounds, dst, dst_bf16 != 0, dst_col, n_experts,
+                                    (int64_t) n_tok * n_used, g_cus, (hipStream_t) stream);
+        } else {
+            dev::launch_mm_ids(*w, up, x_bf16, x_row, r->src1, r->dst, r->bounds, dst, dst_bf16 != 0, dst_col, n_experts, n_tok, n_used,
                                g_cus, (hipStream_t) stream);
         }
         launch_check("mm_ids");
