@@ -16,14 +16,34 @@ constexpr int WAVE_LDS_WORDS = RING + RING_PAD;
 
 // 16 bytes that a launch reads once, loaded with the non-temporal hint: 8 % faster on the 248320 x 2048 GEMV (126
 // against 136 us). Planes that other columns or passes of the launch read again (routed experts with many tokens, small
-// matrices in a column loop) keep the default policy, which is faster there. Stream blocks start at any 16-byte
-// boundary, so consecutive blocks share a cache line, and with the hint that line is fetched twice (3 % more memory
-// traffic): the GEMVs and the routed batched kernels are still faster with it inside a decode step, a large dense matrix
-// in the batched tile kernel is 5 % slower, so the stream hint is a flag of its own (w64_dec::once)
+// matrices in a column loop) keep the default policy, which is faster there. Stream blocks start on 128-byte lines, so
+// no line belongs to two blocks (with the hint a shared line is fetched twice): the GEMVs and the routed batched
+// kernels are faster with the hint inside a decode step, a large dense matrix in the batched tile kernel is not, so the
+// stream hint is a flag of its own (w64_dec::once)
 typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 load_once(const uint4 * p) {
     const u32x4_nt v = __builtin_nontemporal_load((const u32x4_nt *) p);
     return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// A byte range of device memory behind a buffer descriptor.  The decode loops prefetch a fixed distance ahead with
+// loads that are issued unconditionally (so that the count of loads in flight at every wait is known at compile time);
+// near the end of a wavefront's range those loads point past it.  Through a descriptor such a load is dropped by the
+// address unit and returns zeros: no memory request (clamping the address to the last block instead re-fetched it, and
+// with the non-temporal hint every such repeat went to memory again: 3 KiB per decode chain, 3.6 % of the traffic of
+// the output projection).  The whole offset travels in the vector operand, which is what the range check looks at.
+typedef __amdgpu_buffer_rsrc_t range_t;
+__device__ __forceinline__ range_t make_range(const void * base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int) bytes, 0x00020000); // raw buffer, 32-bit data
+}
+template <bool ONCE>
+__device__ __forceinline__ uint4 range_load16(range_t r, uint32_t byte_off) {
+    const u32x4_nt v = ONCE ? __builtin_amdgcn_raw_buffer_load_b128(r, (int) byte_off, 0, 2)   // nt
+                            : __builtin_amdgcn_raw_buffer_load_b128(r, (int) byte_off, 0, 0);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint4 range_load16(range_t r, uint32_t byte_off, bool once) {
+    return once ? range_load16<true>(r, byte_off) : range_load16<false>(r, byte_off);
 }
 
 struct w64_ptrs { const uint8_t * plane; const uint32_t * lut; const uint32_t * ubase; const uint32_t * stream; };
@@ -59,18 +79,17 @@ struct w64_dec {
     uint64_t took;          // lanes that requested a word at the last check
     uint32_t cons;          // words consumed, relative to src
     uint32_t filled;        // words copied into the ring, relative to src (multiple of BLK)
-    uint32_t last_block;    // first word of the last block that holds words of this wave, relative to src
     uint32_t * ring;
-    const uint32_t * src;   // 16-byte aligned
+    range_t src;            // the blocks that hold words of this wave (starts on a 128-byte line)
     uint4 pend;             // the block that starts at `filled`, in flight
     int lane;
     bool once;              // stream blocks with the non-temporal hint (same in every lane)
 
-    // Every load is unconditional (a block or step past the end re-reads the last one) so that the number of loads in
-    // flight at any point of the loop is fixed and the waits for prefetched data never drain newer loads.
+    // Every load is unconditional (a block past the end is dropped by the range check and reads as zeros) so that the
+    // number of loads in flight at any point of the loop is fixed and the waits for prefetched data never drain newer
+    // loads.
     __device__ __forceinline__ uint4 load_block(uint32_t first_word) const {
-        const uint32_t w = first_word < last_block ? first_word : last_block;
-        return once ? load_once((const uint4 *) (src + w) + lane) : *((const uint4 *) (src + w) + lane);
+        return range_load16(src, 4 * first_word + 16 * (uint32_t) lane, once);
     }
     __device__ __forceinline__ void store_block(uint32_t first_word, const uint4 v) {
         const uint32_t off = first_word & (RING - 1);
@@ -89,9 +108,10 @@ struct w64_dec {
         // of the section that precedes the stream in the same buffer (the header and the table come first)
         const uint32_t a4 = first & ~3u;
         const int32_t a = (int32_t) a4 - (int32_t) (((uintptr_t) (stream + a4) & 127u) >> 2);
-        src = stream + (int32_t) uniform((uint32_t) a); // kernel-argument pointer + scalar offset: stays a global, scalar address
         cons = (uint32_t) ((int32_t) first - a);
-        last_block = (uint32_t) ((int32_t) end - a - 1) / BLK * BLK; // the stream is padded: a block may run past `end`
+        // whole blocks up to the one that holds the last word (the stream is padded: a block may run past `end`)
+        const uint32_t blocks = (uint32_t) ((int32_t) end - a - 1) / BLK + 1;
+        src = make_range(stream + (int32_t) uniform((uint32_t) a), uniform(blocks * BLK * 4));
         const uint4 b0 = load_block(0);
         pend = load_block(BLK);
         store_block(0, b0);

@@ -38,13 +38,11 @@ __device__ __forceinline__ int tile_col(int s, int j, int half) { return 32 * s 
 // asks the same for the stream blocks, which pays for routed experts and not for a large dense matrix
 template <int D, bool ONCE = false> struct tchain_t {
     w64_dec dec;
-    const uint8_t * plane;
-    uint32_t off, last;
+    range_t plane;   // the plane bytes of the chain's tiles
+    uint32_t off;    // byte offset of this lane's 16 bytes in the next step to load
     uint4 sm[D];
-    __device__ __forceinline__ uint4 load_step(int lane) const {
-        const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
-        const uint4 * src = (const uint4 *) (plane + o) + lane;
-        return ONCE ? load_once(src) : *src;
+    __device__ __forceinline__ uint4 load_step(int) const { // past the end of the chain: dropped, reads as zeros
+        return range_load16<ONCE>(plane, off);
     }
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane, bool stream_once = false) {
         start(ring, q, unit0, n_units, lane, q.ubase[unit0], q.ubase[unit0 + n_units], stream_once);
@@ -52,9 +50,8 @@ template <int D, bool ONCE = false> struct tchain_t {
     // first / end: the stream words of the units (their unit bases, read by the caller ahead of time)
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane, uint32_t first,
                                           uint32_t end, bool stream_once = false) {
-        plane = q.plane + uniform64(unit0 * T_BYTES);
-        off = 0;
-        last = (uint32_t) (n_units * T_BYTES - STEP_BYTES);
+        plane = make_range(q.plane + uniform64(unit0 * T_BYTES), uniform((uint32_t) (n_units * T_BYTES)));
+        off = 16 * (uint32_t) lane;
 #pragma unroll
         for (int s = 0; s < D; s++) {
             sm[s] = load_step(lane);

@@ -78,23 +78,20 @@ template <int C> struct geom {
 template <int NB>
 struct chain {
     w64_dec dec;
-    const uint8_t * plane; // first plane byte of the chain's units (uniform)
-    uint32_t off;          // byte offset of the next step to load
-    uint32_t last;         // byte offset of the chain's last step
+    range_t plane;         // the plane bytes of the chain's units
+    uint32_t off;          // byte offset of this lane's 16 bytes in the next step to load
     uint4 sm[NB];          // plane bytes of the body's steps
     int64_t row;           // output row of the next body, relative to the product
     bool once;             // the launch reads the plane bytes once (see load_once)
-    __device__ __forceinline__ uint4 load_step(int lane) const {
-        const uint32_t o = off < last ? off : last; // past the end: the last step again, never used
-        return once ? load_once((const uint4 *) (plane + o) + lane) : *((const uint4 *) (plane + o) + lane);
+    __device__ __forceinline__ uint4 load_step(int) const { // past the end of the chain: dropped, reads as zeros
+        return range_load16(plane, off, once);
     }
     // first / end: the stream words of units [gu0, gu0 + n_units) (unit bases, read by the caller ahead of time)
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t gu0, int64_t n_units, int64_t row0, int R, int K,
                                           int lane, uint32_t first, uint32_t end, bool once_ = false, bool stream_once = false) {
         once = once_;
-        plane = q.plane + uniform64(gu0 * R * K);
-        off = 0;
-        last = (uint32_t) (n_units * R * K - 1024);
+        plane = make_range(q.plane + uniform64(gu0 * R * K), uniform((uint32_t) (n_units * R * K)));
+        off = 16 * (uint32_t) lane;
         row = row0;
 #pragma unroll
         for (int s = 0; s < NB; s++) {
