@@ -112,6 +112,13 @@ int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * 
 int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
                       int32_t * ids, float * weights, void * stream);
 
+/* Read-bandwidth probe (the reference's bench/micro/bwprobe.cu:23-60 as a library call): a kernel that only reads
+ * `bytes` (rounded down to whole KiB) from src, for the memory rate this GPU gives a pure streaming read.  pattern 0:
+ * every wavefront walks its own contiguous range in 1 KiB pieces with non-temporal 16-byte loads, four in flight (the
+ * fused GEMV's access pattern); 1: the same with plain loads; 2 / 3: grid-stride, non-temporal / plain.  waves_per_cu:
+ * wavefronts per CU, 0 = 16 (the fused GEMV's occupancy).  sink: one device word (never written for ordinary data). */
+int bf16n_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, void * stream);
+
 /* ---- load-time conversion and the registry of resident tensors: the reference's llama.cpp adapter without ggml types
  * (engines/llamacpp/patches/0002-ggml-cuda-thin-BF16N-adapter-over-the-shared-core.patch).  An engine stores a converted
  * tensor as rows * K bytes of device memory (the plane); the aux buffer is allocated here and found again by the

@@ -14,9 +14,10 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libbf16n_hip.so")
+BENCH = os.path.join(HERE, "bf16n_bench")  # stand-alone timing program (csrc/bench_mmv.cpp), linked against the library
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "adapter.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip"]
+SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "adapter.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip", "kernels_probe.hip"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall", "-Wno-unused-function"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -45,6 +46,13 @@ def build(force: bool = False) -> str:
         if r.returncode != 0:
             sys.stderr.write(r.stdout + r.stderr)
             raise RuntimeError("link failed")
+    bench_src = os.path.join(CSRC, "bench_mmv.cpp")
+    if force or not os.path.exists(BENCH) or os.path.getmtime(BENCH) < max(os.path.getmtime(bench_src), os.path.getmtime(LIB)):
+        r = subprocess.run([HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", "-I" + os.path.join(ROOT, "include"), bench_src,
+                            "-o", BENCH, "-L" + HERE, "-lbf16n_hip", "-Wl,-rpath,$ORIGIN", "-lpthread"], capture_output=True, text=True)
+        if r.returncode != 0:
+            sys.stderr.write(r.stdout + r.stderr)
+            raise RuntimeError("building bf16n_bench failed")
     return LIB
 
 

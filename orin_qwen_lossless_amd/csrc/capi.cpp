@@ -487,6 +487,20 @@ int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * 
     });
 }
 
+// bench/micro/bwprobe.cu:23-60 of the reference, as a call: a kernel that only reads
+int bf16n_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        require(src && sink && ((uintptr_t) src & 15) == 0, "read_probe: src must be 16-byte aligned, sink non-null");
+        require(pattern >= 0 && pattern <= 3, "read_probe: pattern must be 0..3");
+        require(bytes >= 1024 && waves_per_cu >= 0 && waves_per_cu <= 32, "read_probe: sizes out of range");
+        // a wavefront's range is addressed with 32-bit offsets
+        require(bytes / 1024 / ((uint64_t) g_cus * (waves_per_cu > 0 ? waves_per_cu : 16)) < (1u << 21), "read_probe: buffer too large");
+        dev::launch_read_probe(src, bytes, pattern, waves_per_cu, sink, g_cus, (hipStream_t) stream);
+        launch_check("read_probe");
+    });
+}
+
 int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
                       int32_t * ids, float * weights, void * stream) {
     return guarded([&] {

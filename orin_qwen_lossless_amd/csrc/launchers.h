@@ -53,6 +53,9 @@ void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_
 void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
                         float * weights, hipStream_t stream);
 
+// read-bandwidth probe (kernels_probe.hip)
+void launch_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, int cus, hipStream_t stream);
+
 // batched MoE prefill (kernels_mm_ids.hip)
 void mm_ids_init();
 bool mm_ids_shape_ok(const bf16n_weight & w, const bf16n_weight * up);

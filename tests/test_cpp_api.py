@@ -142,3 +142,19 @@ def test_verify_roundtrip_rejects_a_malformed_weight():
         w.plane, w.aux, w.format, w.R, w.K, w.rows = 0x1000, 0x2000, fmt, R, K, 64
         with pytest.raises(ValueError, match="bf16n:"):
             _lib.check(L.bf16n_verify_roundtrip(C.byref(w), src, C.byref(ok)))
+
+
+@pytest.mark.gpu
+def test_standalone_bench_program_runs():
+    """The torch-free timing program (csrc/bench_mmv.cpp, built next to the library): a small matrix, the bit-exact
+    verify and FP64 check it does before timing, and the read probe's four patterns."""
+    import json
+
+    exe = os.path.join(LIBDIR, "bf16n_bench")
+    assert os.path.exists(exe), "build it with python -m orin_qwen_lossless_amd.build"
+    for extra in ([], ["--tiles", "--rows", "131072", "--K", "1024", "--batch", "3"], ["--f32"]):
+        r = subprocess.run([exe, "--rows", "16384", "--reps", "5", "--warm-ms", "5", "--probe"] + extra, check=True,
+                           capture_output=True, text=True, timeout=120)
+        d = json.loads(r.stdout)
+        assert d["max_err_over_sum_abs"] <= 1e-5 and d["median_us"] > 0 and d["GBps"] > 0
+        assert all(d[f"read_{p}_w16_GBps"] > 100 for p in ("ranges_nt", "ranges_plain", "stride_nt", "stride_plain"))
