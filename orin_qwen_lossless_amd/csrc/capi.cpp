@@ -475,6 +475,55 @@ int bf16n_moe_combine(const float * ys, const void * w, int w_bf16, void * y, in
     });
 }
 
+// The routed down product and the weighted sum over a token's experts as one call: bf16n_mmv with expert ids into
+// per-slot FP32 rows followed by bf16n_moe_combine (launch.cu:313-325 and :562-572), with the same bits.  Tile-layout
+// matrices with at most sixteen slots run as one launch in which the per-slot rows stay on the chip; other shapes take
+// the two launches and need the per-slot workspace.
+int bf16n_moe_down_combine(const bf16n_weight * w, const bf16n_mmv_args * a, const void * wts, int wts_bf16, const void * add0,
+                           const void * add1, void * y, int y_bf16, int n_tok, float * ys_workspace, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(a->ids != nullptr && a->n_used > 0, "moe_down_combine: expert ids are required");
+        require(n_tok > 0 && n_tok <= 65535 && a->ncols == n_tok * a->n_used, "moe_down_combine: ncols must be n_tok * n_used");
+        require(wts && y, "null pointer");
+        require(w->format == FMT_NIBBLE || (a->nrows % w->R == 0 && a->row0 % w->R == 0 && a->rows_per_matrix % w->R == 0),
+                "rows of a product must be whole units");
+        if (a->nrows == 0) {
+            return;
+        }
+        dev::cols p = make_cols(*a);
+        if (dev::tile_down_combine_fits(*w, a->n_used)) {
+            dev::launch_tile_down_combine(*w, p, n_tok, a->x_bf16 != 0, wts, wts_bf16 != 0, add0, add1, y, y_bf16 != 0, (hipStream_t) stream);
+            launch_check("moe_down_combine");
+            return;
+        }
+        require(ys_workspace != nullptr, "moe_down_combine: this layout needs the per-slot workspace (n_tok * n_used * nrows floats)");
+        bf16n_mmv_args b = *a;
+        b.y = ys_workspace;
+        b.y_bf16 = 0;
+        b.y_slot = a->nrows * 4;
+        b.y_tok = (int64_t) a->n_used * a->nrows * 4;
+        if (bf16n_mmv(w, &b, stream, 1) != BF16N_OK) {
+            throw std::invalid_argument(bf16n_last_error());
+        }
+        dev::launch_moe_combine(ys_workspace, wts, wts_bf16 != 0, y, y_bf16 != 0, n_tok, a->n_used, a->nrows, (hipStream_t) stream, add0, add1);
+        launch_check("moe_down_combine");
+    });
+}
+
+// Residual add + RMS norm between the products of a decode step, one launch (engine glue; no counterpart in the
+// reference's core, whose engines bring their own)
+int bf16n_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const uint16_t * gamma, uint16_t * y_sum,
+                      uint16_t * y_norm, int n_tok, int64_t n, float eps, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        require(a && y_norm && n_tok > 0 && n_tok <= 65535 && n > 0, "add_rmsnorm: null pointer or empty input");
+        dev::launch_add_rmsnorm(a, b, c, gamma, y_sum, y_norm, n_tok, n, eps, (hipStream_t) stream);
+        launch_check("add_rmsnorm");
+    });
+}
+
 // launch.cu:574-582
 int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * stream) {
     return guarded([&] {

@@ -16,9 +16,11 @@ __global__ void __launch_bounds__(256) k_swiglu(const float * __restrict__ g, co
     }
 }
 
-// y[t, i] = sum_k w[t, k] * ys[t, k, i], slots in order, one fmaf each (reference launch.cu:539-552)
+// y[t, i] = sum_k w[t, k] * ys[t, k, i], slots in order, one fmaf each (reference launch.cu:539-552); then the optional
+// BF16 vectors add0[t, i], add1[t, i] in FP32 before the rounding
 __global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ ys, const char * __restrict__ w, bool w_bf16,
-                                                     char * __restrict__ y, bool y_bf16, int n_used, int64_t n) {
+                                                     char * __restrict__ y, bool y_bf16, int n_used, int64_t n,
+                                                     const uint16_t * __restrict__ add0, const uint16_t * __restrict__ add1) {
     const int t = blockIdx.y;
     for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) {
         float acc = 0.f;
@@ -26,6 +28,12 @@ __global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ 
             const int64_t s = (int64_t) t * n_used + k;
             const float wk = w_bf16 ? bf16_bits_to_f32(((const uint16_t *) w)[s]) : ((const float *) w)[s];
             acc = fmaf(wk, ys[s * n + i], acc);
+        }
+        if (add0) {
+            acc += bf16_bits_to_f32(add0[(int64_t) t * n + i]);
+        }
+        if (add1) {
+            acc += bf16_bits_to_f32(add1[(int64_t) t * n + i]);
         }
         store_y(y + (int64_t) t * n * (y_bf16 ? 2 : 4), y_bf16, i, acc);
     }
@@ -219,7 +227,61 @@ __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ l
     }
 }
 
+// Residual add + RMS norm of a decode step in one launch (the engines' glue between the products; llama.cpp fuses the
+// same chain in its graph).  Per token: sum = a + b + c in FP32 (b, c optional), y_sum = bf16(sum) (optional: the new
+// residual), y_norm = bf16(sum * rsqrt(mean(sum^2) + eps) * gamma) (gamma optional).  One block per token; the mean is
+// reduced in a fixed order, so the result does not depend on the launch.
+constexpr int NORM_THREADS = 256;
+__global__ void __launch_bounds__(NORM_THREADS) k_add_rmsnorm(const uint16_t * __restrict__ a, const uint16_t * __restrict__ b,
+                                                             const uint16_t * __restrict__ c, const uint16_t * __restrict__ gamma,
+                                                             uint16_t * __restrict__ y_sum, uint16_t * __restrict__ y_norm, int64_t n, float eps) {
+    __shared__ float wave_sq[NORM_THREADS / 64];
+    const int64_t base = (int64_t) blockIdx.x * n;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float sq = 0.f;
+    for (int64_t i = tid; i < n; i += NORM_THREADS) {
+        float v = bf16_bits_to_f32(a[base + i]);
+        if (b) {
+            v += bf16_bits_to_f32(b[base + i]);
+        }
+        if (c) {
+            v += bf16_bits_to_f32(c[base + i]);
+        }
+        sq = fmaf(v, v, sq);
+    }
+    sq = wave_sum(sq);
+    if (lane == 0) {
+        wave_sq[wave] = sq;
+    }
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int k = 0; k < NORM_THREADS / 64; k++) {
+        total += wave_sq[k];
+    }
+    const float scale = 1.0f / sqrtf(total / (float) n + eps);
+    for (int64_t i = tid; i < n; i += NORM_THREADS) {
+        float v = bf16_bits_to_f32(a[base + i]);
+        if (b) {
+            v += bf16_bits_to_f32(b[base + i]);
+        }
+        if (c) {
+            v += bf16_bits_to_f32(c[base + i]);
+        }
+        if (y_sum) {
+            y_sum[base + i] = f32_to_bf16_rne(v);
+        }
+        const float gmm = gamma ? bf16_bits_to_f32(gamma[i]) : 1.0f;
+        y_norm[base + i] = f32_to_bf16_rne(v * scale * gmm);
+    }
+}
+
 } // namespace
+
+void launch_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const uint16_t * gamma, uint16_t * y_sum,
+                        uint16_t * y_norm, int n_tok, int64_t n, float eps, hipStream_t stream) {
+    hipLaunchKernelGGL(k_add_rmsnorm, dim3(n_tok), dim3(NORM_THREADS), 0, stream, a, b, c, gamma, y_sum, y_norm, n, eps);
+}
 
 void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int cus, hipStream_t stream) {
     const int64_t blocks = (n + 255) / 256;
@@ -227,10 +289,10 @@ void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int c
 }
 
 void launch_moe_combine(const float * ys, const void * w, bool w_bf16, void * y, bool y_bf16, int n_tok, int n_used, int64_t n,
-                        hipStream_t stream) {
+                        hipStream_t stream, const void * add0, const void * add1) {
     const int64_t bx = (n + 255) / 256;
     hipLaunchKernelGGL(k_moe_combine, dim3((unsigned) (bx < 64 ? bx : 64), (unsigned) n_tok), dim3(256), 0, stream, ys, (const char *) w,
-                       w_bf16, (char *) y, y_bf16, n_used, n);
+                       w_bf16, (char *) y, y_bf16, n_used, n, (const uint16_t *) add0, (const uint16_t *) add1);
 }
 
 void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds,

@@ -501,6 +501,63 @@ def moe_combine(ys: torch.Tensor, topk_weights: torch.Tensor, out_dtype: torch.d
     return y
 
 
+def moe_down_combine(a: torch.Tensor, down: Weight, topk_ids: torch.Tensor, topk_weights: torch.Tensor, n_experts: int,
+                     add0: torch.Tensor | None = None, add1: torch.Tensor | None = None,
+                     out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """moe_combine(mmv(a, down, topk_ids, H), topk_weights) as one call with the same bits: a [T, n_used, N] hidden
+    activations of the routed experts, out [T, H].  add0 / add1: optional [T, H] BF16 tensors (a shared expert's
+    output, the residual) added in FP32 before the rounding.  Tile-layout matrices run as one launch."""
+    cw = _cweight(down)
+    _check_ids(topk_ids)
+    T, n_used = topk_ids.shape
+    H = down.meta.rows // n_experts
+    _check_x(a, down.meta.K, "a")
+    if a.dim() != 3 or tuple(a.shape[:2]) != (T, n_used):
+        raise ValueError("bf16n.moe_down_combine: a must be [tokens, n_used, N]")
+    if not (topk_weights.is_cuda and topk_weights.is_contiguous() and tuple(topk_weights.shape) == (T, n_used)
+            and topk_weights.dtype in (torch.float32, torch.bfloat16)):
+        raise ValueError("bf16n.moe_down_combine: topk_weights must be contiguous f32/bf16 [tokens, n_used]")
+    for t in (add0, add1):
+        if t is not None and not (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and tuple(t.shape) == (T, H)):
+            raise ValueError("bf16n.moe_down_combine: add tensors must be contiguous bf16 [tokens, H]")
+    y = torch.empty((T, H), dtype=out_dtype, device=a.device)
+    if T == 0:
+        return y
+    args = _lib.MmvArgs()
+    args.x, args.x_bf16 = a.data_ptr(), int(a.dtype == torch.bfloat16)
+    args.ncols, args.n_used, args.x_per_slot = T * n_used, n_used, n_used
+    args.ids, args.ids_s0, args.ids_s1 = topk_ids.data_ptr(), topk_ids.element_size(), topk_ids.stride(0) * topk_ids.element_size()
+    args.x_tok, args.x_slot = a.stride(0) * a.element_size(), a.stride(1) * a.element_size()
+    args.rows_per_matrix, args.row0, args.nrows = H, 0, H
+    tiles = down.meta.wave64 and down.meta.R == 32 and n_used <= 16
+    ws = None if tiles else torch.empty((T, n_used, H), dtype=torch.float32, device=a.device)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().bf16n_moe_down_combine(
+            C.byref(cw), C.byref(args), topk_weights.data_ptr(), int(topk_weights.dtype == torch.bfloat16),
+            add0.data_ptr() if add0 is not None else None, add1.data_ptr() if add1 is not None else None, y.data_ptr(),
+            int(out_dtype == torch.bfloat16), T, ws.data_ptr() if ws is not None else None, _stream()))
+    return y
+
+
+def add_rmsnorm(a: torch.Tensor, b: torch.Tensor | None = None, c: torch.Tensor | None = None, gamma: torch.Tensor | None = None,
+                eps: float = 1e-6, want_sum: bool = False):
+    """Engine glue of a decode step in one launch: s = a + b + c (FP32), returns bf16(s * rsqrt(mean(s^2) + eps) * gamma),
+    and bf16(s) too when want_sum.  a, b, c: [T, n] BF16 contiguous; gamma: [n] BF16."""
+    for t in (a, b, c):
+        if t is not None and not (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and t.shape == a.shape and t.dim() == 2):
+            raise ValueError("bf16n.add_rmsnorm: inputs must be contiguous bf16 [tokens, n] of one shape")
+    if gamma is not None and not (gamma.is_cuda and gamma.dtype == torch.bfloat16 and gamma.is_contiguous() and gamma.numel() == a.shape[1]):
+        raise ValueError("bf16n.add_rmsnorm: gamma must be contiguous bf16 [n]")
+    T, n = a.shape
+    y = torch.empty_like(a)
+    ysum = torch.empty_like(a) if want_sum else None
+    ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().bf16n_add_rmsnorm(a.data_ptr(), ptr(b), ptr(c), ptr(gamma), ptr(ysum), y.data_ptr(), T, n,
+                                                C.c_float(eps), _stream()))
+    return (y, ysum) if want_sum else y
+
+
 def swiglu(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
     if not (g.is_cuda and g.dtype == torch.float32 and g.is_contiguous() and u.shape == g.shape
             and u.dtype == torch.float32 and u.is_contiguous()):
@@ -540,13 +597,11 @@ def _experts_batched(x, gate, up, down, topk_ids, n_experts):
     return moe_mm_ids(hidden, topk_ids, down, n_experts, out_dtype=torch.float32, routes=(dst, dst, bounds))
 
 
-def _experts_gemv(x, gate, up, down, topk_ids, n_mid, n_out):
-    """The same through one GEMV column per (token, slot): FP32 between the products, gate/up fused where a kernel is."""
+def _experts_gemv_hidden(x, gate, up, topk_ids, n_mid):
+    """silu(gate x) * (up x) per (token, slot) in FP32 through one GEMV column each, fused where a kernel is."""
     if glu2_supported(gate, up):
-        hidden = mmv_glu2(x, gate, up, topk_ids, n_mid)
-    else:
-        hidden = swiglu(mmv(x, gate, topk_ids, n_mid), mmv(x, up, topk_ids, n_mid))
-    return mmv(hidden, down, topk_ids, n_out)
+        return mmv_glu2(x, gate, up, topk_ids, n_mid)
+    return swiglu(mmv(x, gate, topk_ids, n_mid), mmv(x, up, topk_ids, n_mid))
 
 
 def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_weights: torch.Tensor,
@@ -566,7 +621,8 @@ def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_we
     per_expert = MOE_GEMV_PAIRS_PER_EXPERT[0 if tiles else 1]
     gemv_tokens = max(4 if tiles else GEMV_MAX_TOKENS, int(per_expert * n_experts) // n_used)
     if n_tokens > gemv_tokens and mm_ids_supported(gate, up) and mm_ids_supported(down):
-        per_pair = _experts_batched(x, gate, up, down, topk_ids, n_experts)
-    else:
-        per_pair = _experts_gemv(x, gate, up, down, topk_ids, n_mid, n_out)
-    return moe_combine(per_pair, topk_weights, torch.bfloat16)
+        return moe_combine(_experts_batched(x, gate, up, down, topk_ids, n_experts), topk_weights, torch.bfloat16)
+    # one GEMV column per (token, slot), FP32 between the products; the down product and the weighted sum are one call
+    # (one launch for tile-layout experts, with the bits of mmv followed by moe_combine)
+    hidden = _experts_gemv_hidden(x, gate, up, topk_ids, n_mid)
+    return moe_down_combine(hidden, down, topk_ids, topk_weights.contiguous(), n_experts)
