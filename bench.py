@@ -4,15 +4,19 @@ A step is one fused decode+GEMV over the output projection (248320 x 2048 BF16 w
 activation vector N(0, 1), FP32 accumulation, FP32 output) with the encoded weights resident in HBM.  Two copies of the
 weights at different addresses are used in turn so that the 256 MB last-level cache does not serve the stream.
 Reported: compressed bytes per second (metric), the roofline of the GEMV kernel on algorithmic bytes, the BF16 GEMV of
-the stock BLAS on the uncompressed tensor, and the CPU restatement (oracle) of decode+GEMV on a bounded sample.
+the stock BLAS on the uncompressed tensor, a kernel that only reads as many bytes, the other configurations of the path
+(batch 4, the small 4-bit-code matrices, the MoE decode layer as one HIP graph, the batched MoE prefill, the 40-layer
+decode step next to the same step on uncompressed BF16 weights) and the CPU restatement (oracle) of decode+GEMV on
+bounded samples.  All tensors come from the counter-based generator of orin_qwen_lossless_amd/synth.py.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--rows R] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--rows R] [--no-cpu] [--no-configs] [--suite]
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -21,39 +25,35 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-SETTLE_MS = 40.0  # untimed load before the timed region of the headline kernel (see time_kernel)
-# HBM bytes per GEMV launch from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, each factor calibrated
-# on a copy of known size in the same profiler run), for the workloads that were profiled; not measurable in-process.
-MEASURED_TRAFFIC = {(248320, 2048): 711_400_000}
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+SETTLE_MS = 40.0       # untimed load before the timed region of the headline kernel (see time_blocks)
+MIN_TIMED_MS = 50.0    # the block of `steps` launches is repeated until at least this long has been timed
+TRAFFIC_PROFILE = os.path.join("profiles", "k_w64_mmv_lm_head_248320x2048_hbm_traffic_pmc.txt")
 
 
-def gen_weights(rows: int, K: int, seed: int):
-    """N(0, 0.02) -> BF16 (RNE) on the GPU, returned as a CPU bf16 tensor and kept on the device for the BLAS baseline."""
+def measured_traffic(rows: int, K: int):
+    """HBM bytes per launch of the headline kernel from hardware counters (not measurable in-process): the line
+    `traffic_bytes_per_launch[<rows>x<K>] = N` of the committed counter summary, or None."""
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch\[%dx%d\]\s*=\s*(\d+)" % (rows, K), text)
+    return int(m.group(1)) if m else None
+
+
+def time_kernel(fn, steps: int, warmup: int, settle_ms: float = 0.0):
+    """Per-launch durations (ms) of `steps` calls from HIP events recorded around every call on the launch stream
+    (torch's current stream, which is the one the library launches on), after `warmup` untimed calls and, for
+    settle_ms, further untimed calls: the events are created first, so that nothing idles the GPU between the untimed
+    calls and the timed ones."""
     import torch
 
-    g = torch.Generator(device="cuda").manual_seed(seed)
-    w = torch.empty((rows, K), dtype=torch.bfloat16, device="cuda")
-    step = 1 << 15
-    for r0 in range(0, rows, step):
-        n = min(step, rows - r0)
-        w[r0: r0 + n] = (torch.randn((n, K), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
-    return w
-
-
-def time_kernel(fn, steps: int, warmup: int, graph: bool = False, settle_ms: float = 0.0):
-    """Wall time of `steps` back-to-back launches (synchronised on both sides), then per-launch durations (ms) of a
-    second pass from HIP events recorded around every launch on the launch stream (torch's current stream, which is the
-    one the library launches on).  graph: the `steps` launches of the wall-time pass are captured into one HIP graph
-    first and the timed region is its replay (the launchers only enqueue kernels), which keeps host launch overhead and
-    inter-launch gaps out of the job time."""
-    import torch
-
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for i in range(warmup):
         fn(i)
-    torch.cuda.synchronize()
     if settle_ms > 0:
-        # the first 15 ms of load after idle run up to 15 % slow on this part (clocks settle): keep launching, untimed,
-        # until that long has passed, so that a short timed region measures the same state as a long one
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         i = warmup
         while (time.perf_counter() - t0) * 1e3 < settle_ms:
@@ -61,58 +61,63 @@ def time_kernel(fn, steps: int, warmup: int, graph: bool = False, settle_ms: flo
                 fn(i)
                 i += 1
             torch.cuda.synchronize()
-    if graph:
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            for i in range(steps):
-                fn(i)
-        g.replay()  # untimed: the first replay uploads the graph
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        g.replay()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        del g
-    else:
-        t0 = time.perf_counter()
-        for i in range(steps):
-            fn(i)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i in range(4):
+            fn(i)  # the queue is not empty when the first timed call arrives
     for i in range(steps):
         ev[i][0].record()
         fn(i)
         ev[i][1].record()
     torch.cuda.synchronize()
-    return [a.elapsed_time(b) for a, b in ev], wall
+    return [a.elapsed_time(b) for a, b in ev]
 
 
-def cpu_baseline(wbits, K: int, xf, sample_rows: int):
-    """The oracle's decode+GEMV (reference layout, R = 16) on the first sample_rows rows, all host threads available
-    to this process (capped at 16)."""
+def time_blocks(fn, steps: int, warmup: int, settle_ms: float, min_ms: float):
+    """Wall time of blocks of `steps` back-to-back launches (synchronised on both sides), repeated until min_ms have
+    been timed (three blocks at least); returns the per-block wall times in ms.  The first 15 ms of load after idle
+    run up to 15 % slow on this part (clocks settle): after the warm-up the kernel keeps running, untimed, until
+    settle_ms have passed, so that a short block measures the same state as a long one."""
+    import torch
+
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    i = warmup
+    while (time.perf_counter() - t0) * 1e3 < settle_ms:
+        for _ in range(16):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+    blocks, total = [], 0.0
+    while len(blocks) < 3 or total < min_ms:
+        t0 = time.perf_counter()
+        for j in range(steps):
+            fn(j)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) * 1e3
+        blocks.append(dt)
+        total += dt
+    return blocks
+
+
+def med_us(fn, steps: int = 50, warmup: int = 5) -> float:
     import numpy as np
 
-    from oracle import pyoracle as O
-    from orin_qwen_lossless_amd import ops
+    return float(np.median(time_kernel(fn, steps, warmup))) * 1e3
 
-    threads = max(1, min(16, len(os.sched_getaffinity(0))))
-    sub = np.ascontiguousarray(wbits[:sample_rows])
-    plane, aux, _, _ = ops.encode_bits(sub, 3, 16, False)
-    nbytes = plane.size + aux.size
-    O.decode_gemv(plane, aux, xf, 0, sample_rows, threads)  # warm-up
-    reps, t_total, best = 0, 0.0, None
-    while t_total < 12.0 and reps < 5000:
-        t0 = time.perf_counter()
-        O.decode_gemv(plane, aux, xf, 0, sample_rows, threads)
-        dt = time.perf_counter() - t0
-        t_total += dt
-        reps += 1
-        best = dt if best is None else min(best, dt)
-    med = t_total / reps
-    return {"value": round(nbytes / med / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"first {sample_rows} of the workload's rows ({sample_rows}x{K}, HUFPAIR R=16 reference layout, "
-                      f"{nbytes} compressed bytes), mean of {reps} runs ({med * 1e3:.1f} ms each, best {best * 1e3:.1f} ms)"}
+
+def graph_us(fn, n: int = 16, reps: int = 30) -> float:
+    """Per-call time of a short operation: n calls captured into one HIP graph (alternating weight copies through the
+    call index), the graph replayed `reps` times between HIP events; host launch overhead stays out of the figure."""
+    import torch
+
+    fn(0)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(n):
+            fn(i)
+    return med_us(lambda i: graph.replay(), reps, 3) / n
 
 
 def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: str = "mi355x", matrix_core_order: bool = False):
@@ -134,211 +139,216 @@ def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: s
     return ws, plane.size + aux.size, desc
 
 
-def med_us(fn, steps: int = 50, warmup: int = 5) -> float:
+def read_probe_gbs(ops, nbytes: int) -> dict:
+    """The library's read-only kernel (bf16n_read_probe) over as many bytes as the compressed matrix, two buffers in
+    turn: GB/s per access pattern (median of 30 launches each)."""
+    import torch
+
+    bufs = [torch.randint(0, 255, (nbytes // 1024 * 1024,), dtype=torch.uint8, device="cuda") for _ in range(2)]
+    out = {}
+    for pattern, name in ((0, "wavefront_ranges_nontemporal"), (1, "wavefront_ranges_plain"), (2, "grid_stride_nontemporal"), (3, "grid_stride_plain")):
+        for wpc in (8, 16):
+            t = med_us(lambda i: ops.read_probe(bufs[i & 1], pattern, wpc), 30, 5)
+            out[f"{name}_{wpc}_waves_per_cu"] = round(bufs[0].numel() / t / 1e3, 1)
+    return out
+
+
+# ---------------------------------------------------------------- CPU baseline (the oracle as the thing timed)
+
+def cpu_baseline(wbits, K: int, xf, sample_rows: int, budget_s: float):
+    """The oracle's decode+GEMV (reference layout, R = 16) on the first sample_rows rows of the workload, all host
+    threads available to this process (capped at 16); and the CPU reference configuration, one 2048 x 2048 pair-coded
+    matrix, on one thread and on all."""
     import numpy as np
 
-    d, _ = time_kernel(fn, steps, warmup)
-    return float(np.median(d)) * 1e3
+    from oracle import pyoracle as O
+    from orin_qwen_lossless_amd import ops, synth
+
+    threads = max(1, min(16, len(os.sched_getaffinity(0))))
+
+    def run(plane, aux, x, nrows, nthreads, seconds):
+        O.decode_gemv(plane, aux, x, 0, nrows, nthreads)  # warm-up
+        reps, total, best = 0, 0.0, None
+        while total < seconds and reps < 5000:
+            t0 = time.perf_counter()
+            O.decode_gemv(plane, aux, x, 0, nrows, nthreads)
+            dt = time.perf_counter() - t0
+            total += dt
+            reps += 1
+            best = dt if best is None else min(best, dt)
+        return total / reps, best, reps
+
+    sub = np.ascontiguousarray(wbits[:sample_rows])
+    plane, aux, _, _ = ops.encode_bits(sub, 3, 16, False)
+    nbytes = plane.size + aux.size
+    mean, best, reps = run(plane, aux, xf, sample_rows, threads, budget_s * 0.6)
+    out = {"value": round(nbytes / mean / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+           "sample": f"first {sample_rows} of the workload's rows ({sample_rows}x{K}, HUFPAIR R=16 reference layout, "
+                     f"{nbytes} compressed bytes), mean of {reps} runs ({mean * 1e3:.1f} ms each, best {best * 1e3:.1f} ms)"}
+    # the CPU reference configuration: 2048 x 2048, pair code, reference layout (R = 4, what its policy gives the shape)
+    w1 = synth.weights(2048, 2048, 11)
+    x1 = synth.bf16_bits_to_f32(synth.activations(1, 2048, 12)[0])
+    p1, a1, _, _ = ops.encode_bits(w1, 3, 4, False)
+    assert np.array_equal(O.decode(p1, a1), w1), "round trip of the 2048 x 2048 matrix"
+    b1 = p1.size + a1.size
+    cfg1 = {"workload": "2048x2048 BF16 N(0,0.02), HUFPAIR R=4 reference layout, round trip verified, decode+GEMV FP32",
+            "compressed_bytes": int(b1)}
+    for nt in sorted({1, threads}):
+        m1, best1, r1 = run(p1, a1, x1, 2048, nt, budget_s * 0.2)
+        cfg1[f"threads_{nt}"] = {"us": round(m1 * 1e6, 1), "GBps": round(b1 / m1 / 1e9, 3), "runs": r1}
+    out["config1_2048x2048"] = cfg1
+    return out
 
 
-def graph_us(fn, n: int = 16, reps: int = 30) -> float:
-    """Per-call time of a short operation: n calls captured into one HIP graph (alternating weight copies through the
-    call index), the graph replayed `reps` times between HIP events; host launch overhead stays out of the figure."""
+# ---------------------------------------------------------------- the other configurations of the path
+
+def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4), n_layers: int = 40, n_sets: int = 4) -> dict:
+    """The 40-layer decode step as one HIP graph on BF16N weights and on uncompressed BF16 weights with stock kernels
+    (orin_qwen_lossless_amd/decode_step.py), output projection included.  n_sets distinct weight sets are used in turn;
+    every layer's input is the previous layer's output, so layers that share a set route to other experts."""
     import numpy as np
     import torch
 
-    fn(0)
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        for i in range(n):
-            fn(i)
-    d, _ = time_kernel(lambda i: graph.replay(), reps, 3)
-    return float(np.median(d)) * 1e3 / n
+    from orin_qwen_lossless_amd import decode_step as D, synth
 
-
-def decode_step(ops, head, randw, randx, K: int, n_layers: int = 40, n_sets: int = 4, head_tiles=None) -> dict:
-    """One decode step of the 35B-A3B shape as a single HIP graph: n_layers x (qkv 5120 x K, o K x 4096, router, top-8 of
-    256 experts, fused gate/up, down, combine, shared expert) + the output projection.  n_sets distinct weight sets are
-    used in turn and every layer's input is the previous layer's output (re-normalised), so that layers sharing a
-    weight set route to different experts; attention itself is not part of this path."""
-    import numpy as np
-    import torch
-
-    E, topk, N = 256, 8, 512
-    sets, nbytes = [], {}
-    for _ in range(n_sets):
-        d = {}
-        for name, (rows, k, nm) in {"qkv": (5120, K, 1), "o": (K, 4096, 1), "router": (E, K, 1), "gate": (E * N, K, E),
-                                    "up": (E * N, K, E), "down": (E * K, N, E), "sh_gate_up": (2 * N, K, 1),
-                                    "sh_down": (K, N, 1)}.items():
-            ws, nb, _ = encode_to_device(ops, randw(rows, k), n_matrices=nm)
-            d[name] = ws[0]
-            nbytes[name] = nb
-        sets.append(d)
-    touched = n_layers * (nbytes["qkv"] + nbytes["o"] + nbytes["router"] + nbytes["sh_gate_up"] + nbytes["sh_down"]
-                          + (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * topk // E)
-    res = {"layers": n_layers, "weight_sets": n_sets}
-    for T, hd, tag in ((1, head, ""), (4, head, ""), (16, head, ""), (16, head_tiles, "_head_as_tiles")):
-        if hd is None:
-            continue
-        xin = [randx(T, K) for _ in range(4)]
-        xbuf = xin[0].clone()
-
-        def step():
-            # the glue between the products is two residual adds and two norms per layer (without the norms the SwiGLU
-            # squares the activations layer after layer); the engine's attention is outside this path
-            h = xbuf
-            for layer in range(n_layers):
-                w = sets[layer % n_sets]
-                q = ops.linear(h, w["qkv"])
-                h = torch.nn.functional.rms_norm(h + ops.linear(q[:, :4096], w["o"]), (K,))
-                wts, ids = ops.router_topk(ops.mmv(h, w["router"]), topk)
-                y = ops.moe_experts(h, w["gate"], w["up"], w["down"], wts, ids, E)
-                sh = ops.mmv(ops.mmv_glu(h, w["sh_gate_up"]), w["sh_down"], out_dtype=torch.bfloat16)
-                h = torch.nn.functional.rms_norm(h + y + sh, (K,))
-            return ops.linear(h, hd)
-
-        step()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
-
-        def replay(i):
-            xbuf.copy_(xin[i & 3])
+    sets, raw, nbytes = D.make_layer_sets(ops, gen, n_sets, True)
+    head_bytes = head.plane.numel() + head.aux.numel()
+    res = {"layers": n_layers, "weight_sets": n_sets, "launches_per_layer": 8,
+           "bf16_comparator": "the same graph on uncompressed BF16 weights: torch linear / bmm (hipBLASLt) for every product, the "
+                              "experts a token selects gathered by index_select (the routing is decided on the device), "
+                              "the same glue and top-k launches"}
+    for T in batches:
+        xin = [synth.activations_torch(T, K, 300 + i, "cuda") for i in range(4)]
+        hbuf = xin[0].clone()
+        entry = {}
+        for name, step in (("bf16n", D.Bf16nStep(ops, sets, head, n_layers, T)), ("bf16", D.Bf16Step(ops, raw, head_bf16, n_layers, T))):
+            graph, out = D.capture(step, hbuf)
+            eager = step(hbuf).clone()
             graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), "graph replay differs from the eager step"
 
-        d, _ = time_kernel(replay, 12, 3)
-        t = float(np.median(d)) * 1e3
-        # experts touched: at most T * top-k distinct ones per layer
-        tb = touched + (n_layers * (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * topk // E) * (min(T, E // topk) - 1) + hd.plane.numel() + hd.aux.numel()
-        res[f"batch{T}{tag}"] = {"graph_us": round(t, 1), "compressed_bytes_touched_upper_bound": int(tb),
-                            "GBps": round(tb / t / 1e3, 1), "tokens_per_s": round(T / t * 1e6, 1)}
-        del graph
+            def replay(i):
+                hbuf.copy_(xin[i & 3])
+                graph.replay()
+
+            entry[name] = float(np.median(time_kernel(replay, 12, 3))) * 1e3
+            del graph
+        touched = n_layers * D.layer_bytes(nbytes, T) + head_bytes
+        bf16_bytes = 2 * (n_layers * (sum(r * k for n_, (r, k, m) in D.SHAPES.items() if m == 1)
+                                      + (min(T * D.TOPK, D.E) + 1) * 3 * D.N_MID * K) + head_bf16.numel())
+        t = entry["bf16n"]
+        res[f"batch{T}"] = {"us": round(t, 1), "compressed_bytes_touched_upper_bound": int(touched), "GBps": round(touched / t / 1e3, 1),
+                            "frac_of_hbm_peak": round(touched / t / 1e3 / HBM_PEAK_GBS, 4), "tokens_per_s": round(T / t * 1e6, 1),
+                            "bf16_us": round(entry["bf16"], 1), "speedup_vs_bf16": round(entry["bf16"] / t, 2),
+                            "bf16_bytes_touched": int(bf16_bytes), "bf16_us_at_hbm_peak": round(bf16_bytes / HBM_PEAK_GBS / 1e3, 1),
+                            "eager_equals_graph": True}
+    res["layer_sets"] = sets
+    res["nbytes"] = nbytes
     return res
 
 
-def suite(ops, w_head, head_copies, x1, K: int) -> dict:
-    """The other configurations of the path, each timed with HIP events (median of 50 launches): batch 4 on the output
-    projection, the small NIBBLE matrices, one MoE layer at batch 1 as a captured HIP graph, and the batched prefill."""
+def configs(ops, w_head, head_copies, comp_bytes: int, K: int) -> dict:
+    """The other configurations, compact: batch 4 on the output projection, the two small matrices, the MoE decode
+    layer as one HIP graph, the batched prefill at 2048 and 8192 tokens, the 40-layer decode step at batch 1 and 4."""
     import numpy as np
     import torch
 
+    from orin_qwen_lossless_amd import decode_step as D, synth
+
     out = {}
-    g = torch.Generator(device="cuda").manual_seed(3)
+    seed = [1000]
 
-    def randw(rows, k):
-        return (torch.randn((rows, k), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    def gen(rows, k):
+        seed[0] += 1
+        return synth.weights_torch(rows, k, seed[0], "cuda")
 
-    def randx(*shape):
-        return torch.randn(shape, generator=g, device="cuda").to(torch.bfloat16)
+    rows = w_head.shape[0]
+    x4 = synth.activations_torch(4, K, 21, "cuda")
+    t4 = med_us(lambda i: ops.mmv(x4, head_copies[i & 1]), 30, 5)
+    algo4 = comp_bytes + 4 * K * 2 + 4 * rows * 4
+    out["lm_head_batch4"] = {"us": round(t4, 2), "GBps": round(algo4 / t4 / 1e3, 1), "frac_of_hbm_peak": round(algo4 / t4 / 1e3 / HBM_PEAK_GBS, 4)}
+    for r, k in ((512, 2048), (2048, 512)):
+        ws, nb, desc = encode_to_device(ops, gen(r, k), copies=2)
+        xx = synth.activations_torch(1, k, 22, "cuda")
+        t = graph_us(lambda i: ops.mmv(xx, ws[i & 1]))
+        out[f"gemv_{r}x{k}"] = {"layout": desc, "us": round(t, 2), "GBps": round(nb / t / 1e3, 1), "timing": "16 launches per HIP graph replay"}
+    # decode step (builds the layer sets that the MoE layer and the prefill configurations reuse)
+    step = decode_step_config(ops, gen, head_copies[0], w_head, K)
+    sets, nbytes = step.pop("layer_sets"), step.pop("nbytes")
+    out["decode_step"] = step
+    # MoE decode layer, batch 1: router GEMV, top-8 on the device, 8 routed + the shared expert, weighted sum + norm
+    st = D.Bf16nStep(ops, sets, None, 1, 1)
+    xs = [synth.activations_torch(1, K, 400 + i, "cuda") for i in range(8)]
+    xbuf, hres = xs[0].clone(), synth.activations_torch(1, K, 399, "cuda")
+    layer_i = [0]
 
-    # batch 4 on the output projection (one decode shared by the four columns)
-    x4 = randx(4, K)
-    t4 = med_us(lambda i: ops.mmv(x4, head_copies[i & 1]))
-    out["lm_head_batch4_us"] = round(t4, 2)
-    # the output projection at other batch sizes: groups of up to eight columns per decode in the layout above, then
-    # dequant + a stock GEMM; and the same matrix as 32 x 256 tiles (the policy's matrix-core order for dense matrices),
-    # where BF16 activations go through the matrix cores at any batch size
+    def moe_layer():
+        ys, wts, ids = st.experts(sets[layer_i[0] % len(sets)], xbuf)
+        return ops.add_rmsnorm(hres, ys=ys, topk_weights=wts)
+
+    graph, _ = D.capture(moe_layer)
+
+    def replay(i):
+        xbuf.copy_(xs[i & 7])  # other tokens pick other experts: the routed experts are not cache-resident
+        graph.replay()
+
+    t_layer = med_us(replay, 64, 8)
+    touched = nbytes["router"] + (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * (D.TOPK + 1) // D.EA
+    out["moe_layer_batch1_graph"] = {"us": round(t_layer, 2), "launches": 5, "compressed_bytes_touched": int(touched),
+                                     "GBps": round(touched / t_layer / 1e3, 1), "frac_of_hbm_peak": round(touched / t_layer / 1e3 / HBM_PEAK_GBS, 4),
+                                     "experts": "256 routed (top-8, softmax weights renormalised) + 1 shared, 32x256 tiles"}
+    del graph
+    # batched prefill: routing lists, fused gate/up + SwiGLU (BF16 out), down; experts as in the decode step
+    w = sets[0]
+    for T in (2048, 8192):
+        xp = synth.activations_torch(T, K, 500 + T, "cuda")
+        _, ids = ops.router_topk(synth.normal_torch(T * D.E, 600 + T, "cuda").view(T, D.E), D.TOPK)
+
+        def prefill(i):
+            src1, dst, bounds = ops.mm_ids_route(ids, D.EA, False)
+            a = ops.moe_mm_ids(xp, ids, w["gate"], D.EA, up=w["up"], out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
+            return ops.moe_mm_ids(a, ids, w["down"], D.EA, routes=(dst, dst, bounds))
+
+        t = med_us(prefill, 10, 2)
+        flops = 2.0 * T * D.TOPK * 3 * D.N_MID * K
+        wbytes = (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * D.E // D.EA
+        out[f"moe_prefill_T{T}"] = {"us": round(t, 1), "TFLOPs": round(flops / t / 1e6, 1),
+                                    "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                    "weight_decode_GBps": round(wbytes / t / 1e3, 1), "tokens_per_s": round(T / t * 1e6, 0)}
+    return out
+
+
+def suite(ops, w_head, head_copies, K: int) -> dict:
+    """A wider sweep, on request: the output projection at other batch sizes in both of its layouts."""
+    from orin_qwen_lossless_amd import synth
+
     batches = {}
     tiles, tbytes, tdesc = encode_to_device(ops, w_head, copies=2, matrix_core_order=True)
     for T in (1, 2, 4, 8, 16, 32, 128):
-        xT = randx(T, K)
+        xT = synth.activations_torch(T, K, 700 + T, "cuda")
         base = graph_us(lambda i: ops.mmv(xT, head_copies[i & 1]), 4, 10) if T <= 8 else med_us(lambda i: ops.linear(xT, head_copies[i & 1]), 10, 2)
         batches[str(T)] = {"units_of_16_rows_us": round(base, 1), "path": "gemv" if T <= 8 else "dequant + BF16 GEMM",
                            "tiles_us": round(graph_us(lambda i: ops.mmv(xT, tiles[i & 1]), 4, 10), 1)}
-    out["lm_head_batches"] = {"tiles": tdesc, "tiles_bytes": tbytes, "by_batch": batches}
-    head_tiles = tiles[0]
-    del tiles
-    # small NIBBLE matrices
-    for rows, k in ((512, 2048), (2048, 512)):
-        ws, nbytes, desc = encode_to_device(ops, randw(rows, k), copies=2)
-        xx = randx(1, k)
-        t = graph_us(lambda i: ops.mmv(xx, ws[i & 1]))
-        out[f"gemv_{rows}x{k}"] = {"layout": desc, "us": round(t, 2), "GBps": round(nbytes / t / 1e3, 1),
-                                   "timing": "16 launches per HIP graph replay"}
-    # one MoE layer of the 35B-A3B shape: router 256x2048, 256 experts x (gate 512x2048, up 512x2048, down 2048x512),
-    # top-8 of 256 computed on the device (softmax, renormalised top-k weights)
-    E, topk, N = 256, 8, 512
-    router, rb, rdesc = encode_to_device(ops, randw(E, K))
-    wg, wu = randw(E * N, K), randw(E * N, K)
-    down, db, ddesc = encode_to_device(ops, randw(E * K, N), n_matrices=E)
-    router, down = router[0], down[0]
-    xs = [randx(1, K) for _ in range(8)]
-    xbuf = xs[0].clone()
-    pairs = {}
-    for engine in ("mi355x", "llama"):  # gate / up: this build's wave64 units, and the reference's chunk-major units
-        gate, gb, gdesc = encode_to_device(ops, wg, n_matrices=E, engine=engine)
-        up, ub, _ = encode_to_device(ops, wu, n_matrices=E, engine=engine)
-        gate, up = gate[0], up[0]
-        pairs[engine] = (gate, up, gdesc)
-
-        def layer():
-            wts, ids = ops.router_topk(ops.mmv(xbuf, router), topk)
-            return ops.moe_experts(xbuf, gate, up, down, wts, ids, E)
-
-        layer()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            layer()
-
-        def replay(i):
-            xbuf.copy_(xs[i & 7])  # other tokens pick other experts: the 8 routed experts are not cache-resident
-            graph.replay()
-
-        t_layer = med_us(replay, 64, 8)
-        touched = rb + (gb + ub + db) * topk // E
-        out[f"moe_layer_batch1_gate_up_{engine}"] = {
-            "layouts": {"router": rdesc, "gate_up": gdesc, "down": ddesc}, "graph_us": round(t_layer, 2),
-            "compressed_bytes_touched": int(touched), "GBps": round(touched / t_layer / 1e3, 1),
-            "routing": "softmax over 256 logits, top-8 (ties: lower index), weights renormalised to sum 1"}
-        del graph
-    # prefill: fused gate/up + SwiGLU (BF16 out), then down, over routing lists computed on the device
-    for T in (2048, 8192):
-        xp = randx(T, K)
-        lg = torch.randn((T, E), generator=g, device="cuda")
-        wts, ids = ops.router_topk(lg, topk)
-        for engine, (gate, up, gdesc) in pairs.items():
-
-            def prefill(i):  # as ops.moe_experts does it: one routing pass, fused gate/up + SwiGLU (BF16), down
-                src1, dst, bounds = ops.mm_ids_route(ids, E, False)
-                a = ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
-                return ops.moe_mm_ids(a, ids, down, E, routes=(dst, dst, bounds))
-
-            t = med_us(prefill, 10, 2)
-            t_gu = med_us(lambda i: ops.moe_mm_ids(xp, ids, gate, E, up=up, out_dtype=torch.bfloat16), 10, 2)
-            flops = 2.0 * T * topk * (2 * N * K + K * N)
-            out[f"moe_prefill_T{T}_gate_up_{engine}"] = {
-                "gate_up": gdesc, "us": round(t, 1), "gate_up_us": round(t_gu, 1), "TFLOPs": round(flops / t / 1e6, 2),
-                "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / 2500.0, 4), "tokens_per_s": round(T / t * 1e6, 0)}
-    out["decode_step"] = decode_step(ops, head_copies[0], randw, randx, K, head_tiles=head_tiles)
-    return out
+    return {"lm_head_batches": {"tiles": tdesc, "tiles_bytes": tbytes, "by_batch": batches}}
 
 
 def prefill_only(T: int, steps: int) -> None:
     """Only the batched MoE kernels of one 35B-A3B-shaped layer (256 experts x (gate, up 512 x 2048; down 2048 x 512),
     top-8, experts in the mi355x policy's layout) on T tokens: routing lists once, then fused gate/up + SwiGLU (BF16)
     and down, `steps` times.  For profiling these kernels alone; prints its own JSON line."""
-    import numpy as np
     import torch
 
-    from orin_qwen_lossless_amd import ops
+    from orin_qwen_lossless_amd import ops, synth
 
     torch.cuda.set_device(0)
     ops.init()
     E, topk, N, K = 256, 8, 512, 2048
-    g = torch.Generator(device="cuda").manual_seed(3)
-
-    def randw(rows, k):
-        return (torch.randn((rows, k), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
-
-    (gate,), _, gdesc = encode_to_device(ops, randw(E * N, K), n_matrices=E)
-    (up,), _, _ = encode_to_device(ops, randw(E * N, K), n_matrices=E)
-    (down,), _, ddesc = encode_to_device(ops, randw(E * K, N), n_matrices=E)
-    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
-    _, ids = ops.router_topk(torch.randn((T, E), generator=g, device="cuda"), topk)
+    (gate,), gb, gdesc = encode_to_device(ops, synth.weights_torch(E * N, K, 31, "cuda"), n_matrices=E)
+    (up,), ub, _ = encode_to_device(ops, synth.weights_torch(E * N, K, 32, "cuda"), n_matrices=E)
+    (down,), db, ddesc = encode_to_device(ops, synth.weights_torch(E * K, N, 33, "cuda"), n_matrices=E)
+    x = synth.activations_torch(T, K, 34, "cuda")
+    _, ids = ops.router_topk(synth.normal_torch(T * E, 35, "cuda").view(T, E), topk)
     src1, dst, bounds = ops.mm_ids_route(ids, E, False)
 
     def gate_up(i):
@@ -349,32 +359,42 @@ def prefill_only(T: int, steps: int) -> None:
     t_dn = med_us(lambda i: ops.moe_mm_ids(a, ids, down, E, routes=(dst, dst, bounds)), steps, 2)
     flops_gu, flops_dn = 2.0 * T * topk * 2 * N * K, 2.0 * T * topk * K * N
     print(json.dumps({"workload": f"MoE prefill, {T} tokens, top-{topk} of {E} experts", "gate_up": gdesc, "down": ddesc,
-                      "gate_up_us": round(t_gu, 1), "down_us": round(t_dn, 1),
+                      "gate_up_us": round(t_gu, 1), "down_us": round(t_dn, 1), "gate_up_bytes": gb + ub, "down_bytes": db,
                       "gate_up_TFLOPs": round(flops_gu / t_gu / 1e6, 1), "down_TFLOPs": round(flops_dn / t_dn / 1e6, 1),
-                      "frac_of_bf16_mfma_peak": round((flops_gu + flops_dn) / (t_gu + t_dn) / 1e6 / 2500.0, 4)}))
+                      "frac_of_bf16_mfma_peak": round((flops_gu + flops_dn) / (t_gu + t_dn) / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}))
 
 
-def head_tiles_only(T: int, steps: int, rows: int, K: int) -> None:
-    """Only the output projection in the policy's matrix-core order (32 x 256 tiles) at batch T: bf16n_mmv with BF16
-    activations, which runs on the matrix cores, `steps` times on two alternated copies.  For profiling this kernel
-    alone; prints its own JSON line."""
+def decode_only(T: int, steps: int) -> None:
+    """Only the 40-layer decode step on BF16N weights at batch T, `steps` graph replays (for profiling); prints its own
+    JSON line."""
+    import numpy as np
     import torch
 
-    from orin_qwen_lossless_amd import ops
+    from orin_qwen_lossless_amd import decode_step as D, ops, synth
 
     torch.cuda.set_device(0)
     ops.init()
-    w = gen_weights(rows, K, 1)
-    tiles, nbytes, desc = encode_to_device(ops, w, copies=2, matrix_core_order=True)
-    g = torch.Generator(device="cuda").manual_seed(2)
-    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
-    y = ops.mmv(x, tiles[0])
-    err = float(((y.double() - x.double() @ w.double().t()).abs() / (x.double().abs() @ w.double().abs().t())).max())
-    t = med_us(lambda i: ops.mmv(x, tiles[i & 1]), steps, 5)
-    algo = nbytes + T * K * 2 + T * rows * 4
-    print(json.dumps({"workload": f"output projection {rows}x{K}, {desc}, batch {T} BF16 activations, FP32 out", "us": round(t, 2),
-                      "compressed_bytes": nbytes, "algorithmic_bytes": algo, "GBps": round(algo / t / 1e3, 1),
-                      "frac_of_hbm_peak": round(algo / t / 1e3 / HBM_PEAK_GBS, 4), "max_err_over_sum_abs": err}))
+    K = D.K_MODEL
+    seed = [2000]
+
+    def gen(rows, k):
+        seed[0] += 1
+        return synth.weights_torch(rows, k, seed[0], "cuda")
+
+    sets, _, nbytes = D.make_layer_sets(ops, gen, 4, False)
+    (head,), hb, _ = encode_to_device(ops, gen(248320, K))
+    xin = [synth.activations_torch(T, K, 300 + i, "cuda") for i in range(4)]
+    hbuf = xin[0].clone()
+    graph, _ = D.capture(D.Bf16nStep(ops, sets, head, 40, T), hbuf)
+
+    def replay(i):
+        hbuf.copy_(xin[i & 3])
+        graph.replay()
+
+    t = float(np.median(time_kernel(replay, steps, 3))) * 1e3
+    touched = 40 * D.layer_bytes(nbytes, T) + hb
+    print(json.dumps({"workload": f"40-layer decode step + output projection, batch {T}, one HIP graph", "us": round(t, 1),
+                      "compressed_bytes_touched_upper_bound": int(touched), "GBps": round(touched / t / 1e3, 1)}))
 
 
 def main() -> None:
@@ -386,34 +406,34 @@ def main() -> None:
     ap.add_argument("--K", type=int, default=2048)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=16384)
-    ap.add_argument("--graph", action="store_true", help="time the steps as one HIP graph replay instead of separate launches")
-    ap.add_argument("--suite", action="store_true", help="also time batch 4, the NIBBLE matrices, a MoE layer and the prefill")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU work of the baseline leg, about")
+    ap.add_argument("--no-configs", action="store_true", help="only the headline kernel: skip the other configurations")
+    ap.add_argument("--suite", action="store_true", help="also sweep the output projection over batch sizes in both layouts")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="run only the batched MoE kernels of one layer on T tokens (for profiling) and exit")
-    ap.add_argument("--head-tiles", type=int, default=0, metavar="T",
-                    help="run only the output projection as 32 x 256 tiles at batch T (for profiling) and exit")
+    ap.add_argument("--decode-step", type=int, default=0, metavar="T",
+                    help="run only the 40-layer decode step at batch T (for profiling) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path has no collective); run with --gpus 1")
     if args.prefill > 0:
         prefill_only(args.prefill, min(args.steps, 20))
         return
-    if args.head_tiles > 0:
-        head_tiles_only(args.head_tiles, min(args.steps, 50), args.rows, args.K)
+    if args.decode_step > 0:
+        decode_only(args.decode_step, min(args.steps, 20))
         return
 
     import numpy as np
     import torch
 
-    from orin_qwen_lossless_amd import ops
+    from orin_qwen_lossless_amd import ops, synth
 
     torch.cuda.set_device(0)
     ops.init()
     rows, K = args.rows, args.K
     t0 = time.perf_counter()
-    w_dev = gen_weights(rows, K, seed=1)
-    w_cpu = w_dev.cpu()
-    wbits = w_cpu.view(torch.int16).numpy().view(np.uint16)
+    w_dev = synth.weights_torch(rows, K, 1, "cuda")
+    wbits = w_dev.cpu().view(torch.int16).numpy().view(np.uint16)
     fmt, R, cm, _, w64 = ops.choose(rows, K, engine="mi355x")
     t1 = time.perf_counter()
     plane, aux, fmt_out, _ = ops.encode_bits(wbits, fmt, R, cm, wave64=w64)
@@ -422,8 +442,7 @@ def main() -> None:
     meta = ops.parse_header(ta)
     copies = [ops.upload(torch.from_numpy(plane), ta, meta, "cuda") for _ in range(2)]
     assert ops.roundtrip_equal(copies[0], w_dev), "GPU decode is not bit-exact"  # the load-time verify, before timing
-    g = torch.Generator(device="cuda").manual_seed(2)
-    x = torch.randn((1, K), generator=g, device="cuda").to(torch.bfloat16)
+    x = synth.activations_torch(1, K, 2, "cuda")
     y = ops.mmv(x, copies[0])
     ref = (w_dev.float() @ x[0].float())
     err = float(((y[0] - ref).abs() / (w_dev.float().abs() @ x[0].float().abs())).max())
@@ -431,24 +450,19 @@ def main() -> None:
 
     comp_bytes = plane.size + aux.size
     algo_bytes = comp_bytes + K * 2 + rows * 4  # weights (plane + aux incl. table, unit bases, padding) + x + y
-    # the steps are launched one by one: at 135 us per step the launches keep ahead of the GPU, and a HIP graph replay of
-    # the same steps measured slower (138 us per step at 200 steps, a fixed cost of about half a millisecond per replay)
-    use_graph = args.graph
-    durs, wall = time_kernel(lambda i: ops.mmv(x, copies[i & 1]), args.steps, args.warmup, graph=use_graph, settle_ms=SETTLE_MS)
-    ms = wall * 1e3 / args.steps
+    step = lambda i: ops.mmv(x, copies[i & 1])  # noqa: E731
+    blocks = time_blocks(step, args.steps, args.warmup, SETTLE_MS, MIN_TIMED_MS)
+    ms = float(np.median(blocks)) / args.steps
+    durs = time_kernel(step, args.steps, args.warmup, SETTLE_MS)
     kern_ms = float(np.mean(durs))
-    # stock BF16 GEMV on the uncompressed tensor (the "vs BF16" column), same timing loop
+    # stock BF16 GEMV on the uncompressed tensor (the "vs BF16" column), same timing
     w2 = [w_dev, w_dev.clone()]
     xt = x[0].contiguous()
-    bd, _ = time_kernel(lambda i: torch.mv(w2[i & 1], xt), min(args.steps, 100), 10)
-    blas_us = float(np.median(bd)) * 1e3
-    # a plain streaming read of as many bytes as the compressed matrix (stock reduction over an FP64 view, two
-    # buffers alternated): what the memory system gives a kernel that does nothing but read
-    nread = comp_bytes // 8 * 8
-    bufs = [torch.randint(0, 255, (nread,), dtype=torch.uint8, device="cuda") for _ in range(2)]
-    sd, _ = time_kernel(lambda i: bufs[i & 1].view(torch.float64).sum(), 30, 5)
-    stream_gbs = nread / (float(np.median(sd)) * 1e-3) / 1e9
-    del bufs
+    blas_us = med_us(lambda i: torch.mv(w2[i & 1], xt), min(args.steps, 100), 10)
+    del w2
+    probe = read_probe_gbs(ops, comp_bytes)
+    stream_gbs = max(probe.values())
+    traffic = measured_traffic(rows, K)
 
     out = {
         "metric": "fused decode+GEMV HBM GB/s (% peak, compressed bytes); us/decode step vs BF16",
@@ -458,27 +472,31 @@ def main() -> None:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"output projection {rows}x{K} BF16 N(0,0.02), {ops.FORMAT_NAMES[fmt_out]} R={R} "
                                f"{'wave64' if w64 else 'reference'} layout, fused decode+GEMV, batch 1 BF16 activations "
-                               "N(0,1), FP32 accumulate/out; 2 weight copies alternated; the timed steps are "
-                               + ("one HIP graph replay" if use_graph else "separate launches")
-                               + f"; after the {args.warmup} warm-up steps the kernel keeps running untimed until {SETTLE_MS:.0f} ms have passed (clocks settle)",
+                               "N(0,1), FP32 accumulate/out; 2 weight copies alternated; the timed steps are separate launches, "
+                               f"in blocks of {args.steps} repeated until {MIN_TIMED_MS:.0f} ms are timed (median block of {len(blocks)}); "
+                               f"after the {args.warmup} warm-up steps the kernel keeps running untimed until {SETTLE_MS:.0f} ms have passed (clocks settle)",
                    "rows": rows, "K": K, "batch": 1, "compressed_bytes": comp_bytes, "bits_per_weight": round(8 * comp_bytes / (rows * K), 4),
-                   "ratio_of_bf16": round(comp_bytes / (2 * rows * K), 4)},
+                   "ratio_of_bf16": round(comp_bytes / (2 * rows * K), 4), "generator": "synth.py: splitmix64 counters + Box-Muller, seeds 1 (weights) and 2 (activations)"},
         "roofline": {"bound": "hbm", "achieved": round(algo_bytes / (kern_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((rows, K)),
+                     "traffic": traffic, "traffic_source": TRAFFIC_PROFILE if traffic is not None else None,
                      "kernel": "k_w64_mmv<bf16_t, 4, 1, 2>", "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 2),
                      "median_launch_us": round(float(np.median(durs)) * 1e3, 2)},
         "extra": {"pct_of_hbm_peak_compressed": round(100 * comp_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
-                  "us_per_matrix": round(ms * 1e3, 2), "blas_bf16_gemv_us": round(blas_us, 2),
-                  "speedup_vs_blas_bf16": round(blas_us / (ms * 1e3), 3),
-                  "plain_stream_read_GBps": round(stream_gbs, 1), "kernel_vs_plain_stream_read": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / stream_gbs, 3), "tokens_per_s_lm_head_only": round(1e3 / ms, 1),
-                  "host_encode_s": round(t_enc, 2), "max_err_over_sum_abs": err, "setup_s": round(time.perf_counter() - t0, 1)},
+                  "us_per_matrix": round(ms * 1e3, 2), "block_us_per_step_min_max": [round(min(blocks) / args.steps * 1e3, 2), round(max(blocks) / args.steps * 1e3, 2)],
+                  "blas_bf16_gemv_us": round(blas_us, 2), "speedup_vs_blas_bf16": round(blas_us / (ms * 1e3), 3),
+                  "plain_stream_read_GBps": round(stream_gbs, 1), "read_probe_GBps": probe,
+                  "kernel_vs_plain_stream_read": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / stream_gbs, 3), "tokens_per_s_lm_head_only": round(1e3 / ms, 1),
+                  "host_encode_s": round(t_enc, 2), "max_err_over_sum_abs": err},
     }
+    if not args.no_configs:
+        out["extra"]["configs"] = configs(ops, w_dev, copies, comp_bytes, K)
     if args.suite:
-        out["extra"]["suite"] = suite(ops, w_dev, copies, x, K)
+        out["extra"]["suite"] = suite(ops, w_dev, copies, K)
+    out["extra"]["gpu_s"] = round(time.perf_counter() - t0, 1)
     if not args.no_cpu:
         xf = x[0].float().cpu().numpy()
-        out["cpu_baseline"] = cpu_baseline(wbits, K, xf, min(args.cpu_rows, rows // 16 * 16))
+        out["cpu_baseline"] = cpu_baseline(wbits, K, xf, min(args.cpu_rows, rows // 16 * 16), args.cpu_seconds)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -104,18 +104,13 @@ int bf16n_moe_mm_ids_static(const bf16n_weight * w, const bf16n_weight * up, con
 int bf16n_moe_combine(const float * ys, const void * w, int w_bf16, void * y, int y_bf16, int n_tok, int n_used,
                       int64_t n, void * stream);                                                /* launch.h:82-83, launch.cu:562-572 */
 int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * stream);       /* launch.h:85, launch.cu:574-582 */
-/* mmv with expert ids (launch.h:52) + moe_combine (launch.h:82-83) as one call with the bits of the two: a = the routed
- * product's arguments (x: one activation row per (token, slot); ids; ncols = n_tok * n_used; y unused), wts: n_tok x
- * n_used routing weights, y: n_tok x nrows.  add0 / add1: optional n_tok x nrows BF16 vectors (a shared expert's output,
- * the residual) added in FP32 before the rounding to y.  Tile-layout matrices with at most 16 slots run as one launch;
- * other layouts run the two launches and need ys_workspace (n_tok * n_used * nrows floats; may be null otherwise). */
-int bf16n_moe_down_combine(const bf16n_weight * w, const bf16n_mmv_args * a, const void * wts, int wts_bf16, const void * add0,
-                           const void * add1, void * y, int y_bf16, int n_tok, float * ys_workspace, void * stream);
-/* Engine glue of a decode step in one launch (the reference leaves it to the engines): per token, sum = a + b + c in FP32
- * (BF16 inputs of n elements; b, c may be null), y_sum = bf16(sum) if non-null, y_norm = bf16(sum * rsqrt(mean(sum^2) +
- * eps) * gamma) (gamma: n BF16 values or null). */
-int bf16n_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const uint16_t * gamma, uint16_t * y_sum,
-                      uint16_t * y_norm, int n_tok, int64_t n, float eps, void * stream);
+/* Engine glue of a decode step in one launch (the reference leaves it to the engines): per token, in FP32,
+ *   sum = a + b + c + sum_k wts[k] * ys[k]     (BF16 rows a, b, c of n elements; FP32 rows ys of n_used slots, combined
+ *                                                by bf16n_moe_combine's fmaf chain; every addend but a may be null)
+ *   y_sum = bf16(sum) if non-null;  y_norm = bf16(sum * rsqrt(mean(sum^2) + eps) * gamma)  (gamma: n BF16 values or null) */
+int bf16n_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const float * ys, const void * wts, int wts_bf16,
+                      int n_used, const uint16_t * gamma, uint16_t * y_sum, uint16_t * y_norm, int n_tok, int64_t n, float eps,
+                      void * stream);
 
 /* Router softmax + top-k on the device, so that a whole MoE decode step can be captured into one HIP graph.  The
  * reference leaves this to the engines (vllm_bf16n/moe.py:62-67 receives topk_weights/topk_ids); it has no core
@@ -123,6 +118,10 @@ int bf16n_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c
  * softmax probabilities of the k largest logits (ties: lower index), renormalised to sum 1 when renorm != 0. */
 int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
                       int32_t * ids, float * weights, void * stream);
+/* the same into rows of out_stride >= k elements: a caller that always runs further experts beside the routed ones (a
+ * shared expert stacked behind them) keeps their ids and weights in the columns from k on */
+int bf16n_router_topk_strided(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
+                              int32_t * ids, float * weights, int64_t out_stride, void * stream);
 
 /* Read-bandwidth probe (the reference's bench/micro/bwprobe.cu:23-60 as a library call): a kernel that only reads
  * `bytes` (rounded down to whole KiB) from src, for the memory rate this GPU gives a pure streaming read.  pattern 0:

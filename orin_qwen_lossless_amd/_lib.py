@@ -51,10 +51,10 @@ SYMBOLS = {
     "bf16n_mm_ids": (_i, [_WP, _WP, _vp, _i64, _vp, _vp, _vp, _vp, _i, _i64, _i, _i, _i, _vp]),
     "bf16n_moe_mm_ids_static": (_i, [_WP, _WP, _vp, _i64, _vp, _i, _i64, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     "bf16n_moe_combine": (_i, [_vp, _vp, _i, _vp, _i, _i, _i, _i64, _vp]),
-    "bf16n_moe_down_combine": (_i, [_WP, _AP, _vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp]),
-    "bf16n_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, C.c_float, _vp]),
+    "bf16n_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i64, C.c_float, _vp]),
     "bf16n_swiglu": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "bf16n_router_topk": (_i, [_vp, _i64, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "bf16n_router_topk_strided": (_i, [_vp, _i64, _i, _i, _i, _i, _vp, _vp, _i64, _vp]),
     "bf16n_read_probe": (_i, [_vp, C.c_uint64, _i, _i, _vp, _vp]),
     "bf16n_adapter_choose": (_i, [_i64, _i64, _i64, _cp, _i64, _i, _i]),
     "bf16n_adapter_convert": (_i, [_vp, _vp, _i64, _i64, _i64, _i, _i, _i, _vp, _cp, _i, C.POINTER(_i)]),

@@ -475,51 +475,19 @@ int bf16n_moe_combine(const float * ys, const void * w, int w_bf16, void * y, in
     });
 }
 
-// The routed down product and the weighted sum over a token's experts as one call: bf16n_mmv with expert ids into
-// per-slot FP32 rows followed by bf16n_moe_combine (launch.cu:313-325 and :562-572), with the same bits.  Tile-layout
-// matrices with at most sixteen slots run as one launch in which the per-slot rows stay on the chip; other shapes take
-// the two launches and need the per-slot workspace.
-int bf16n_moe_down_combine(const bf16n_weight * w, const bf16n_mmv_args * a, const void * wts, int wts_bf16, const void * add0,
-                           const void * add1, void * y, int y_bf16, int n_tok, float * ys_workspace, void * stream) {
-    return guarded([&] {
-        ensure_init();
-        check_weight(*w);
-        require(a->ids != nullptr && a->n_used > 0, "moe_down_combine: expert ids are required");
-        require(n_tok > 0 && n_tok <= 65535 && a->ncols == n_tok * a->n_used, "moe_down_combine: ncols must be n_tok * n_used");
-        require(wts && y, "null pointer");
-        require(w->format == FMT_NIBBLE || (a->nrows % w->R == 0 && a->row0 % w->R == 0 && a->rows_per_matrix % w->R == 0),
-                "rows of a product must be whole units");
-        if (a->nrows == 0) {
-            return;
-        }
-        dev::cols p = make_cols(*a);
-        if (dev::tile_down_combine_fits(*w, a->n_used)) {
-            dev::launch_tile_down_combine(*w, p, n_tok, a->x_bf16 != 0, wts, wts_bf16 != 0, add0, add1, y, y_bf16 != 0, (hipStream_t) stream);
-            launch_check("moe_down_combine");
-            return;
-        }
-        require(ys_workspace != nullptr, "moe_down_combine: this layout needs the per-slot workspace (n_tok * n_used * nrows floats)");
-        bf16n_mmv_args b = *a;
-        b.y = ys_workspace;
-        b.y_bf16 = 0;
-        b.y_slot = a->nrows * 4;
-        b.y_tok = (int64_t) a->n_used * a->nrows * 4;
-        if (bf16n_mmv(w, &b, stream, 1) != BF16N_OK) {
-            throw std::invalid_argument(bf16n_last_error());
-        }
-        dev::launch_moe_combine(ys_workspace, wts, wts_bf16 != 0, y, y_bf16 != 0, n_tok, a->n_used, a->nrows, (hipStream_t) stream, add0, add1);
-        launch_check("moe_down_combine");
-    });
-}
-
-// Residual add + RMS norm between the products of a decode step, one launch (engine glue; no counterpart in the
-// reference's core, whose engines bring their own)
-int bf16n_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const uint16_t * gamma, uint16_t * y_sum,
-                      uint16_t * y_norm, int n_tok, int64_t n, float eps, void * stream) {
+// Residual add + weighted combine + RMS norm between the products of a decode step, one launch (engine glue; no
+// counterpart in the reference's core, whose engines bring their own)
+int bf16n_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const float * ys, const void * wts, int wts_bf16,
+                      int n_used, const uint16_t * gamma, uint16_t * y_sum, uint16_t * y_norm, int n_tok, int64_t n, float eps,
+                      void * stream) {
     return guarded([&] {
         ensure_init();
         require(a && y_norm && n_tok > 0 && n_tok <= 65535 && n > 0, "add_rmsnorm: null pointer or empty input");
-        dev::launch_add_rmsnorm(a, b, c, gamma, y_sum, y_norm, n_tok, n, eps, (hipStream_t) stream);
+        require(!ys || (wts && n_used > 0 && n_used < 1024), "add_rmsnorm: rows to combine need weights and a slot count below 1024");
+        dev::add_norm_args p;
+        p.a = a; p.b = b; p.c = c; p.ys = ys; p.wts = wts; p.wts_bf16 = wts_bf16 != 0; p.n_used = n_used;
+        p.gamma = gamma; p.y_sum = y_sum; p.y_norm = y_norm; p.n = n; p.eps = eps;
+        dev::launch_add_rmsnorm(p, n_tok, (hipStream_t) stream);
         launch_check("add_rmsnorm");
     });
 }
@@ -550,15 +518,22 @@ int bf16n_read_probe(const void * src, uint64_t bytes, int pattern, int waves_pe
     });
 }
 
-int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
-                      int32_t * ids, float * weights, void * stream) {
+int bf16n_router_topk_strided(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
+                              int32_t * ids, float * weights, int64_t out_stride, void * stream) {
     return guarded([&] {
         ensure_init();
         require(n_tok > 0 && n_experts > 0 && k > 0 && k <= n_experts && k <= 64, "router_topk: need 0 < k <= min(n_experts, 64)");
         require(n_experts <= 1024, "router_topk: at most 1024 experts");
-        dev::launch_router_topk(logits, logits_stride, n_tok, n_experts, k, renorm != 0, ids, weights, (hipStream_t) stream);
+        require(out_stride >= k, "router_topk: the output row stride must be at least k");
+        dev::launch_router_topk_strided(logits, logits_stride, n_tok, n_experts, k, renorm != 0, ids, weights, out_stride,
+                                        (hipStream_t) stream);
         launch_check("router_topk");
     });
+}
+
+int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
+                      int32_t * ids, float * weights, void * stream) {
+    return bf16n_router_topk_strided(logits, logits_stride, n_tok, n_experts, k, renorm, ids, weights, k, stream);
 }
 
 } // extern "C"

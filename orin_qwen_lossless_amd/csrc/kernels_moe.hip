@@ -16,11 +16,9 @@ __global__ void __launch_bounds__(256) k_swiglu(const float * __restrict__ g, co
     }
 }
 
-// y[t, i] = sum_k w[t, k] * ys[t, k, i], slots in order, one fmaf each (reference launch.cu:539-552); then the optional
-// BF16 vectors add0[t, i], add1[t, i] in FP32 before the rounding
+// y[t, i] = sum_k w[t, k] * ys[t, k, i], slots in order, one fmaf each (reference launch.cu:539-552)
 __global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ ys, const char * __restrict__ w, bool w_bf16,
-                                                     char * __restrict__ y, bool y_bf16, int n_used, int64_t n,
-                                                     const uint16_t * __restrict__ add0, const uint16_t * __restrict__ add1) {
+                                                     char * __restrict__ y, bool y_bf16, int n_used, int64_t n) {
     const int t = blockIdx.y;
     for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t) gridDim.x * 256) {
         float acc = 0.f;
@@ -28,12 +26,6 @@ __global__ void __launch_bounds__(256) k_moe_combine(const float * __restrict__ 
             const int64_t s = (int64_t) t * n_used + k;
             const float wk = w_bf16 ? bf16_bits_to_f32(((const uint16_t *) w)[s]) : ((const float *) w)[s];
             acc = fmaf(wk, ys[s * n + i], acc);
-        }
-        if (add0) {
-            acc += bf16_bits_to_f32(add0[(int64_t) t * n + i]);
-        }
-        if (add1) {
-            acc += bf16_bits_to_f32(add1[(int64_t) t * n + i]);
         }
         store_y(y + (int64_t) t * n * (y_bf16 ? 2 : 4), y_bf16, i, acc);
     }
@@ -176,7 +168,7 @@ __global__ void __launch_bounds__(ROUTE_THREADS) k_route(const char * __restrict
 // arithmetic in the kernels that follow.
 template <int NQ>
 __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ logits, int64_t stride, int n_experts, int k, bool renorm,
-                                                    int32_t * __restrict__ ids, float * __restrict__ weights) {
+                                                    int32_t * __restrict__ ids, float * __restrict__ weights, int64_t out_stride) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float * lg = logits + (int64_t) t * stride;
     float val[NQ];
@@ -215,7 +207,7 @@ __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ l
         top += pj;
         if (lane == (j & 63)) {
             mine = pj; // k <= 64
-            ids[(int64_t) t * k + j] = (int32_t) bi;
+            ids[(int64_t) t * out_stride + j] = (int32_t) bi;
         }
 #pragma unroll
         for (int q = 0; q < NQ; q++) {
@@ -223,30 +215,67 @@ __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ l
         }
     }
     if (lane < k) {
-        weights[(int64_t) t * k + lane] = renorm ? mine / top : mine;
+        weights[(int64_t) t * out_stride + lane] = renorm ? mine / top : mine;
     }
 }
 
 // Residual add + RMS norm of a decode step in one launch (the engines' glue between the products; llama.cpp fuses the
-// same chain in its graph).  Per token: sum = a + b + c in FP32 (b, c optional), y_sum = bf16(sum) (optional: the new
-// residual), y_norm = bf16(sum * rsqrt(mean(sum^2) + eps) * gamma) (gamma optional).  One block per token; the mean is
-// reduced in a fixed order, so the result does not depend on the launch.
-constexpr int NORM_THREADS = 256;
-__global__ void __launch_bounds__(NORM_THREADS) k_add_rmsnorm(const uint16_t * __restrict__ a, const uint16_t * __restrict__ b,
-                                                             const uint16_t * __restrict__ c, const uint16_t * __restrict__ gamma,
-                                                             uint16_t * __restrict__ y_sum, uint16_t * __restrict__ y_norm, int64_t n, float eps) {
+// same chain in its graph).  Per token: sum = a + b + c + sum_k w_k ys_k in FP32 (every addend but a optional; the
+// weighted sum over slots is k_moe_combine's fmaf chain, added last), y_sum = bf16(sum) (optional: the new residual),
+// y_norm = bf16(sum * rsqrt(mean(sum^2) + eps) * gamma) (gamma optional).  One block per token; a thread keeps its
+// elements in registers between the reduction and the scaling (up to NORM_PER_THREAD * 1024 elements per token, the
+// rest is recomputed), and the mean is reduced in a fixed order, so the result does not depend on the launch.
+constexpr int NORM_THREADS = 1024, NORM_PER_THREAD = 4;
+__device__ __forceinline__ float add_norm_value(const add_norm_args & p, const float * wsm, int64_t base, int64_t tok, int64_t i) {
+    float v = bf16_bits_to_f32(p.a[base + i]);
+    if (p.b) {
+        v += bf16_bits_to_f32(p.b[base + i]);
+    }
+    if (p.c) {
+        v += bf16_bits_to_f32(p.c[base + i]);
+    }
+    if (p.ys) {
+        const float * row = p.ys + tok * p.n_used * p.n + i;
+        float acc = 0.f;
+        for (int k0 = 0; k0 < p.n_used; k0 += 8) { // the loads of eight slots at once, then their fmaf chain in order
+            float yk[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                yk[j] = k0 + j < p.n_used ? row[(int64_t) (k0 + j) * p.n] : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (k0 + j < p.n_used) {
+                    acc = fmaf(wsm[k0 + j], yk[j], acc);
+                }
+            }
+        }
+        v += acc;
+    }
+    return v;
+}
+__global__ void __launch_bounds__(NORM_THREADS) k_add_rmsnorm(const add_norm_args p) {
     __shared__ float wave_sq[NORM_THREADS / 64];
-    const int64_t base = (int64_t) blockIdx.x * n;
+    __shared__ float wsm[NORM_THREADS]; // the token's routing weights (n_used < 1024)
+    const int64_t tok = blockIdx.x, base = tok * p.n;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (p.ys) {
+        if (tid < p.n_used) {
+            const int64_t s = tok * p.n_used + tid;
+            wsm[tid] = p.wts_bf16 ? bf16_bits_to_f32(((const uint16_t *) p.wts)[s]) : ((const float *) p.wts)[s];
+        }
+        __syncthreads();
+    }
+    float keep[NORM_PER_THREAD];
     float sq = 0.f;
-    for (int64_t i = tid; i < n; i += NORM_THREADS) {
-        float v = bf16_bits_to_f32(a[base + i]);
-        if (b) {
-            v += bf16_bits_to_f32(b[base + i]);
-        }
-        if (c) {
-            v += bf16_bits_to_f32(c[base + i]);
-        }
+#pragma unroll
+    for (int j = 0; j < NORM_PER_THREAD; j++) {
+        const int64_t i = tid + (int64_t) j * NORM_THREADS;
+        keep[j] = i < p.n ? add_norm_value(p, wsm, base, tok, i) : 0.f;
+        sq = fmaf(keep[j], keep[j], sq);
+    }
+    for (int64_t i = tid + (int64_t) NORM_PER_THREAD * NORM_THREADS; i < p.n; i += NORM_THREADS) {
+        const float v = add_norm_value(p, wsm, base, tok, i);
         sq = fmaf(v, v, sq);
     }
     sq = wave_sum(sq);
@@ -259,28 +288,30 @@ __global__ void __launch_bounds__(NORM_THREADS) k_add_rmsnorm(const uint16_t * _
     for (int k = 0; k < NORM_THREADS / 64; k++) {
         total += wave_sq[k];
     }
-    const float scale = 1.0f / sqrtf(total / (float) n + eps);
-    for (int64_t i = tid; i < n; i += NORM_THREADS) {
-        float v = bf16_bits_to_f32(a[base + i]);
-        if (b) {
-            v += bf16_bits_to_f32(b[base + i]);
+    const float scale = 1.0f / sqrtf(total / (float) p.n + p.eps);
+#pragma unroll
+    for (int j = 0; j < NORM_PER_THREAD; j++) {
+        const int64_t i = tid + (int64_t) j * NORM_THREADS;
+        if (i < p.n) {
+            if (p.y_sum) {
+                p.y_sum[base + i] = f32_to_bf16_rne(keep[j]);
+            }
+            p.y_norm[base + i] = f32_to_bf16_rne(keep[j] * scale * (p.gamma ? bf16_bits_to_f32(p.gamma[i]) : 1.0f));
         }
-        if (c) {
-            v += bf16_bits_to_f32(c[base + i]);
+    }
+    for (int64_t i = tid + (int64_t) NORM_PER_THREAD * NORM_THREADS; i < p.n; i += NORM_THREADS) {
+        const float v = add_norm_value(p, wsm, base, tok, i);
+        if (p.y_sum) {
+            p.y_sum[base + i] = f32_to_bf16_rne(v);
         }
-        if (y_sum) {
-            y_sum[base + i] = f32_to_bf16_rne(v);
-        }
-        const float gmm = gamma ? bf16_bits_to_f32(gamma[i]) : 1.0f;
-        y_norm[base + i] = f32_to_bf16_rne(v * scale * gmm);
+        p.y_norm[base + i] = f32_to_bf16_rne(v * scale * (p.gamma ? bf16_bits_to_f32(p.gamma[i]) : 1.0f));
     }
 }
 
 } // namespace
 
-void launch_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const uint16_t * gamma, uint16_t * y_sum,
-                        uint16_t * y_norm, int n_tok, int64_t n, float eps, hipStream_t stream) {
-    hipLaunchKernelGGL(k_add_rmsnorm, dim3(n_tok), dim3(NORM_THREADS), 0, stream, a, b, c, gamma, y_sum, y_norm, n, eps);
+void launch_add_rmsnorm(const add_norm_args & a, int n_tok, hipStream_t stream) {
+    hipLaunchKernelGGL(k_add_rmsnorm, dim3(n_tok), dim3(NORM_THREADS), 0, stream, a);
 }
 
 void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int cus, hipStream_t stream) {
@@ -289,10 +320,10 @@ void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int c
 }
 
 void launch_moe_combine(const float * ys, const void * w, bool w_bf16, void * y, bool y_bf16, int n_tok, int n_used, int64_t n,
-                        hipStream_t stream, const void * add0, const void * add1) {
+                        hipStream_t stream) {
     const int64_t bx = (n + 255) / 256;
     hipLaunchKernelGGL(k_moe_combine, dim3((unsigned) (bx < 64 ? bx : 64), (unsigned) n_tok), dim3(256), 0, stream, ys, (const char *) w,
-                       w_bf16, (char *) y, y_bf16, n_used, n, (const uint16_t *) add0, (const uint16_t *) add1);
+                       w_bf16, (char *) y, y_bf16, n_used, n);
 }
 
 void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds,
@@ -307,13 +338,18 @@ void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_
     }
 }
 
+// out_stride: elements between the tokens' rows of ids and weights (k when they are dense)
+void launch_router_topk_strided(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
+                                float * weights, int64_t out_stride, hipStream_t stream) {
+    if (n_experts <= 256) {
+        hipLaunchKernelGGL(k_router_topk<4>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights, out_stride);
+    } else {
+        hipLaunchKernelGGL(k_router_topk<16>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights, out_stride);
+    }
+}
 void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
                         float * weights, hipStream_t stream) {
-    if (n_experts <= 256) {
-        hipLaunchKernelGGL(k_router_topk<4>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights);
-    } else {
-        hipLaunchKernelGGL(k_router_topk<16>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights);
-    }
+    launch_router_topk_strided(logits, stride, n_tok, n_experts, k, renorm, ids, weights, k, stream);
 }
 
 } // namespace dev

@@ -652,87 +652,6 @@ __global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(con
     }
 }
 
-// The routed down product of a decode step and the weighted sum over a token's experts in one launch: what k_tile_mmv
-// with expert ids followed by k_moe_combine computes, bit for bit (the per-slot FP32 row sums never leave the block).
-// A block is one row group of one token: n_used * wpg wavefronts, wavefront (slot, i) decodes tiles [i * upw,
-// (i + 1) * upw) of the row group in the matrix of expert ids[token, slot] against that slot's activations; then
-//   y[token, row] = round(sum over slots, in order, of fmaf(wts[token, slot], row sum of the slot, .) + add0 + add1)
-// with the optional BF16 vectors add0 / add1 (a shared expert's output, the residual) added in FP32 before the rounding.
-struct combine_args {
-    const char * wts; bool wts_bf16;   // [n_tok, n_used] routing weights
-    const uint16_t * add0, * add1;     // [n_tok, rows] BF16 or null
-    char * y; bool y_bf16;             // [n_tok, rows]
-    int64_t rows;                      // elements per token in y, add0 and add1
-};
-template <typename TX, bool ONCE>
-__global__ void __launch_bounds__(TV_WAVES * 64) k_tile_down_combine(const bf16n_weight w, const cols p, const combine_args c, int wpg, int upw) {
-    __shared__ __align__(16) uint32_t lut[LUT_WORDS];
-    __shared__ float part[TV_WAVES][32];
-    extern __shared__ __align__(16) uint32_t rings[];
-    const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
-    const int slabs = (int) (w.K / TILE_K);
-    const int slot = wave / wpg, wi = wave % wpg, tok = blockIdx.y;
-    const col_view cv = col_setup(p, tok * p.n_used + slot);
-    const int64_t g = blockIdx.x;
-    const w64_ptrs q = w64p(w);
-    const int64_t unit0 = (cv.rbase / TILE_R + g) * slabs + wi * upw;
-    const uint32_t first = q.ubase[unit0], end = q.ubase[unit0 + upw];
-    stage_lut(lut, q.lut);
-    tchain_t<4, ONCE> ch[1];
-    ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end, ONCE);
-    __syncthreads();
-    float acc = 0.f;
-    for (int u = 0; u < upw; u++) {
-        const int k0 = (wi * upw + u) * TILE_K + 8 * half;
-        ch[0].begin_tile();
-#pragma unroll 1
-        for (int hh = 0; hh < 2; hh++) {
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                const int kk = k0 + 32 * (4 * hh + s);
-                x8<TX> xa, xb;
-                if (sizeof(TX) == 2) {
-                    xa.load(cv.x, kk);
-                    xb.load(cv.x, kk + 16);
-                }
-                uint32_t wp[1][8];
-                tile_step<1, 4, ONCE>(ch, lut, 0, s, wp);
-                ch[0].reload(s, lane);
-                if (sizeof(TX) != 2) {
-                    xa.load(cv.x, kk);
-                    xb.load(cv.x, kk + 16);
-                }
-                acc = xb.dot(wp[0] + 4, xa.dot(wp[0], acc));
-            }
-        }
-    }
-    const float v = acc + __shfl_xor(acc, 32, 64);
-    if (half == 0) {
-        part[wave][l32] = v;
-    }
-    __syncthreads();
-    if (wave == 0 && half == 0) {
-        const int64_t row = g * TILE_R + l32;
-        float sum = 0.f;
-        for (int k = 0; k < p.n_used; k++) {
-            float ys = part[k * wpg][l32];
-            for (int i = 1; i < wpg; i++) {
-                ys += part[k * wpg + i][l32];
-            }
-            const int64_t j = (int64_t) tok * p.n_used + k;
-            const float wk = c.wts_bf16 ? bf16_bits_to_f32(((const uint16_t *) c.wts)[j]) : ((const float *) c.wts)[j];
-            sum = fmaf(wk, ys, sum);
-        }
-        if (c.add0) {
-            sum += bf16_bits_to_f32(c.add0[tok * c.rows + row]);
-        }
-        if (c.add1) {
-            sum += bf16_bits_to_f32(c.add1[tok * c.rows + row]);
-        }
-        store_y(c.y + tok * c.rows * (c.y_bf16 ? 2 : 4), c.y_bf16, row, sum);
-    }
-}
-
 // ---------------------------------------------------------------- dequant / row gather
 
 // one step of a tile as exact BF16 (or FP32) values; only_l >= 0: just that row of the tile, to `out`
@@ -983,41 +902,6 @@ void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols
         TILE_MMV(float, false, w)
     }
 #undef TILE_MMV
-}
-
-// shapes the fused down + combine launch covers: every slot of a token in one block of at most sixteen wavefronts
-bool tile_down_combine_fits(const bf16n_weight & w, int n_used) {
-    return is_tile_layout(w) && n_used >= 1 && n_used <= TV_WAVES; // one wavefront per slot, if need be over all its tiles
-}
-
-// p: the routed product's columns (ids, strides, rows per matrix; y unused); n_tok tokens of p.n_used slots each
-void launch_tile_down_combine(const bf16n_weight & w, const cols & p, int n_tok, bool x_bf16, const void * wts, bool wts_bf16,
-                              const void * add0, const void * add1, void * y, bool y_bf16, hipStream_t stream) {
-    const int slabs = (int) (w.K / TILE_K);
-    int upw = 1;
-    while (slabs % upw != 0 || slabs / upw * p.n_used > TV_WAVES) {
-        upw++;
-    }
-    const int wpg = slabs / upw, waves = wpg * p.n_used;
-    combine_args c;
-    c.wts = (const char *) wts; c.wts_bf16 = wts_bf16;
-    c.add0 = (const uint16_t *) add0; c.add1 = (const uint16_t *) add1;
-    c.y = (char *) y; c.y_bf16 = y_bf16; c.rows = p.nrows;
-    const dim3 grid((unsigned) (p.nrows / TILE_R), n_tok), nt(waves * 64);
-    const size_t shm = (size_t) waves * WAVE_LDS_WORDS * 4;
-    const int64_t n_experts = p.rows_per_matrix > 0 ? w.rows / p.rows_per_matrix : 1;
-    const bool once = n_tok == 1 || (int64_t) n_tok * p.n_used * 4 <= n_experts; // as launch_tile_mmv decides it
-    if (x_bf16) {
-        if (once) {
-            hipLaunchKernelGGL((k_tile_down_combine<bf16_t, true>), grid, nt, shm, stream, w, p, c, wpg, upw);
-        } else {
-            hipLaunchKernelGGL((k_tile_down_combine<bf16_t, false>), grid, nt, shm, stream, w, p, c, wpg, upw);
-        }
-    } else if (once) {
-        hipLaunchKernelGGL((k_tile_down_combine<float, true>), grid, nt, shm, stream, w, p, c, wpg, upw);
-    } else {
-        hipLaunchKernelGGL((k_tile_down_combine<float, false>), grid, nt, shm, stream, w, p, c, wpg, upw);
-    }
 }
 
 void launch_tile_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, hipStream_t stream) {

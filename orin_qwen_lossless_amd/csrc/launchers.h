@@ -39,10 +39,6 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
                         const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
                         int64_t n_pairs, int cus, hipStream_t stream);
 
-bool tile_down_combine_fits(const bf16n_weight & w, int n_used);
-void launch_tile_down_combine(const bf16n_weight & w, const cols & p, int n_tok, bool x_bf16, const void * wts, bool wts_bf16,
-                              const void * add0, const void * add1, void * y, bool y_bf16, hipStream_t stream);
-
 bool tile_mm_dense_pays(const bf16n_weight & w, int64_t nrows, int cus);
 constexpr int TILE_DENSE_F32_COLS = 10; // FP32 columns per dense tile product: three BF16 components each, 32 per pass
 void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, const void * x, bool x_bf16, int64_t x_row, int ncols,
@@ -51,13 +47,22 @@ void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, c
 // MoE glue (kernels_moe.hip)
 void launch_swiglu(const float * g, const float * u, float * y, int64_t n, int cus, hipStream_t stream);
 void launch_moe_combine(const float * ys, const void * w, bool w_bf16, void * y, bool y_bf16, int n_tok, int n_used, int64_t n,
-                        hipStream_t stream, const void * add0 = nullptr, const void * add1 = nullptr);
+                        hipStream_t stream);
 void launch_route(const void * ids, bool ids_i64, int64_t ids_row_stride, int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds,
                   int n_experts, int n_tok, int n_used, int nchannels_y, int sis1, hipStream_t stream);
 void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
                         float * weights, hipStream_t stream);
-void launch_add_rmsnorm(const uint16_t * a, const uint16_t * b, const uint16_t * c, const uint16_t * gamma, uint16_t * y_sum,
-                        uint16_t * y_norm, int n_tok, int64_t n, float eps, hipStream_t stream);
+struct add_norm_args {
+    const uint16_t * a, * b, * c;         // [n_tok, n] BF16; b, c may be null
+    const float * ys; const void * wts;   // [n_tok, n_used, n] FP32 rows and [n_tok, n_used] weights to combine, or null
+    bool wts_bf16; int n_used;
+    const uint16_t * gamma;               // [n] BF16 or null
+    uint16_t * y_sum, * y_norm;           // [n_tok, n] BF16; y_sum may be null
+    int64_t n; float eps;
+};
+void launch_add_rmsnorm(const add_norm_args & a, int n_tok, hipStream_t stream);
+void launch_router_topk_strided(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
+                                float * weights, int64_t out_stride, hipStream_t stream);
 
 // read-bandwidth probe (kernels_probe.hip)
 void launch_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, int cus, hipStream_t stream);

@@ -501,60 +501,34 @@ def moe_combine(ys: torch.Tensor, topk_weights: torch.Tensor, out_dtype: torch.d
     return y
 
 
-def moe_down_combine(a: torch.Tensor, down: Weight, topk_ids: torch.Tensor, topk_weights: torch.Tensor, n_experts: int,
-                     add0: torch.Tensor | None = None, add1: torch.Tensor | None = None,
-                     out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-    """moe_combine(mmv(a, down, topk_ids, H), topk_weights) as one call with the same bits: a [T, n_used, N] hidden
-    activations of the routed experts, out [T, H].  add0 / add1: optional [T, H] BF16 tensors (a shared expert's
-    output, the residual) added in FP32 before the rounding.  Tile-layout matrices run as one launch."""
-    cw = _cweight(down)
-    _check_ids(topk_ids)
-    T, n_used = topk_ids.shape
-    H = down.meta.rows // n_experts
-    _check_x(a, down.meta.K, "a")
-    if a.dim() != 3 or tuple(a.shape[:2]) != (T, n_used):
-        raise ValueError("bf16n.moe_down_combine: a must be [tokens, n_used, N]")
-    if not (topk_weights.is_cuda and topk_weights.is_contiguous() and tuple(topk_weights.shape) == (T, n_used)
-            and topk_weights.dtype in (torch.float32, torch.bfloat16)):
-        raise ValueError("bf16n.moe_down_combine: topk_weights must be contiguous f32/bf16 [tokens, n_used]")
-    for t in (add0, add1):
-        if t is not None and not (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and tuple(t.shape) == (T, H)):
-            raise ValueError("bf16n.moe_down_combine: add tensors must be contiguous bf16 [tokens, H]")
-    y = torch.empty((T, H), dtype=out_dtype, device=a.device)
-    if T == 0:
-        return y
-    args = _lib.MmvArgs()
-    args.x, args.x_bf16 = a.data_ptr(), int(a.dtype == torch.bfloat16)
-    args.ncols, args.n_used, args.x_per_slot = T * n_used, n_used, n_used
-    args.ids, args.ids_s0, args.ids_s1 = topk_ids.data_ptr(), topk_ids.element_size(), topk_ids.stride(0) * topk_ids.element_size()
-    args.x_tok, args.x_slot = a.stride(0) * a.element_size(), a.stride(1) * a.element_size()
-    args.rows_per_matrix, args.row0, args.nrows = H, 0, H
-    tiles = down.meta.wave64 and down.meta.R == 32 and n_used <= 16
-    ws = None if tiles else torch.empty((T, n_used, H), dtype=torch.float32, device=a.device)
-    with torch.cuda.device(a.device):
-        _lib.check(_lib.lib().bf16n_moe_down_combine(
-            C.byref(cw), C.byref(args), topk_weights.data_ptr(), int(topk_weights.dtype == torch.bfloat16),
-            add0.data_ptr() if add0 is not None else None, add1.data_ptr() if add1 is not None else None, y.data_ptr(),
-            int(out_dtype == torch.bfloat16), T, ws.data_ptr() if ws is not None else None, _stream()))
-    return y
-
-
-def add_rmsnorm(a: torch.Tensor, b: torch.Tensor | None = None, c: torch.Tensor | None = None, gamma: torch.Tensor | None = None,
-                eps: float = 1e-6, want_sum: bool = False):
-    """Engine glue of a decode step in one launch: s = a + b + c (FP32), returns bf16(s * rsqrt(mean(s^2) + eps) * gamma),
-    and bf16(s) too when want_sum.  a, b, c: [T, n] BF16 contiguous; gamma: [n] BF16."""
+def add_rmsnorm(a: torch.Tensor, b: torch.Tensor | None = None, c: torch.Tensor | None = None, ys: torch.Tensor | None = None,
+                topk_weights: torch.Tensor | None = None, gamma: torch.Tensor | None = None, eps: float = 1e-6,
+                want_sum: bool = False):
+    """Engine glue of a decode step in one launch: s = a + b + c + moe_combine(ys, topk_weights) in FP32 (every addend
+    but a optional), returns bf16(s * rsqrt(mean(s^2) + eps) * gamma), and bf16(s) too when want_sum.
+    a, b, c: [T, n] BF16 contiguous; ys: [T, n_used, n] FP32 with topk_weights [T, n_used]; gamma: [n] BF16."""
     for t in (a, b, c):
         if t is not None and not (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and t.shape == a.shape and t.dim() == 2):
             raise ValueError("bf16n.add_rmsnorm: inputs must be contiguous bf16 [tokens, n] of one shape")
     if gamma is not None and not (gamma.is_cuda and gamma.dtype == torch.bfloat16 and gamma.is_contiguous() and gamma.numel() == a.shape[1]):
         raise ValueError("bf16n.add_rmsnorm: gamma must be contiguous bf16 [n]")
     T, n = a.shape
+    n_used = 0
+    if ys is not None:
+        if not (ys.is_cuda and ys.dtype == torch.float32 and ys.is_contiguous() and ys.dim() == 3 and ys.shape[0] == T and ys.shape[2] == n):
+            raise ValueError("bf16n.add_rmsnorm: ys must be contiguous f32 [tokens, n_used, n]")
+        n_used = ys.shape[1]
+        w = topk_weights
+        if w is None or not (w.is_cuda and w.is_contiguous() and tuple(w.shape) == (T, n_used) and w.dtype in (torch.float32, torch.bfloat16)):
+            raise ValueError("bf16n.add_rmsnorm: topk_weights must be contiguous f32/bf16 [tokens, n_used]")
     y = torch.empty_like(a)
     ysum = torch.empty_like(a) if want_sum else None
     ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
     with torch.cuda.device(a.device):
-        _lib.check(_lib.lib().bf16n_add_rmsnorm(a.data_ptr(), ptr(b), ptr(c), ptr(gamma), ptr(ysum), y.data_ptr(), T, n,
-                                                C.c_float(eps), _stream()))
+        _lib.check(_lib.lib().bf16n_add_rmsnorm(
+            a.data_ptr(), ptr(b), ptr(c), ptr(ys), ptr(topk_weights) if ys is not None else None,
+            int(ys is not None and topk_weights.dtype == torch.bfloat16), n_used, ptr(gamma), ptr(ysum), y.data_ptr(), T, n,
+            C.c_float(eps), _stream()))
     return (y, ysum) if want_sum else y
 
 
@@ -568,17 +542,42 @@ def swiglu(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
     return y
 
 
-def router_topk(logits: torch.Tensor, k: int, renorm: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
-    """Softmax over experts + k largest on the device: (topk_weights f32 [T, k], topk_ids int32 [T, k])."""
+def router_topk(logits: torch.Tensor, k: int, renorm: bool = True, out: tuple[torch.Tensor, torch.Tensor] | None = None
+                ) -> tuple[torch.Tensor, torch.Tensor]:
+    """Softmax over experts + k largest on the device: (topk_weights f32 [T, k], topk_ids int32 [T, k]).
+    out = (weights, ids): contiguous [T, m >= k] tensors whose first k columns are written (a caller that runs fixed
+    experts beside the routed ones keeps their weights and ids in the columns from k on); they are returned."""
     if not (logits.is_cuda and logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1):
         raise ValueError("bf16n.router_topk: logits must be f32 [tokens, n_experts], contiguous along experts")
     T, E = logits.shape
-    ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
-    wts = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    if out is None:
+        ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+        wts = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    else:
+        wts, ids = out
+        if not (wts.dtype == torch.float32 and ids.dtype == torch.int32 and wts.shape == ids.shape and wts.dim() == 2
+                and wts.shape[0] == T and wts.shape[1] >= k and wts.is_contiguous() and ids.is_contiguous()
+                and wts.device == logits.device and ids.device == logits.device):
+            raise ValueError("bf16n.router_topk: out must be contiguous (f32, int32) [tokens, m >= k] tensors on the logits' device")
     with torch.cuda.device(logits.device):
-        _lib.check(_lib.lib().bf16n_router_topk(logits.data_ptr(), logits.stride(0), T, E, k, int(renorm), ids.data_ptr(),
-                                                wts.data_ptr(), _stream()))
+        _lib.check(_lib.lib().bf16n_router_topk_strided(logits.data_ptr(), logits.stride(0), T, E, k, int(renorm), ids.data_ptr(),
+                                                        wts.data_ptr(), ids.shape[1], _stream()))
     return wts, ids
+
+
+_probe_sink: dict = {}
+
+
+def read_probe(buf: torch.Tensor, pattern: int = 0, waves_per_cu: int = 0) -> None:
+    """One launch of the library's read-only kernel over a contiguous device buffer (bf16n_read_probe: the yardstick of
+    the reference's bench/micro/bwprobe.cu).  pattern 0 / 1: a contiguous range per wavefront, non-temporal / plain
+    loads; 2 / 3: grid-stride."""
+    if not (buf.is_cuda and buf.is_contiguous() and buf.data_ptr() % 16 == 0):
+        raise ValueError("bf16n.read_probe: a contiguous, 16-byte aligned device buffer is required")
+    sink = _probe_sink.setdefault(buf.device, torch.zeros(1, dtype=torch.int32, device=buf.device))
+    with torch.cuda.device(buf.device):
+        _lib.check(_lib.lib().bf16n_read_probe(buf.data_ptr(), buf.numel() * buf.element_size(), pattern, waves_per_cu,
+                                               sink.data_ptr(), _stream()))
 
 
 def glu2_supported(gate: Weight, up: Weight) -> bool:
@@ -604,10 +603,10 @@ def _experts_gemv_hidden(x, gate, up, topk_ids, n_mid):
     return swiglu(mmv(x, gate, topk_ids, n_mid), mmv(x, up, topk_ids, n_mid))
 
 
-def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_weights: torch.Tensor,
-                topk_ids: torch.Tensor, n_experts: int) -> torch.Tensor:
-    """Routed experts of one MoE layer, BF16 out: for every token the weighted sum over its top-k experts of
-    down_e(silu(gate_e x) * (up_e x)) (engines/vllm/vllm_bf16n/ops.py:251-271).
+def moe_experts_rows(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_ids: torch.Tensor, n_experts: int
+                     ) -> torch.Tensor:
+    """The per-(token, slot) outputs down_e(silu(gate_e x) * (up_e x)) of the routed experts, FP32 [T, n_used, H]:
+    moe_experts before the weighted sum (callers that fold the sum into their own next launch, add_rmsnorm, stop here).
 
     The reference switches from expert GEMVs to the batched kernels above 8 tokens.  Here the GEMVs stay ahead only
     while the routed pairs are few against the experts (each pair decodes one expert matrix in its own GEMV column; the
@@ -621,8 +620,13 @@ def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_we
     per_expert = MOE_GEMV_PAIRS_PER_EXPERT[0 if tiles else 1]
     gemv_tokens = max(4 if tiles else GEMV_MAX_TOKENS, int(per_expert * n_experts) // n_used)
     if n_tokens > gemv_tokens and mm_ids_supported(gate, up) and mm_ids_supported(down):
-        return moe_combine(_experts_batched(x, gate, up, down, topk_ids, n_experts), topk_weights, torch.bfloat16)
-    # one GEMV column per (token, slot), FP32 between the products; the down product and the weighted sum are one call
-    # (one launch for tile-layout experts, with the bits of mmv followed by moe_combine)
-    hidden = _experts_gemv_hidden(x, gate, up, topk_ids, n_mid)
-    return moe_down_combine(hidden, down, topk_ids, topk_weights.contiguous(), n_experts)
+        return _experts_batched(x, gate, up, down, topk_ids, n_experts)
+    # one GEMV column per (token, slot), FP32 between the products
+    return mmv(_experts_gemv_hidden(x, gate, up, topk_ids, n_mid), down, topk_ids, n_out)
+
+
+def moe_experts(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_weights: torch.Tensor,
+                topk_ids: torch.Tensor, n_experts: int) -> torch.Tensor:
+    """Routed experts of one MoE layer, BF16 out: for every token the weighted sum over its top-k experts of
+    down_e(silu(gate_e x) * (up_e x)) (engines/vllm/vllm_bf16n/ops.py:251-271); see moe_experts_rows for the paths."""
+    return moe_combine(moe_experts_rows(x, gate, up, down, topk_ids, n_experts), topk_weights, torch.bfloat16)

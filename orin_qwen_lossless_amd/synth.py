@@ -94,3 +94,63 @@ def nibble_rows_with_exponents(rows: int, K: int, n_exp: int, seed: int) -> np.n
         sign = (uniform(K, seed + r, 7) < 0.5).astype(np.uint16)
         out[r] = (sign << 15) | (exps[perm] << 7) | mant
     return out
+
+
+# ---------------------------------------------------------------- the same generator on a torch device
+
+def _i64(c: int) -> int:
+    """A 64-bit constant as the two's-complement int64 torch holds."""
+    return c - (1 << 64) if c >= (1 << 63) else c
+
+
+def _splitmix64_torch(x):
+    """splitmix64 on int64 tensors: additions and multiplications wrap modulo 2^64 as the unsigned ones do; the right
+    shifts are made logical by masking the sign extension away."""
+    def shr(v, s):
+        return (v >> s) & ((1 << (64 - s)) - 1)
+
+    z = x + _i64(0x9E3779B97F4A7C15)
+    z = (z ^ shr(z, 30)) * _i64(0xBF58476D1CE4E5B9)
+    z = (z ^ shr(z, 27)) * _i64(0x94D049BB133111EB)
+    return z ^ shr(z, 31)
+
+
+def normal_torch(n: int, seed: int, device, first: int = 0):
+    """Elements [first, first + n) of normal(., seed) as a float32 tensor on `device` (first even): the same counters,
+    the same Box-Muller in float64.  The integer part is exact; log / sqrt / cos / sin come from the device's math
+    library, whose last-bit differences from numpy's survive the rounding to float32 in about one element in 10^8."""
+    import math
+
+    import torch
+
+    assert first % 2 == 0
+    m = (n + 1) // 2
+    i = torch.arange(first // 2, first // 2 + m, dtype=torch.int64, device=device)
+    u = []
+    for stream in (1, 2):
+        z = _splitmix64_torch(i + _i64(((seed << 32) + (stream << 56)) & ((1 << 64) - 1)))
+        u.append((((z >> 11) & ((1 << 53) - 1)).to(torch.float64) + 0.5) * (1.0 / (1 << 53)))
+    r = torch.sqrt(-2.0 * torch.log(u[0]))
+    ang = (2 * math.pi) * u[1]
+    out = torch.stack((r * torch.cos(ang), r * torch.sin(ang)), dim=1).reshape(-1)
+    return out[:n].to(torch.float32)
+
+
+def weights_torch(rows: int, K: int, seed: int, device, scale: float = 0.02, block_rows: int = 1 << 15):
+    """weights(rows, K, seed) as a BF16 tensor on `device`, generated there in blocks of rows."""
+    import torch
+
+    w = torch.empty((rows, K), dtype=torch.bfloat16, device=device)
+    assert K % 2 == 0
+    for r0 in range(0, rows, block_rows):
+        nr = min(block_rows, rows - r0)
+        f = normal_torch(nr * K, seed, device, first=r0 * K) * torch.tensor(scale, dtype=torch.float32, device=device)
+        w[r0: r0 + nr] = f.to(torch.bfloat16).view(nr, K)
+    return w
+
+
+def activations_torch(T: int, K: int, seed: int, device):
+    """activations(T, K, seed) as a BF16 tensor on `device`."""
+    import torch
+
+    return normal_torch(T * K, seed, device).to(torch.bfloat16).view(T, K)

@@ -22,7 +22,7 @@ def test_more_than_one_gpu_is_refused():
 def test_one_json_line_with_roofline_and_cpu_baseline():
     # a reduced matrix (the same kernel instance: K = 2048, 16-row units) so that the test takes seconds
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--rows", "65536", "--steps", "10", "--warmup", "2",
-                        "--cpu-rows", "2048"], capture_output=True, text=True, timeout=600)
+                        "--cpu-rows", "2048", "--cpu-seconds", "3"], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
     assert len(lines) == 1
@@ -40,3 +40,35 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert cb["kind"] in ("port", "reference") and cb["cores"] >= 1 and cb["value"] > 0 and cb["unit"] == "GB/s" and cb["sample"]
     assert d["value"] > 100 * cb["value"] / 10                   # a GPU, not a fallback
     assert d["extra"]["max_err_over_sum_abs"] <= 1e-5           # the timed kernel's result was checked in the same run
+    assert rf["traffic"] is None and rf["traffic_source"] is None   # counters exist for the full-size workload only
+    assert "timed" in d["config"]["workload"] and "generator" in d["config"]
+    # the timed region: blocks of `steps` launches until 50 ms have been timed, the median block reported
+    lo, hi = d["extra"]["block_us_per_step_min_max"]
+    assert lo <= d["ms_per_step"] * 1e3 <= hi
+    # a read-only kernel of the library's own as the yardstick, in its four access patterns
+    assert len(d["extra"]["read_probe_GBps"]) == 8 and d["extra"]["plain_stream_read_GBps"] == max(d["extra"]["read_probe_GBps"].values())
+    # the CPU reference configuration, one thread and all
+    c1 = cb["config1_2048x2048"]
+    assert c1["threads_1"]["us"] > 0 and c1["compressed_bytes"] > 0 and f"threads_{cb['cores']}" in c1
+    # the other configurations of the path, measured in the same run
+    cf = d["extra"]["configs"]
+    for key in ("lm_head_batch4", "gemv_512x2048", "gemv_2048x512", "moe_layer_batch1_graph", "moe_prefill_T2048", "moe_prefill_T8192",
+                "decode_step"):
+        assert key in cf, key
+    for b in ("batch1", "batch4"):
+        e = cf["decode_step"][b]
+        assert e["us"] > 0 and e["bf16_us"] > 0 and e["eager_equals_graph"] and 0 < e["frac_of_hbm_peak"] < 1
+        assert abs(e["speedup_vs_bf16"] - e["bf16_us"] / e["us"]) < 0.02
+    for T in (2048, 8192):
+        e = cf[f"moe_prefill_T{T}"]
+        assert 0 < e["frac_of_bf16_mfma_peak"] < 1 and e["weight_decode_GBps"] > 0
+
+
+def test_counter_traffic_comes_from_the_committed_profile():
+    sys.path.insert(0, ROOT)
+    import bench
+
+    t = bench.measured_traffic(248320, 2048)
+    assert t is not None and 0.98 * 686_670_516 < t < 1.10 * 686_670_516
+    assert bench.measured_traffic(65536, 2048) is None
+    assert os.path.exists(os.path.join(ROOT, bench.TRAFFIC_PROFILE))

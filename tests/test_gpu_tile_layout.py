@@ -262,50 +262,43 @@ def test_moe_experts_path_switch_by_routed_pairs_per_expert(ops, T, monkeypatch)
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
 
 
-@pytest.mark.parametrize("layout", ["tiles", "units"])
-@pytest.mark.parametrize("T", [1, 3, 6])
-def test_down_product_and_combine_in_one_call(ops, layout, T):
-    """moe_down_combine == moe_combine(mmv(a, down, ids)) bit for bit (one launch for tiles, the two launches for other
-    layouts), FP32 and BF16 hidden activations and weights, FP32 and BF16 out; the optional added vectors enter in FP32
-    before the rounding."""
-    E, k, N, H = 12, 8, 512, 256
-    r = 32 if layout == "tiles" else 16
-    down = enc(ops, synth.weights(E * H, N, 301), 3, r, False, True)
-    rng = np.random.default_rng(T)
-    ids = torch.from_numpy(np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)).cuda()
-    a = torch.from_numpy(rng.standard_normal((T, k, N)).astype(np.float32)).cuda()
-    wts = torch.softmax(torch.from_numpy(rng.standard_normal((T, k)).astype(np.float32)).cuda(), -1)
-    add0 = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).cuda().to(torch.bfloat16)
-    add1 = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).cuda().to(torch.bfloat16)
-    for hidden in (a, a.to(torch.bfloat16)):
-        for w in (wts, wts.to(torch.bfloat16)):
-            ys = ops.mmv(hidden, down, ids, H)
-            for odt in (torch.float32, torch.bfloat16):
-                want = ops.moe_combine(ys, w, odt)
-                got = ops.moe_down_combine(hidden, down, ids, w, E, out_dtype=odt)
-                assert torch.equal(got, want), (hidden.dtype, w.dtype, odt)
-            comb = ops.moe_combine(ys, w, torch.float32)
-            want1 = (comb + add0.float()).to(torch.bfloat16)
-            assert torch.equal(ops.moe_down_combine(hidden, down, ids, w, E, add0=add0), want1)
-            want2 = ((comb + add0.float()) + add1.float()).to(torch.bfloat16)
-            assert torch.equal(ops.moe_down_combine(hidden, down, ids, w, E, add0=add0, add1=add1), want2)
-    with pytest.raises(ValueError):
-        ops.moe_down_combine(a[:, :4], down, ids, wts, E)
-
-
-@pytest.mark.parametrize("T,n", [(1, 2048), (4, 2048), (3, 1000), (2, 5120)])
+@pytest.mark.parametrize("T,n", [(1, 2048), (4, 2048), (3, 1000), (2, 5120), (1, 4104)])
 def test_add_rmsnorm_glue(ops, T, n):
+    """The decode step's glue launch: the FP32 sum of its addends (BF16 rows in argument order, then the weighted sum
+    over expert slots with moe_combine's fmaf chain) rounded once to BF16, and its RMS norm against FP64."""
     rng = np.random.default_rng(n + T)
     mk = lambda s=1.0: torch.from_numpy((rng.standard_normal((T, n)) * s).astype(np.float32)).cuda().to(torch.bfloat16)  # noqa: E731
     a, b, c = mk(), mk(0.3), mk(3.0)
     gamma = torch.from_numpy((1 + 0.1 * rng.standard_normal(n)).astype(np.float32)).cuda().to(torch.bfloat16)
-    for bb, cc, gg in ((None, None, None), (b, None, None), (b, c, None), (b, c, gamma), (None, c, gamma)):
-        y, ysum = ops.add_rmsnorm(a, bb, cc, gg, eps=1e-6, want_sum=True)
-        s32 = a.float()
-        for t in (bb, cc):
-            s32 = s32 + t.float() if t is not None else s32
-        assert torch.equal(ysum, s32.to(torch.bfloat16))           # the FP32 sum in argument order, rounded once
-        s64 = s32.double()
-        ref = s64 * torch.rsqrt((s64 * s64).mean(-1, keepdim=True) + 1e-6) * (gg.double() if gg is not None else 1.0)
-        assert torch.all((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-30)
-        assert torch.equal(ops.add_rmsnorm(a, bb, cc, gg, eps=1e-6), y)
+    ys = torch.from_numpy(rng.standard_normal((T, 9, n)).astype(np.float32)).cuda()
+    wts = torch.softmax(torch.from_numpy(rng.standard_normal((T, 9)).astype(np.float32)).cuda(), -1)
+    for bb, cc, yy, gg in ((None, None, None, None), (b, None, None, None), (b, c, None, None), (b, c, ys, gamma),
+                           (None, None, ys, None), (None, c, None, gamma)):
+        for w in (wts, wts.to(torch.bfloat16)):
+            y, ysum = ops.add_rmsnorm(a, bb, cc, ys=yy, topk_weights=w if yy is not None else None, gamma=gg, eps=1e-6, want_sum=True)
+            s32 = a.float()
+            for t in (bb, cc):
+                s32 = s32 + t.float() if t is not None else s32
+            if yy is not None:
+                s32 = s32 + ops.moe_combine(yy, w, torch.float32)
+            assert torch.equal(ysum, s32.to(torch.bfloat16))
+            s64 = s32.double()
+            ref = s64 * torch.rsqrt((s64 * s64).mean(-1, keepdim=True) + 1e-6) * (gg.double() if gg is not None else 1.0)
+            assert torch.all((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-30)
+            assert torch.equal(ops.add_rmsnorm(a, bb, cc, ys=yy, topk_weights=w if yy is not None else None, gamma=gg, eps=1e-6), y)
+    with pytest.raises(ValueError):
+        ops.add_rmsnorm(a, ys=ys, topk_weights=wts[:, :4].contiguous())
+
+
+def test_router_topk_into_wider_rows(ops):
+    """The router's top-k written into the first k columns of wider rows: the other columns (a stacked shared expert's
+    id and weight) stay as the caller set them, and the k columns equal the dense call's."""
+    lg = torch.randn((5, 256), generator=torch.Generator().manual_seed(3)).cuda()
+    wts, ids = torch.full((5, 9), 1.0, device="cuda"), torch.full((5, 9), 256, dtype=torch.int32, device="cuda")
+    w2, i2 = ops.router_topk(lg, 8, out=(wts, ids))
+    dw, di = ops.router_topk(lg, 8)
+    assert w2 is wts and i2 is ids
+    assert torch.equal(ids[:, :8], di) and torch.equal(wts[:, :8], dw)
+    assert bool((ids[:, 8] == 256).all()) and bool((wts[:, 8] == 1.0).all())
+    with pytest.raises(ValueError):
+        ops.router_topk(lg, 8, out=(wts[:, :4].contiguous(), ids[:, :4].contiguous()))
