@@ -69,6 +69,23 @@ inline int release(const void * owner) {
     return n;
 }
 
+// The dense path above gemv_max_tokens(w) tokens (patch 0002:423-437: exact BF16 reconstruction, then the stock BF16
+// GEMM): y (n_tok x rows) = x (n_tok x K) W^T, BF16 in and out, FP32 accumulation; row strides in elements.  Scratch for
+// the decoded rows and the GEMM's workspace are the caller's (dense_sizes says how much; also to be called once before
+// the first capture), so the call itself allocates nothing.
+struct dense_sizes_t { uint64_t scratch_bytes, gemm_workspace_bytes; };
+inline dense_sizes_t dense_sizes(const weight & w) {
+    const bf16n_weight c = bf16n::detail::c_view(w);
+    dense_sizes_t s{};
+    bf16n::detail::check(bf16n_linear_dense_sizes(&c, &s.scratch_bytes, &s.gemm_workspace_bytes));
+    return s;
+}
+inline void linear_dense(const weight & w, const uint16_t * x, int64_t x_row, int n_tok, uint16_t * y, int64_t y_row, void * scratch,
+                         uint64_t scratch_bytes, void * gemm_workspace, uint64_t gemm_workspace_bytes, hipStream_t stream) {
+    const bf16n_weight c = bf16n::detail::c_view(w);
+    bf16n::detail::check(bf16n_linear_dense(&c, x, x_row, n_tok, y, y_row, scratch, scratch_bytes, gemm_workspace, gemm_workspace_bytes, stream));
+}
+
 inline bool verify_roundtrip(const weight & w, const uint16_t * bf16_host) {
     const bf16n_weight c = bf16n::detail::c_view(w);
     int ok = 0;

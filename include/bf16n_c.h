@@ -78,6 +78,17 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
  * reference's fixed rule, core/torch/torch_bindings.cpp:195 and ops.py:25-27; 16 for matrices of 128 Mi weights and more
  * in wave64 units; 512 where the product runs on the matrix cores) */
 int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out);
+/* The dense path beyond bf16n_gemv_max_tokens: y (n_tok x rows, BF16) = x (n_tok x K, BF16) W^T through exact dequant of
+ * the matrix, in pieces of at most 64 MiB, into `scratch`, and a stock BF16 GEMM with FP32 accumulation (hipBLASLt) on
+ * each piece: what the reference's llama.cpp adapter does above 8 tokens with a pool allocation and cuBLAS
+ * (engines/llamacpp/patches/0002-...patch:423-437, switch at :157) and its torch binding with at::mm
+ * (core/torch/torch_bindings.cpp:195-239).  Row strides in elements.  Nothing is allocated in the call: scratch (at
+ * least one unit of decoded rows; *scratch_bytes of bf16n_linear_dense_sizes for the fewest pieces) and the GEMM
+ * workspace (*gemm_workspace_bytes) are the caller's.  Call bf16n_linear_dense_sizes once before capturing the call
+ * into a HIP graph: it loads the BLAS and creates its handle. */
+int bf16n_linear_dense_sizes(const bf16n_weight * w, uint64_t * scratch_bytes, uint64_t * gemm_workspace_bytes);
+int bf16n_linear_dense(const bf16n_weight * w, const uint16_t * x, int64_t x_row, int n_tok, uint16_t * y, int64_t y_row,
+                       void * scratch, uint64_t scratch_bytes, void * gemm_workspace, uint64_t gemm_workspace_bytes, void * stream);
 int bf16n_mmv_glu(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream);            /* mmv_glu merged [gate;up], launch.h:55, launch.cu:327-339 */
 int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf16n_mmv_args * a, void * stream); /* mmv_glu(gate, up), launch.h:61, launch.cu:341-365 */
 int bf16n_dequant(const bf16n_weight * w, int64_t row0, int64_t nrows, uint16_t * out, void * stream); /* dequant, launch.h:63, launch.cu:367-402 */

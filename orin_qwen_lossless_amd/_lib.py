@@ -42,6 +42,8 @@ SYMBOLS = {
     "bf16n_cu_count": (_i, [C.POINTER(_i)]),
     "bf16n_mmv": (_i, [_WP, _AP, _vp, _i]),
     "bf16n_gemv_max_tokens": (_i, [_WP, C.POINTER(_i)]),
+    "bf16n_linear_dense_sizes": (_i, [_WP, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "bf16n_linear_dense": (_i, [_WP, _vp, _i64, _i, _vp, _i64, _vp, C.c_uint64, _vp, C.c_uint64, _vp]),
     "bf16n_mmv_glu": (_i, [_WP, _AP, _vp]),
     "bf16n_mmv_glu2": (_i, [_WP, _WP, _AP, _vp]),
     "bf16n_dequant": (_i, [_WP, _i64, _i64, _vp, _vp]),

@@ -17,7 +17,7 @@ LIB = os.path.join(HERE, "libbf16n_hip.so")
 BENCH = os.path.join(HERE, "bf16n_bench")  # stand-alone timing program (csrc/bench_mmv.cpp), linked against the library
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "adapter.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip", "kernels_probe.hip"]
+SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "adapter.cpp", "dense.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip", "kernels_probe.hip"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall", "-Wno-unused-function"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -29,7 +29,8 @@ def _compile(src: str, force: bool) -> str:
         os.path.join(ROOT, "include", "bf16n_c.h"), os.path.join(ROOT, "include", "bf16n", "format.h")]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
         return obj
-    cmd = [HIPCC] + COMMON + (HIP_FLAGS if src.endswith(".hip") else ["-x", "hip"] + HIP_FLAGS if src == "adapter.cpp" else ["-x", "hip", "--offload-arch=gfx950"] if src == "capi.cpp" else []) + ["-c", path, "-o", obj]
+    cmd = [HIPCC] + COMMON + (HIP_FLAGS if src.endswith(".hip") else ["-x", "hip"] + HIP_FLAGS if src == "adapter.cpp" else ["-x", "hip", "--offload-arch=gfx950"] if src == "capi.cpp"
+                             else ["-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include"] if src == "dense.cpp" else []) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         sys.stderr.write(r.stdout + r.stderr)
@@ -42,7 +43,7 @@ def build(force: bool = False) -> str:
     with ThreadPoolExecutor(max_workers=4) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), SOURCES))
     if force or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs):
-        r = subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs + ["-lpthread"], capture_output=True, text=True)
+        r = subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs + ["-lpthread", "-ldl"], capture_output=True, text=True)
         if r.returncode != 0:
             sys.stderr.write(r.stdout + r.stderr)
             raise RuntimeError("link failed")

@@ -410,6 +410,32 @@ def linear(x: torch.Tensor, w: Weight, bias: torch.Tensor | None = None) -> torc
     return y.view(oshape)
 
 
+def linear_dense(x: torch.Tensor, w: Weight, scratch: torch.Tensor | None = None, gemm_workspace: torch.Tensor | None = None
+                 ) -> torch.Tensor:
+    """y = x W^T in BF16 through the library's dense path (bf16n_linear_dense: exact dequant in pieces into `scratch`
+    + hipBLASLt BF16 GEMM, FP32 accumulation), the path of linear() above gemv_max_tokens without torch's GEMM.  scratch /
+    gemm_workspace: uint8 device buffers (allocated here when not given; a caller under graph capture passes its own)."""
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != w.meta.K or not x.is_cuda:
+        raise ValueError("bf16n.linear_dense: x must be a bf16 device tensor [tokens, K]")
+    _check_x(x, w.meta.K, "x")
+    cw = _cweight(w)
+    need_s, need_g = C.c_uint64(), C.c_uint64()
+    L = _lib.lib()
+    _lib.check(L.bf16n_linear_dense_sizes(C.byref(cw), C.byref(need_s), C.byref(need_g)))
+    if scratch is None:
+        scratch = torch.empty(need_s.value, dtype=torch.uint8, device=x.device)
+    if gemm_workspace is None:
+        gemm_workspace = torch.empty(need_g.value, dtype=torch.uint8, device=x.device)
+    T = x.shape[0]
+    y = torch.empty((T, w.meta.rows), dtype=torch.bfloat16, device=x.device)
+    if T == 0:
+        return y
+    with torch.cuda.device(x.device):
+        _lib.check(L.bf16n_linear_dense(C.byref(cw), x.data_ptr(), x.stride(0), T, y.data_ptr(), y.stride(0), scratch.data_ptr(),
+                                        scratch.numel(), gemm_workspace.data_ptr(), gemm_workspace.numel(), _stream()))
+    return y
+
+
 def get_rows(ids: torch.Tensor, w: Weight, out_dtype: torch.dtype = torch.bfloat16, row0: int = 0) -> torch.Tensor:
     cw = _cweight(w)
     if not ids.is_cuda or ids.dim() != 1:

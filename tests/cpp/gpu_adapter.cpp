@@ -106,6 +106,35 @@ int main() {
     }
     std::printf("mmv %s\n", all_ok ? "ok" : "OUT OF BOUND");
 
+    // more tokens than the GEMV serves: the dense path (exact dequant into caller-owned scratch + the stock BF16 GEMM)
+    {
+        const int T = 12;
+        const int64_t rows = ts[0].rows_per_matrix;
+        std::vector<uint16_t> xs((size_t) T * K);
+        for (auto & v : xs) { v = f32_to_bf16((float) gauss()); }
+        const auto sizes = ad::dense_sizes(base->w);
+        uint16_t * d_xs, * d_ys; void * d_scratch, * d_ws;
+        HIP_OK(hipMalloc(&d_xs, xs.size() * 2)); HIP_OK(hipMalloc(&d_ys, (size_t) T * rows * 2));
+        HIP_OK(hipMalloc(&d_scratch, sizes.scratch_bytes)); HIP_OK(hipMalloc(&d_ws, sizes.gemm_workspace_bytes));
+        HIP_OK(hipMemcpy(d_xs, xs.data(), xs.size() * 2, hipMemcpyHostToDevice));
+        ad::linear_dense(base->w, d_xs, K, T, d_ys, rows, d_scratch, sizes.scratch_bytes, d_ws, sizes.gemm_workspace_bytes, stream);
+        std::vector<uint16_t> ys((size_t) T * rows);
+        HIP_OK(hipMemcpyAsync(ys.data(), d_ys, ys.size() * 2, hipMemcpyDeviceToHost, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        bool dense_ok = true;
+        for (int t = 0; t < T; t++) {
+            for (int64_t r = 0; r < rows; r += 37) {
+                double ref = 0, bound = 0;
+                for (int64_t k = 0; k < K; k++) {
+                    const double q = (double) bf16_to_f32(ts[0].host[r * K + k]) * (double) bf16_to_f32(xs[(size_t) t * K + k]);
+                    ref += q; bound += std::fabs(q);
+                }
+                dense_ok = dense_ok && std::fabs(bf16_to_f32(ys[(size_t) t * rows + r]) - ref) <= std::fabs(ref) / 256 + 1e-5 * bound;
+            }
+        }
+        std::printf("linear_dense %s\n", dense_ok ? "ok" : "OUT OF BOUND");
+    }
+
     // freeing a buffer drops its tensors and their aux storage; the other buffer's tensor stays
     const int dropped = ad::release(&owner_a);
     std::printf("release %s\n", dropped == 2 && !ad::is_registered(ts[0].data) && !ad::is_registered(ts[1].data) && ad::is_registered(ts[2].data) &&

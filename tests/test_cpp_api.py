@@ -70,7 +70,7 @@ def test_cpp_adapter_load_time_path_on_the_device(tmp_path):
     for name in ("output.weight", "blk.0.ffn_gate_exps.weight", "blk.0.ffn_down_shexp.weight"):
         assert f"convert {name} ok" in out, out
     assert "registered 3" in out
-    for line in ("lookup ok", "verify ok", "mmv ok", "release ok"):
+    for line in ("lookup ok", "verify ok", "mmv ok", "linear_dense ok", "release ok"):
         assert line in out, out
     assert "invalid_argument bf16n: adapter: the address is not the start of a row" in out
     assert "invalid_argument bf16n: adapter: the tensor overlaps a registered one" in out

@@ -377,3 +377,43 @@ def test_nibble_every_chunk_count(ops, oracle, K):
     g = ops.mmv(tbf16(xb), enc(ops, wb[: rows // 2], NIB))
     u = ops.mmv(tbf16(xb), enc(ops, wb[rows // 2:], NIB))
     assert torch.equal(fused, ops.swiglu(g, u))
+
+
+@pytest.mark.parametrize("layout", ["nibble", "units", "tiles", "reference"])
+@pytest.mark.parametrize("T", [9, 33, 512])
+def test_linear_dense_through_the_c_abi(ops, layout, T):
+    """The dense path for more tokens than the GEMV serves, behind the C ABI: exact dequant into the caller's scratch in
+    pieces + the stock BF16 GEMM.  Against FP64 products of the exact weights (the output is BF16: one rounding of an
+    FP32-accumulated sum), with a scratch buffer that forces several pieces, and captured into a HIP graph."""
+    rows, K = (1000, 1024) if layout == "nibble" else (2048, 1536) if layout == "reference" else (4096, 2048)
+    wb = synth.weights(rows, K, 700 + T)
+    w = {"nibble": lambda: enc(ops, wb, NIB), "units": lambda: enc(ops, wb, HP, 4, False, True),
+         "tiles": lambda: enc(ops, wb, HP, 32, False, True), "reference": lambda: enc(ops, wb, HP, 8, False, False)}[layout]()
+    x = tbf16(synth.activations(T, K, 701))
+    wd = torch.from_numpy(synth.bf16_bits_to_f32(wb)).cuda().double()
+    ref, bound = x.double() @ wd.t(), x.double().abs() @ wd.abs().t()
+    y = ops.linear_dense(x, w)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (T, rows)
+    assert bool(((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * bound).all())
+    # a scratch buffer of 40 decoded rows: many pieces, the same result (each output element is one GEMM's dot product
+    # whatever the piece it falls into; the BLAS may pick another kernel for the narrower pieces, hence the bound again)
+    small = torch.empty(40 * K * 2, dtype=torch.uint8, device="cuda")
+    y2 = ops.linear_dense(x, w, scratch=small)
+    assert bool(((y2.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * bound).all())
+    with pytest.raises(ValueError, match="scratch"):
+        ops.linear_dense(x, w, scratch=torch.empty(K * 2, dtype=torch.uint8, device="cuda"))
+    # captured: the call allocates nothing when the buffers are the caller's
+    scratch = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    wsp = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
+    ops.linear_dense(x, w, scratch, wsp)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        yg = ops.linear_dense(x, w, scratch, wsp)
+    for rep in range(3):
+        x.copy_(tbf16(synth.activations(T, K, 710 + rep)))
+        want = ops.linear_dense(x, w, scratch, wsp).clone()
+        yg.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(yg, want), rep
