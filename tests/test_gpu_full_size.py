@@ -417,3 +417,89 @@ def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, R):
         assert np.all(np.abs(y1 - y64) <= 1e-5 * bound)
     y16 = ops.linear(x, enc)
     assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y4))
+
+
+# ---- the decode step (40 x [qkv, o, router, top-8, 256 experts + shared, glue]): two layers of it at real size ------------
+
+@pytest.fixture(scope="module")
+def step_sets(ops):
+    from orin_qwen_lossless_amd import decode_step as D, synth
+
+    seed = [4000]
+
+    def gen(rows, k):
+        seed[0] += 1
+        return synth.weights_torch(rows, k, seed[0], "cuda")
+
+    sets, raw, nbytes = D.make_layer_sets(ops, gen, 2, True)
+    for enc_set, raw_set in zip(sets, raw):
+        for name in ("qkv", "o"):
+            assert ops.roundtrip_equal(enc_set[name], raw_set[name])
+    # the layouts the policy gives the step's matrices: short wave64 units for the dense ones, the 4-bit code for the
+    # router, 32 x 256 tiles for the stacked experts
+    m = {k: (v.meta.format, v.meta.R, v.meta.wave64) for k, v in sets[0].items()}
+    assert m == {"qkv": (3, 2, True), "o": (3, 1, True), "router": (1, 0, False), "gate": (3, 32, True), "up": (3, 32, True), "down": (3, 32, True)}
+    return sets, raw, nbytes
+
+
+def rn(t):
+    """Round an FP64 tensor to BF16 and back (the roundings the step makes between its launches)."""
+    return t.float().to(torch.bfloat16).double()
+
+
+def rms(t):
+    return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + 1e-6)
+
+
+@pytest.mark.parametrize("T", [1, 4])
+def test_decode_step_two_layers_as_one_graph(ops, step_sets, T):
+    """Two layers of the decode step at their real size (8 launches each) captured as one HIP graph: every replay on new
+    activations equals the eager step bit for bit; and one layer against an FP64 evaluation on the exact weights that
+    rounds where the step rounds (BF16 between the launches), with the experts the step's router picked."""
+    from orin_qwen_lossless_amd import decode_step as D, synth
+
+    sets, raw, _ = step_sets
+    step = D.Bf16nStep(ops, sets, None, 2, T)
+    hs = [synth.activations_torch(T, D.K_MODEL, 4100 + i, "cuda") for i in range(3)]
+    hbuf = hs[0].clone()
+    graph, out = D.capture(step, hbuf)
+    for rep in range(3):
+        hbuf.copy_(hs[rep])
+        want = step(hbuf).clone()
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep
+    # one layer against FP64
+    w, r = sets[0], raw[0]
+    h = hs[1]
+    x1 = ops.add_rmsnorm(h)
+    x1n, hn = step.layer(w, h, x1)
+    wts, ids = step.routing
+    W = {k: v.double() for k, v in r.items() if k in ("qkv", "o", "router")}
+    hd = h.double()
+    x1r = rn(rms(hd))
+    assert torch.equal(x1.double(), x1r) or bool(((x1.double() - x1r).abs() <= 2.0 ** -8 * x1r.abs()).all())
+    q = rn(x1.double() @ W["qkv"].t())
+    o = rn(q[:, :D.ATT] @ W["o"].t())
+    s = hd + o
+    h2, x2 = rn(s), rn(rms(s))
+    logits = x2 @ W["router"].t()
+    top = torch.topk(logits, D.TOPK, dim=-1)
+    for t in range(T):  # the step's experts are the FP64 top-8 (margins in random data are far above the rounding)
+        assert set(ids[t, :D.TOPK].tolist()) == set(top.indices[t].tolist()), t
+    assert bool((ids[:, D.TOPK] == D.E).all()) and bool((wts[:, D.TOPK] == 1.0).all())
+    comb = torch.zeros((T, D.K_MODEL), dtype=torch.float64, device="cuda")
+    for t in range(T):
+        for k in range(D.TOPK + 1):
+            e = int(ids[t, k])
+            g = r["gate"][e * D.N_MID:(e + 1) * D.N_MID].double() @ x2[t]
+            u = r["up"][e * D.N_MID:(e + 1) * D.N_MID].double() @ x2[t]
+            hid = (g / (1.0 + torch.exp(-g)) * u).float().double()       # the hidden activations stay FP32 in the GEMV path
+            comb[t] += float(wts[t, k]) * (r["down"][e * D.K_MODEL:(e + 1) * D.K_MODEL].double() @ hid)
+    s2 = h2 + comb
+    href, xref = rn(s2), rn(rms(s2))
+    scale = float(href.abs().max())
+    assert bool(((hn.double() - href).abs() <= 2.0 ** -6 * href.abs() + 2e-3 * scale).all())
+    assert bool(((x1n.double() - xref).abs() <= 2.0 ** -6 * xref.abs() + 2e-3 * float(xref.abs().max())).all())
