@@ -277,7 +277,8 @@ def test_prefill_at_the_benchmark_token_counts(ops, oracle, experts, T):
     """Batched MoE prefill of the 256-expert layer at 2048 and 8192 tokens: routing lists equal to the oracle's, and
     sampled (token, slot) outputs of the fused gate/up product and of the down product against FP64 products of the
     exact weights (1e-3 relative / 1e-5 absolute; and the reassociation bound 1e-5 * sum |w x| where the output is not
-    a product of rounded intermediates)."""
+    a product of rounded intermediates); the whole layer output is bitwise equivariant under a permutation of the
+    tokens."""
     (wg, gate), (wu, up), (wd, down) = experts
     g = torch.Generator(device="cuda").manual_seed(100 + T)
     x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
@@ -311,6 +312,11 @@ def test_prefill_at_the_benchmark_token_counts(ops, oracle, experts, T):
     y = ops.moe_experts(x, gate, up, down, wts, ids, E)
     comb = (ys[tokens].double() * wts[tokens].double().unsqueeze(-1)).sum(1)
     assert torch.all((y[tokens].double() - comb).abs() <= 2.0 ** -8 * comb.abs() + 1e-6)
+    # over the whole output: a token's row does not depend on where the token stands in the batch (its place in the
+    # routing lists and in the 32-token blocks changes, its arithmetic does not)
+    perm = torch.randperm(T, generator=g, device="cuda")
+    y_perm = ops.moe_experts(x[perm].contiguous(), gate, up, down, wts[perm].contiguous(), ids[perm].contiguous(), E)
+    assert torch.equal(y_perm, y[perm])
 
 
 @pytest.fixture(scope="module")
