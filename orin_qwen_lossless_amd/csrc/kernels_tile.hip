@@ -96,6 +96,44 @@ __device__ __forceinline__ void tile_step(tchain_t<D, ONCE> * ch, const uint32_t
     }
 }
 
+// One step of two chains against one block of 32 tokens on the matrix cores.  The two matrix instructions of a
+// 16-column block are issued right behind its decode and run while the next block is decoded (2 to 5 % faster than all
+// four at the end of the step, and some registers fewer: no spills at 128).  b(kb): the B operand of 16-column block kb.
+template <int D, bool ONCE, typename B>
+__device__ __forceinline__ void tile_step_mm(tchain_t<D, ONCE> * ch, const uint32_t * lut, int lut_stride, int s, int lane, B b,
+                                             f32x16_t & acc0, f32x16_t & acc1) {
+    uint32_t smw[2][4];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const uint4 v = ch[k].sm[s % D];
+        smw[k][0] = v.x; smw[k][1] = v.y; smw[k][2] = v.z; smw[k][3] = v.w;
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+        bf16x8_t av[2];
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            uint32_t wq[4];
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                uint32_t e0, e1;
+                ch[k].dec.two(lut + k * lut_stride, e0, e1);
+                wq[2 * j] = merge(spread_lo(smw[k][2 * kb + j]), e0);
+                wq[2 * j + 1] = merge(spread_hi(smw[k][2 * kb + j]), e1);
+            }
+            const u32x4_t v = {wq[0], wq[1], wq[2], wq[3]};
+            av[k] = __builtin_bit_cast(bf16x8_t, v);
+        }
+        const bf16x8_t bv = b(kb);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv, acc1, 0, 0, 0);
+    }
+    ch[0].dec.keep_ahead();
+    ch[1].dec.keep_ahead();
+    ch[0].reload(s, lane);
+    ch[1].reload(s, lane);
+}
+
 // ---------------------------------------------------------------- batched MoE prefill
 
 constexpr int MT_SMALL_PAIRS = 16;  // routed pairs per expert up to which the 32-token shape is used
@@ -300,40 +338,10 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                     for (int s = 0; s < 4; s++) {
                         const uint16_t * bp = bcur + l32 * MT_BSTRIDE + 32 * s + 8 * half;
                         if constexpr (NT == 1) {
-                            // one token block: the two matrix instructions of a 16-column block are issued right behind
-                            // its decode and run while the next block is decoded (2 % faster than all four at the end of
-                            // the step, and seven registers fewer: no spills at 128).  With four token blocks the same
-                            // order measured 3 to 4 % slower than the whole step's instructions together.
-                            uint32_t smw[2][4];
-#pragma unroll
-                            for (int k = 0; k < 2; k++) {
-                                const uint4 v = ch[k].sm[s % S::DEPTH];
-                                smw[k][0] = v.x; smw[k][1] = v.y; smw[k][2] = v.z; smw[k][3] = v.w;
-                            }
-#pragma unroll
-                            for (int kb = 0; kb < 2; kb++) {
-                                bf16x8_t av[2];
-#pragma unroll
-                                for (int k = 0; k < 2; k++) {
-                                    uint32_t wq[4];
-#pragma unroll
-                                    for (int j = 0; j < 2; j++) {
-                                        uint32_t e0, e1;
-                                        ch[k].dec.two(lut + (GLU ? k * LUT_WORDS : 0), e0, e1);
-                                        wq[2 * j] = merge(spread_lo(smw[k][2 * kb + j]), e0);
-                                        wq[2 * j + 1] = merge(spread_hi(smw[k][2 * kb + j]), e1);
-                                    }
-                                    const u32x4_t v = {wq[0], wq[1], wq[2], wq[3]};
-                                    av[k] = __builtin_bit_cast(bf16x8_t, v);
-                                }
-                                const bf16x8_t bv = *(const bf16x8_t *) (bp + 16 * kb);
-                                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv, acc[0][0], 0, 0, 0);
-                                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv, acc[1][0], 0, 0, 0);
-                            }
-                            ch[0].dec.keep_ahead();
-                            ch[1].dec.keep_ahead();
-                            ch[0].reload(s, lane);
-                            ch[1].reload(s, lane);
+                            // (with four token blocks the same order measured 3 to 4 % slower than the whole step's
+                            // matrix instructions together)
+                            tile_step_mm(ch, lut, GLU ? LUT_WORDS : 0, s, lane,
+                                         [&](int kb) { return *(const bf16x8_t *) (bp + 16 * kb); }, acc[0][0], acc[1][0]);
                         } else {
                             uint32_t wp[2][8];
                             tile_step<2, S::DEPTH, NT == 1>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
@@ -497,23 +505,7 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
                     const char * xn = xr + (nq < spw * T_STEPS ? nq : 0) * 64; // after the last step: the first again, unused
                     nb0 = *(const bf16x8_t *) xn;
                     nb1 = *(const bf16x8_t *) (xn + 32);
-                    uint32_t wp[2][8];
-                    tile_step<2, 2, true>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
-                    ch[0].reload(s, lane);
-                    ch[1].reload(s, lane);
-                    bf16x8_t av[2][2]; // [chain][16-column block]
-#pragma unroll
-                    for (int c = 0; c < 2; c++) {
-#pragma unroll
-                        for (int kb = 0; kb < 2; kb++) {
-                            const u32x4_t v = {wp[c][4 * kb], wp[c][4 * kb + 1], wp[c][4 * kb + 2], wp[c][4 * kb + 3]};
-                            av[c][kb] = __builtin_bit_cast(bf16x8_t, v);
-                        }
-                    }
-                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0][0], bv0, acc[0], 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][0], bv0, acc[1], 0, 0, 0);
-                    acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0][1], bv1, acc[0], 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][1], bv1, acc[1], 0, 0, 0);
+                    tile_step_mm(ch, lut, GLU ? LUT_WORDS : 0, s, lane, [&](int kb) { return kb ? bv1 : bv0; }, acc[0], acc[1]);
                 }
                 }
             }
