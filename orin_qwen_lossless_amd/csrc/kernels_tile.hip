@@ -575,8 +575,7 @@ template <> struct x8<bf16_t> {
         const uint32_t xw[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            acc = fmaf(__uint_as_float(wp[i] << 16), __uint_as_float(xw[i] << 16), acc);
-            acc = fmaf(__uint_as_float(wp[i] & 0xFFFF0000u), __uint_as_float(xw[i] & 0xFFFF0000u), acc);
+            acc = dot2_bf16(wp[i], xw[i], acc);
         }
         return acc;
     }
