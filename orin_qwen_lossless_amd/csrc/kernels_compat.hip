@@ -249,7 +249,7 @@ __device__ __forceinline__ void nib_load_chunk(const nib_ptrs & w, int64_t gr, i
 }
 
 // partial dot of a decoded chunk with x.  The four per-position sums are combined as in the reference
-// (kernels.cuh:130-187), then over the 32 lanes; result in every lane of the half-wave.
+// (kernels.cuh:130-187), then over the 32 lanes on the VALU (DPP, no LDS traffic); result in lane 31 of the half-wave.
 __device__ __forceinline__ float nib_dot(const uint32_t (&wp)[8], const float (&xv)[16]) {
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
@@ -259,10 +259,30 @@ __device__ __forceinline__ float nib_dot(const uint32_t (&wp)[8], const float (&
         a2 = fmaf(bf16_bits_to_f32(wp[2 * j + 1] & 0xFFFFu), xv[4 * j + 2], a2);
         a3 = fmaf(__uint_as_float(wp[2 * j + 1] & 0xFFFF0000u), xv[4 * j + 3], a3);
     }
-    return half_wave_sum((a0 + a1) + (a2 + a3));
+    return half_wave_sum_dpp((a0 + a1) + (a2 + a3));
 }
 
-// the exact products of a row's escaped weights, summed over the half-wave
+// the same with BF16 activations left as the 8 pairs they arrive in: a pair of weights meets a pair of activations in
+// one dot2 instruction (8 instructions where conversions and FMAs took 48)
+__device__ __forceinline__ void x_pairs16(const char * x, int col0, uint32_t (&xp)[8]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint2 t = *(const uint2 *) (x + 2 * (col0 + 128 * j));
+        xp[2 * j] = t.x;
+        xp[2 * j + 1] = t.y;
+    }
+}
+__device__ __forceinline__ float nib_dot_pairs(const uint32_t (&wp)[8], const uint32_t (&xp)[8]) {
+    float a01 = 0.f, a23 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        a01 = dot2_bf16(wp[2 * j], xp[2 * j], a01);
+        a23 = dot2_bf16(wp[2 * j + 1], xp[2 * j + 1], a23);
+    }
+    return half_wave_sum_dpp(a01 + a23);
+}
+
+// the exact products of a row's escaped weights, summed over the half-wave (result in lane 31)
 template <typename TX>
 __device__ __forceinline__ float nib_escapes(const nib_ptrs & w, int64_t gr, const char * x, int l32) {
     const uint32_t e0 = w.esc_off[gr], e1 = w.esc_off[gr + 1];
@@ -271,7 +291,7 @@ __device__ __forceinline__ float nib_escapes(const nib_ptrs & w, int64_t gr, con
         const uint32_t rec = w.esc[i];
         acc = fmaf(bf16_bits_to_f32(esc_bits(rec)), x_at<TX>(x, (int) (rec & 0xFFFu)), acc);
     }
-    return e1 > e0 ? half_wave_sum(acc) : 0.f;
+    return e1 > e0 ? half_wave_sum_dpp(acc) : 0.f;
 }
 
 // NIBBLE GEMV; GLU 1: rows_per_matrix = [gate (nrows); up (nrows)] of one matrix; GLU 2: separate gate / up matrices.
@@ -305,16 +325,29 @@ __global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16
         }
 #pragma unroll
         for (int j = 0; j < NC; j++) {
-            float xv[16];
-            x_chunk16<TX>(cv[j].x, c * CHUNK + 4 * l32, xv);
-            float v = nib_dot(wg, xv), vu = GLU ? nib_dot(wu, xv) : 0.f;
+            float v, vu = 0.f;
+            if constexpr (sizeof(TX) == 2) {
+                uint32_t xp[8];
+                x_pairs16(cv[j].x, c * CHUNK + 4 * l32, xp);
+                v = nib_dot_pairs(wg, xp);
+                if (GLU) {
+                    vu = nib_dot_pairs(wu, xp);
+                }
+            } else {
+                float xv[16];
+                x_chunk16<TX>(cv[j].x, c * CHUNK + 4 * l32, xv);
+                v = nib_dot(wg, xv);
+                if (GLU) {
+                    vu = nib_dot(wu, xv);
+                }
+            }
             if (c == 0) {
                 v += nib_escapes<TX>(g, gr, cv[j].x, l32);
                 if (GLU) {
                     vu += nib_escapes<TX>(u, gr, cv[j].x, l32);
                 }
             }
-            if (l32 == 0) {
+            if (l32 == 31) {
                 part[0][j][half] = v;
                 part[1][j][half] = vu;
             }
@@ -391,7 +424,10 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
         const int rpb = HALVES / (int) (w.K / CHUNK);
         // dense batches: four (two) columns share one decode of the matrix once there are columns enough to keep at
         // least four groups of blocks (below that the columns run side by side on the idle CUs, which is faster)
-        const int nc = p.ids ? 1 : ncols >= 16 ? 4 : ncols >= 8 ? 2 : 1, ngroups = (ncols + nc - 1) / nc;
+        const int64_t blocks1 = (p.nrows + rpb - 1) / rpb;
+        const bool fills = blocks1 >= 4 * (int64_t) cus; // one column's blocks keep every CU busy by themselves
+        const int nc = p.ids ? 1 : fills ? (ncols >= 3 ? 4 : ncols == 2 ? 2 : 1) : ncols >= 16 ? 4 : ncols >= 8 ? 2 : 1;
+        const int ngroups = (ncols + nc - 1) / nc;
         const dim3 grid(grid_for((p.nrows + rpb - 1) / rpb * HALVES, ngroups, cus), ngroups);
 #define NIBC(TX, G, N) hipLaunchKernelGGL((k_nib_mmv<TX, G, N>), grid, dim3(NT), 0, stream, w, wu, p, ncols)
 #define NIB(TX, G) do { if (nc == 4) NIBC(TX, G, 4); else if (nc == 2) NIBC(TX, G, 2); else NIBC(TX, G, 1); } while (0)

@@ -48,7 +48,8 @@ bool reaches(int64_t rows, int64_t K, int64_t n, int64_t threshold) noexcept {
 // mi355x dense: one wavefront decodes one unit, and 256 CUs hold 4096 wavefronts at once.  A matrix with more rows than
 // that streams: it takes the longest units (16 rows: fewest unit starts, fewest bytes).  A smaller one is a single
 // round of wavefronts whose time is the length of one unit's decode chain, so it takes the shortest units that still
-// fit the round, i.e. the smallest R with rows / R <= 4096 (measured, K = 2048: 5120 rows 7.9 us with R = 2 against
+// fit the round, i.e. the smallest R with rows / R <= 4096 (in hybrid mode the smallest of these units, 4096 weights,
+// give way to the 4-bit code: see choose) (measured, K = 2048: 5120 rows 7.9 us with R = 2 against
 // 9.2 with R = 4 and 8.9 with R = 1; 2048 x 4096: 6.7 us with R = 1 against 7.7 with R = 2), at 6 % more bytes per
 // halving.  Units of at least 4096 weights: every unit ends with about 512 bytes of stream words that were requested
 // and never used, one bit per weight at that size (units of 2048 weights compress to 0.82 of BF16 instead of 0.70-0.74).
@@ -115,6 +116,16 @@ bool choose(int64_t rows, int64_t K, int64_t n, int engine, int mode, int64_t de
             return true;
         } else {
             R = mi355x_dense_unit_rows(rows, K);
+            if (mode == 0 && (int64_t) R * K <= 4096 && !reaches(rows, K, 1, dense_min + dense_min / 2)) {
+                // a matrix up to half as large again as the dense minimum that fits one round of wavefronts only in
+                // units of 4096 weights: such units compress to 0.74 of BF16 (a quarter of their stream is the three
+                // start words per lane), the 4-bit code to 0.75, and its GEMV has no decode chain (5120 x 2048 from
+                // HBM: 7.3 us against 8.9, 12.7 against 12.6 at four tokens; a 40-layer decode step with qkv and o this
+                // way: 55.1 us per layer against 59.7 at one token, 100.7 against 103.5 at four).  Twice the dense
+                // minimum is too large for it: 8192 x 2048 takes 10.6 against 10.2 us, 17.4 against 13.5 at four tokens.
+                out = {FMT_NIBBLE, 0, false, false, false};
+                return true;
+            }
         }
         // the wave64 layout where the fused GEMV has an instance (K in {512, 1024, 2048, 4096}, units of whole loop
         // bodies); it is row-major: the batched kernel decodes whole rows per step and needs no chunk-major order.

@@ -29,7 +29,7 @@ struct tensor {
 
 int main() {
     namespace ad = bf16n::adapter;
-    tensor ts[3] = {{"output.weight", 4096, 2048, 1, {}}, {"blk.0.ffn_gate_exps.weight", 64, 2048, 8, {}}, {"blk.0.ffn_down_shexp.weight", 2048, 512, 1, {}}};
+    tensor ts[3] = {{"output.weight", 8192, 2048, 1, {}}, {"blk.0.ffn_gate_exps.weight", 64, 2048, 8, {}}, {"blk.0.ffn_down_shexp.weight", 2048, 512, 1, {}}};
     int owner_a = 0, owner_b = 0; // two "buffers"
     for (auto & t : ts) {
         t.host.resize(t.rows_per_matrix * t.n * t.K);

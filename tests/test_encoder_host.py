@@ -151,7 +151,9 @@ def test_policy_contract_cases():
     assert c(16388, 512, 1, "vllm")[1] == 2 and c(18436, 512, 1, "vllm")[1] == 2 and c(20484, 512, 1, "vllm")[1] == 4
     for engine in ("llama", "vllm", "mi355x"):
         for rows in (16383, 16384, 16385):
-            assert c(rows, 512, 1, engine)[0] == (NIB if rows < 16384 else HP)
+            # (mi355x keeps the 4-bit code beyond the dense minimum where its units would be 4096 weights)
+            assert c(rows, 512, 1, engine)[0] == (NIB if rows < 16384 or engine == "mi355x" else HP)
+            assert c(rows, 512, 1, engine, "huffman")[0] == HP
         assert c(512, 2048, 2, engine, "nibble", 0, True)[0] == NIB
         for K in (-1, 0, 1, 256, 511, 513, 1000, 4095, 4097, 4608):
             assert c(2048, K, 1, engine) is None and c(2048, K, 2, engine) is None
@@ -167,13 +169,21 @@ def test_policy_mi355x():
     # the benchmark shapes: wave64 row-major units; 16 rows for a matrix that streams (more than 4096 units), the
     # shortest units that fit one round of 4096 wavefronts for a smaller one
     assert ops.choose(248320, 2048) == (HP, 16, False, False, True)
-    assert ops.choose(5120, 2048) == (HP, 2, False, False, True)
-    assert ops.choose(2048, 4096) == (HP, 1, False, False, True)
     assert ops.choose(16384, 2048) == (HP, 4, False, False, True)
     assert ops.choose(65536, 2048) == (HP, 16, False, False, True)
-    assert ops.choose(16384, 512) == (HP, 8, False, False, True)       # units of at least 4096 weights
-    assert ops.choose(4096, 2048) == (HP, 2, False, False, True)
-    assert ops.choose(8192, 1024) == (HP, 4, False, False, True)
+    assert ops.choose(8192, 2048) == (HP, 2, False, False, True) and ops.choose(32768, 512) == (HP, 8, False, False, True)
+    huf = lambda rows, K: ops.choose(rows, K, mode="huffman")  # noqa: E731
+    assert huf(5120, 2048) == (HP, 2, False, False, True)
+    assert huf(2048, 4096) == (HP, 1, False, False, True)
+    assert huf(16384, 512) == (HP, 8, False, False, True)              # units of at least 4096 weights
+    assert huf(4096, 2048) == (HP, 2, False, False, True)
+    assert huf(8192, 1024) == (HP, 4, False, False, True)
+    # ... and in hybrid mode a matrix of less than 1.5 x the dense minimum whose units would be that small (4096 weights
+    # compress no better than the 4-bit code, whose GEMV has no decode chain) takes the 4-bit code
+    for shape in ((5120, 2048), (2048, 4096), (16384, 512), (4096, 2048), (8192, 1024), (6143, 2048)):
+        assert ops.choose(*shape)[0] == NIB and ops.choose(*shape, dense_frag_order=True)[0] == NIB
+    assert ops.choose(6144, 2048)[:2] == (HP, 2) and ops.choose(3072, 4096)[:2] == (HP, 1)
+    assert ops.choose(5120, 2048, dense_min=4 << 20)[:2] == (HP, 2) and ops.choose(5120, 2048, dense_min=0)[:2] == (HP, 2)
     # experts: 32 x 256 tiles in matrix-core operand order where the rows per expert allow it, else units of 4 rows
     assert ops.choose(512, 2048, 256, expert=True) == (HP, 32, False, False, True)
     assert ops.choose(2048, 512, 256, expert=True) == (HP, 32, False, False, True)
@@ -190,7 +200,7 @@ def test_policy_mi355x():
     assert ops.choose(131040, 2048, dense_frag_order=True) == (HP, 16, False, False, True)   # too few rows
     assert ops.choose(248336, 2048, dense_frag_order=True) == (HP, 16, False, False, True)   # not a multiple of 32
     assert ops.choose(248320, 512, dense_frag_order=True) == (HP, 16, False, False, True)    # K too short
-    assert ops.choose(5120, 2048, dense_frag_order=True) == (HP, 2, False, False, True)
+    assert ops.choose(5120, 2048, mode="huffman", dense_frag_order=True) == (HP, 2, False, False, True)
     # shapes without a wave64 GEMV instance keep the reference layouts
     assert ops.choose(16384, 1536) == (HP, 4, False, False, False)
     assert ops.choose(520, 1536, 8, expert=True) == (HP, 8, True, False, False)

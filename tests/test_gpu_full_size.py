@@ -393,18 +393,20 @@ def test_moe_decode_layer_256_experts_as_one_graph(ops, experts, moe_small_parts
         assert torch.all((shared[t].double() - want_sh).abs() <= 2.0 ** -7 * want_sh.abs() + 1e-5), t
 
 
-@pytest.mark.parametrize("name,rows,k,R", [("qkv", 5120, 2048, 2), ("o", 2048, 4096, 1), ("cfg1", 2048, 2048, 2)])
-def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, R):
-    """The per-layer dense projections in the layouts the mi355x policy gives them (short wave64 units), and the
-    2048 x 2048 matrix of the CPU reference configuration, at batch 1 and 4 against the oracle's FP32-accumulated GEMV
-    and its FP64 bound; the decode is bit-exact and the pair table equals the oracle encoder's."""
+@pytest.mark.parametrize("name,rows,k,mode,want", [
+    ("qkv", 5120, 2048, "hybrid", (1, 0, False, False)), ("o", 2048, 4096, "hybrid", (1, 0, False, False)),
+    ("qkv", 5120, 2048, "huffman", (3, 2, False, True)), ("o", 2048, 4096, "huffman", (3, 1, False, True)),
+    ("cfg1", 2048, 2048, "huffman", (3, 2, False, True))])
+def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, mode, want):
+    """The per-layer dense projections in the layouts the mi355x policy gives them (the 4-bit code in hybrid mode, short
+    wave64 units when the Huffman family is asked for), and the 2048 x 2048 matrix of the CPU reference configuration
+    (its configuration names the pair code), at batch 1 and 4 against the oracle's FP32-accumulated GEMV and its FP64
+    bound; the decode is bit-exact and the oracle decodes the encoder's bytes to the same weights."""
     from orin_qwen_lossless_amd import synth
 
     wb = synth.weights(rows, k, 500 + rows % 97)
-    # 2048 x 2048 is below the policy's dense minimum (it would take the 4-bit code); its configuration names the pair
-    # code, so the policy is asked for the Huffman family there
-    fmt, r, cm, _, w64 = ops.choose(rows, k, engine="mi355x", mode="huffman" if name == "cfg1" else "hybrid")
-    assert (fmt, r, cm, w64) == (3, R, False, True)
+    fmt, r, cm, _, w64 = ops.choose(rows, k, engine="mi355x", mode=mode)
+    assert (fmt, r, cm, w64) == want
     plane, aux, _, _ = ops.encode_bits(wb, fmt, r, cm, wave64=w64)
     assert np.array_equal(oracle.decode(plane, aux), wb)
     ta = torch.from_numpy(aux)
@@ -441,10 +443,10 @@ def step_sets(ops):
     for enc_set, raw_set in zip(sets, raw):
         for name in ("qkv", "o"):
             assert ops.roundtrip_equal(enc_set[name], raw_set[name])
-    # the layouts the policy gives the step's matrices: short wave64 units for the dense ones, the 4-bit code for the
-    # router, 32 x 256 tiles for the stacked experts
+    # the layouts the policy gives the step's matrices: the 4-bit code for the dense ones (all below 1.5 x the dense
+    # minimum), 32 x 256 tiles for the stacked experts
     m = {k: (v.meta.format, v.meta.R, v.meta.wave64) for k, v in sets[0].items()}
-    assert m == {"qkv": (3, 2, True), "o": (3, 1, True), "router": (1, 0, False), "gate": (3, 32, True), "up": (3, 32, True), "down": (3, 32, True)}
+    assert m == {"qkv": (1, 0, False), "o": (1, 0, False), "router": (1, 0, False), "gate": (3, 32, True), "up": (3, 32, True), "down": (3, 32, True)}
     return sets, raw, nbytes
 
 
