@@ -14,6 +14,9 @@
 #include "dev_w64.h"
 #include "launchers.h"
 
+#include <algorithm>
+#include <cmath>
+
 #include <stdexcept>
 
 namespace bf16n {
@@ -432,33 +435,34 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
 }
 
 // Few active experts (decode at small batch): a pass over an expert is one decode chain per wavefront, K / 32 steps
-// long, and nothing runs beside it, so the chain is cut instead: WPI = K / 256 wavefronts share a work item (expert,
-// pair of row groups, or gate and up of one group), each decodes one tile per chain (8 steps) against its 256 columns of
-// the activations, read straight from memory (16 bytes per lane and matrix instruction, one step ahead: no staging, no
+// long, and nothing runs beside it, so the chain is cut instead: WPI wavefronts share a work item (expert, pair of row
+// groups, or gate and up of one group), each decodes K / 256 / WPI tiles per chain against its columns of the
+// activations, read straight from memory (16 bytes per lane and matrix instruction, one step ahead: no staging, no
 // barrier inside the chain), and the partial accumulators are added in K order through LDS (the rings, idle by then).
 // Sixteen wavefronts per block: 16 / WPI items.  Passes of 32 tokens; the block runs as many as its busiest item needs.
+// WPI is chosen by the block itself once it has listed the active experts: the most wavefronts per item (the
+// shortest chains) for which every item of the call runs at once.  The host only knows the routed pairs, an upper
+// bound of the active experts that is up to a third too high (tokens share experts), and an item count just above
+// what the GPU holds at once doubles the time (a second round of blocks) where the next split down would not.
 constexpr int KS_WAVES = 16;
 
+struct ks_ctx {
+    uint32_t * lut, * rings; uint16_t * act;
+    int n_items, per_expert, groups, slabs;
+};
+
 template <bool GLU, int WPI>
-__global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight w, const bf16n_weight w_up, const mm_args a, const int spw) {
-    constexpr int NM = GLU ? 2 : 1, IPB = KS_WAVES / WPI, RPW = 16 / WPI; // items per block; accumulator registers a wavefront adds up
-    extern __shared__ __align__(16) uint32_t shm[];
-    uint32_t * lut = shm;
-    uint32_t * rings = shm + NM * LUT_WORDS;
+__device__ __forceinline__ void ks_items(const bf16n_weight & w, const bf16n_weight & w_up, const mm_args & a, const ks_ctx & c) {
+    constexpr int IPB = KS_WAVES / WPI, RPW = 16 / WPI; // items per block; accumulator registers a wavefront adds up
+    uint32_t * lut = c.lut;
+    uint32_t * rings = c.rings;
     float * part = (float *) rings;                           // [wavefront][register][lane], 6 KB apart
-    uint16_t * act = (uint16_t *) (rings + KS_WAVES * 2 * WAVE_LDS_WORDS);
+    uint16_t * act = c.act;
     const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
     const int is = wave / WPI, kw = wave % WPI;               // item of the block, K part
-    stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
-    if (GLU) {
-        stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
-    }
-    const int groups = (int) (a.rows / TILE_R);
-    const int per_expert = GLU ? groups : (groups + 1) / 2;   // items per expert
+    const int groups = c.groups, per_expert = c.per_expert, n_items = c.n_items, spw = c.slabs / WPI;
     const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
     uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-    const int n_items = list_active(act, a, wave, lane, KS_WAVES) * per_expert;
-    __syncthreads();
     for (int base = blockIdx.x * IPB; base < n_items; base += gridDim.x * IPB) {
         int maxn = 0;
 #pragma unroll
@@ -480,10 +484,10 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
             const int tk = tp + l32;
             f32x16_t acc[2];
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
+            for (int m = 0; m < 2; m++) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    acc[c][i] = 0.f;
+                    acc[m][i] = 0.f;
                 }
             }
             if (tp < n) {
@@ -509,39 +513,49 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
                 }
                 }
             }
-            __syncthreads(); // every ring is idle: they hold the partial sums now
             float r[2][RPW];
+            if constexpr (WPI == 1) { // a wavefront has the whole sums
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
+                for (int m = 0; m < 2; m++) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    part[(wave * (2 * WAVE_LDS_WORDS)) + i * 64 + lane] = acc[c][i];
-                }
-                __syncthreads();
-#pragma unroll
-                for (int q = 0; q < RPW; q++) {
-                    float sum = 0.f;
-#pragma unroll
-                    for (int k = 0; k < WPI; k++) {
-                        sum += part[((is * WPI + k) * (2 * WAVE_LDS_WORDS)) + (kw * RPW + q) * 64 + lane];
+                    for (int q = 0; q < RPW; q++) {
+                        r[m][q] = acc[m][q];
                     }
-                    r[c][q] = sum;
                 }
-                __syncthreads();
+            } else {
+                __syncthreads(); // every ring is idle: they hold the partial sums now
+#pragma unroll
+                for (int m = 0; m < 2; m++) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        part[(wave * (2 * WAVE_LDS_WORDS)) + i * 64 + lane] = acc[m][i];
+                    }
+                    __syncthreads();
+#pragma unroll
+                    for (int q = 0; q < RPW; q++) {
+                        float sum = 0.f;
+#pragma unroll
+                        for (int k = 0; k < WPI; k++) {
+                            sum += part[((is * WPI + k) * (2 * WAVE_LDS_WORDS)) + (kw * RPW + q) * 64 + lane];
+                        }
+                        r[m][q] = sum;
+                    }
+                    __syncthreads();
+                }
             }
             // accumulator element i of a lane: row 8 (i / 4) + 4 (lane / 32) + i % 4 of the group, token lane % 32
             if (tk < n) {
                 const int64_t col = (int64_t) a.ids_dst[j0 + tk] * a.dst_col;
 #pragma unroll
-                for (int c = 0; c < (GLU ? 1 : 2); c++) {
-                    if (c == 1 && !has1) {
+                for (int m = 0; m < (GLU ? 1 : 2); m++) {
+                    if (m == 1 && !has1) {
                         continue;
                     }
 #pragma unroll
                     for (int q = 0; q < RPW; q++) {
                         const int i = kw * RPW + q;
-                        const int64_t o = col + (int64_t) (c ? g1 : g0) * TILE_R + 8 * (i >> 2) + 4 * half + (i & 3);
-                        const float v = GLU ? r[1][q] * silu(r[0][q]) : r[c][q];
+                        const int64_t o = col + (int64_t) (m ? g1 : g0) * TILE_R + 8 * (i >> 2) + 4 * half + (i & 3);
+                        const float v = GLU ? r[1][q] * silu(r[0][q]) : r[m][q];
                         if (a.dst_bf16) {
                             ((uint16_t *) a.dst)[o] = f32_to_bf16_rne(v);
                         } else {
@@ -551,6 +565,46 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
                 }
             }
         }
+    }
+}
+
+template <bool GLU>
+__global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+    constexpr int NM = GLU ? 2 : 1;
+    extern __shared__ __align__(16) uint32_t shm[];
+    ks_ctx c;
+    c.lut = shm;
+    c.rings = shm + NM * LUT_WORDS;
+    c.act = (uint16_t *) (c.rings + KS_WAVES * 2 * WAVE_LDS_WORDS);
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6);
+    // the tables are requested first (one 16-byte load per thread and table) and stored once the block knows that it
+    // has work: their way from memory overlaps the listing of the active experts
+    static_assert(LUT_WORDS / 4 == KS_WAVES * 64, "one uint4 of a table per thread");
+    const uint4 t0 = ((const uint4 *) (w.aux + w.off_a))[threadIdx.x];
+    const uint4 t1 = GLU ? ((const uint4 *) (w_up.aux + w_up.off_a))[threadIdx.x] : make_uint4(0, 0, 0, 0);
+    c.groups = (int) (a.rows / TILE_R);
+    c.per_expert = GLU ? c.groups : (c.groups + 1) / 2;       // items per expert
+    c.slabs = (int) (w.K / TILE_K);
+    c.n_items = list_active(c.act, a, wave, lane, KS_WAVES) * c.per_expert;
+    // the most wavefronts per item for which the launch's blocks hold every item at once
+    int wpi = KS_WAVES;
+    while (wpi > 1 && (c.slabs % wpi != 0 || (int64_t) c.n_items * wpi > (int64_t) gridDim.x * KS_WAVES)) {
+        wpi >>= 1;
+    }
+    if ((int64_t) blockIdx.x * (KS_WAVES / wpi) >= c.n_items) {
+        return; // (the same in every thread of the block)
+    }
+    ((uint4 *) c.lut)[threadIdx.x] = t0;
+    if (GLU) {
+        ((uint4 *) (c.lut + LUT_WORDS))[threadIdx.x] = t1;
+    }
+    __syncthreads();
+    switch (wpi) {
+        case 16: ks_items<GLU, 16>(w, w_up, a, c); break;
+        case 8: ks_items<GLU, 8>(w, w_up, a, c); break;
+        case 4: ks_items<GLU, 4>(w, w_up, a, c); break;
+        case 2: ks_items<GLU, 2>(w, w_up, a, c); break;
+        default: ks_items<GLU, 1>(w, w_up, a, c); break;
     }
 }
 
@@ -764,8 +818,8 @@ bool is_tile_layout(const bf16n_weight & w) {
 template <bool GLU, int NT, int W> void mt_attr() {
     (void) hipFuncSetAttribute((const void *) k_mm_tile<GLU, NT, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<NT, W>(GLU));
 }
-template <bool GLU, int WPI> void ks_attr() {
-    (void) hipFuncSetAttribute((const void *) k_mm_tile_ks<GLU, WPI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ks_shm(GLU));
+template <bool GLU> void ks_attr() {
+    (void) hipFuncSetAttribute((const void *) k_mm_tile_ks<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ks_shm(GLU));
 }
 
 void tile_init() {
@@ -774,8 +828,7 @@ void tile_init() {
     mt_attr<true, 1, 16>();
     mt_attr<false, 1, 16>();
     (void) hipFuncSetAttribute((const void *) k_mm_tile<false, 1, 16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<1, 16>(false));
-    ks_attr<true, 2>(); ks_attr<false, 2>(); ks_attr<true, 4>(); ks_attr<false, 4>();
-    ks_attr<true, 8>(); ks_attr<false, 8>(); ks_attr<true, 16>(); ks_attr<false, 16>();
+    ks_attr<true>(); ks_attr<false>();
 }
 
 template <int W> int64_t mt_items(const mm_args & a, bool glu) {
@@ -795,42 +848,22 @@ void mt_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & 
     }
 }
 
-template <int WPI>
-void ks_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int64_t blocks, int spw, hipStream_t stream) {
-    if (up) {
-        hipLaunchKernelGGL((k_mm_tile_ks<true, WPI>), dim3((unsigned) blocks), dim3(KS_WAVES * 64), ks_shm(true), stream, w, *up, a, spw);
-    } else {
-        hipLaunchKernelGGL((k_mm_tile_ks<false, WPI>), dim3((unsigned) blocks), dim3(KS_WAVES * 64), ks_shm(false), stream, w, w, a, spw);
-    }
-}
-
-// passes of 32 tokens: whole experts (or 32 row groups) per block of sixteen wavefronts, unless the experts that can be
-// active (one per routed pair at most) are so few that K can be split over 2 to 16 wavefronts per item and the blocks
-// still fit the GPU (nearly) at once: the most wavefronts per item (the shortest chains) for which they do.  The bound
-// counts every routed pair as an expert of its own, which is some 15 % high at these sizes: 1.25 x the CUs measured
-// faster than whole experts per block (92 against 122 us at 20 tokens), 1.5 x slower (147 against 120 at 24).
+// Passes of 32 tokens.  While the experts that can be active are few enough that K may be split over wavefronts
+// (k_mm_tile_ks: one block per CU, the split chosen on the device from the experts that are active), that kernel; else
+// whole experts (or 32 row groups) per block of sixteen wavefronts with the activations staged in LDS.  The estimate of
+// the active experts is the expectation for uniform routing; when it is too low the K-split kernel runs unsplit, which
+// measured up to a quarter behind the staged kernel at 32 tokens, and never runs a second round of blocks.
 void mt_launch_small(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int64_t n_pairs, int cus, hipStream_t stream) {
-    const int64_t active = n_pairs < a.n_experts ? n_pairs : a.n_experts;
     const int slabs = (int) (w.K / TILE_K), groups = (int) (a.rows / TILE_R);
-    const int64_t items = active * (up ? groups : (groups + 1) / 2);
-    int wpi = 0;
-    if (a.bounds && a.n_experts <= MT_MAX_LISTED) {
-        for (int c = KS_WAVES; c >= 2; c /= 2) {
-            if (slabs % c == 0 && (items * c + KS_WAVES - 1) / KS_WAVES <= cus + cus / 4) {
-                wpi = c;
-                break;
-            }
-        }
-    }
-    if (wpi) {
-        int64_t blocks = (items * wpi + KS_WAVES - 1) / KS_WAVES;
-        blocks = blocks > 0 ? blocks : 1;
-        const int spw = slabs / wpi;
-        switch (wpi) {
-            case 2: ks_launch<2>(w, up, a, blocks, spw, stream); break;
-            case 4: ks_launch<4>(w, up, a, blocks, spw, stream); break;
-            case 8: ks_launch<8>(w, up, a, blocks, spw, stream); break;
-            default: ks_launch<16>(w, up, a, blocks, spw, stream); break;
+    const double e = (double) a.n_experts;
+    const double active = std::min((double) n_pairs, e * (1.0 - std::pow(1.0 - 1.0 / e, (double) n_pairs)));
+    const double items = active * (up ? groups : (groups + 1) / 2);
+    const bool split = a.bounds && a.n_experts <= MT_MAX_LISTED && slabs % 2 == 0 && items * 2 <= (double) cus * KS_WAVES;
+    if (split) {
+        if (up) {
+            hipLaunchKernelGGL((k_mm_tile_ks<true>), dim3((unsigned) cus), dim3(KS_WAVES * 64), ks_shm(true), stream, w, *up, a);
+        } else {
+            hipLaunchKernelGGL((k_mm_tile_ks<false>), dim3((unsigned) cus), dim3(KS_WAVES * 64), ks_shm(false), stream, w, w, a);
         }
     } else {
         mt_launch<1, 16>(w, up, a, cus, stream);

@@ -25,8 +25,10 @@ FLAG_CHUNK_MAJOR, FLAG_FRAG_ORDER, FLAG_WAVE64 = 1, 2, 4
 # up to 8 tokens through the GEMV kernels, more through the batched MoE kernel / dequant + GEMM
 # (engines/vllm/vllm_bf16n/ops.py:25-27, core/torch/torch_bindings.cpp:195)
 GEMV_MAX_TOKENS = 8
-# moe_experts: expert GEMVs up to this many routed (token, slot) pairs per expert (tile layout, other layouts)
-MOE_GEMV_PAIRS_PER_EXPERT = (0.2, 0.7)
+# moe_experts: expert GEMVs up to this many routed (token, slot) pairs per expert (tile layout, other layouts), and in
+# the tile layout up to this many pairs whatever the number of experts
+MOE_GEMV_PAIRS_PER_EXPERT = (0.14, 0.7)
+MOE_GEMV_MIN_PAIRS = 24
 DEQUANT_CHUNK_BYTES = 64 << 20
 
 ENGINES = {"llama": 0, "vllm": 1, "mi355x": 2}
@@ -636,16 +638,20 @@ def moe_experts_rows(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, to
 
     The reference switches from expert GEMVs to the batched kernels above 8 tokens.  Here the GEMVs stay ahead only
     while the routed pairs are few against the experts (each pair decodes one expert matrix in its own GEMV column; the
-    batched kernel decodes every active expert once).  Tile layout: up to 0.2 pairs per expert (6 tokens for top-8 of
-    256; measured 57 / 97 us GEMV against 64 / 83 us batched at 4 / 8 tokens), its batched kernel splits K over
-    wavefronts while few experts are active; other layouts: 0.7 and never below the reference's 8 tokens."""
+    batched kernel decodes every active expert once).  Tile layout: up to 0.14 pairs per expert and never below 24 pairs
+    (top-8 of 256: 4 tokens; with a ninth slot that every token shares, 3; measured, GEMVs against batched kernels, at
+    4 / 5 / 6 tokens: 50 / 64 / 68 against 55 / 67 / 64 us with 8 slots, 61 / 67 / 80 against 57 / 69 / 67 us with 9),
+    its batched kernel splits K over wavefronts while few experts are active; other layouts: 0.7 pairs per expert and
+    never below the reference's 8 tokens."""
     n_tokens, n_used = x.shape[0], max(int(topk_ids.shape[1]), 1)
     n_mid, n_out = gate.meta.rows // n_experts, down.meta.rows // n_experts
     x = x.contiguous()
     tiles = all(m.meta.wave64 and m.meta.R == 32 for m in (gate, up, down))
-    per_expert = MOE_GEMV_PAIRS_PER_EXPERT[0 if tiles else 1]
-    gemv_tokens = max(4 if tiles else GEMV_MAX_TOKENS, int(per_expert * n_experts) // n_used)
-    if n_tokens > gemv_tokens and mm_ids_supported(gate, up) and mm_ids_supported(down):
+    if tiles:
+        gemv = n_tokens * n_used <= max(MOE_GEMV_MIN_PAIRS, MOE_GEMV_PAIRS_PER_EXPERT[0] * n_experts)
+    else:
+        gemv = n_tokens <= max(GEMV_MAX_TOKENS, int(MOE_GEMV_PAIRS_PER_EXPERT[1] * n_experts) // n_used)
+    if not gemv and mm_ids_supported(gate, up) and mm_ids_supported(down):
         return _experts_batched(x, gate, up, down, topk_ids, n_experts)
     # one GEMV column per (token, slot), FP32 between the products
     return mmv(_experts_gemv_hidden(x, gate, up, topk_ids, n_mid), down, topk_ids, n_out)

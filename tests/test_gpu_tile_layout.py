@@ -241,9 +241,10 @@ def test_moe_experts_in_both_token_regimes(ops, T):
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
 
 
-@pytest.mark.parametrize("T", [11, 12, 13, 30])
+@pytest.mark.parametrize("T", [7, 8, 9, 30])
 def test_moe_experts_path_switch_by_routed_pairs_per_expert(ops, T, monkeypatch):
-    # 240 experts, top-4: expert GEMVs up to 0.2 * 240 / 4 = 12 tokens, the batched kernels above; both within tolerance
+    # 240 experts, top-4: expert GEMVs up to 0.14 * 240 = 33.6 routed pairs (8 tokens), the batched kernels above; both
+    # within tolerance
     E, k, Kd, N = 240, 4, 512, 512
     gate = enc(ops, synth.weights(E * N, Kd, 81), HP, 32, False, True)
     up = enc(ops, synth.weights(E * N, Kd, 82), HP, 32, False, True)
@@ -256,7 +257,7 @@ def test_moe_experts_path_switch_by_routed_pairs_per_expert(ops, T, monkeypatch)
     wts = torch.softmax(torch.randn((T, k), generator=torch.Generator().manual_seed(T)), dim=-1).cuda()
     x = tbf16(synth.activations(T, Kd, 84))
     got = ops.moe_experts(x, gate, up, down, wts, ids, E).float().cpu().numpy()
-    assert len(batched_calls) == (0 if T <= 12 else 2)
+    assert len(batched_calls) == (0 if T <= 8 else 2)
     ref = moe_layer_exact(ops, x, gate, up, down, wts, ids, E).float().cpu().numpy()
     scale = np.abs(ref).max()
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * scale)
