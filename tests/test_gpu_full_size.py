@@ -257,6 +257,37 @@ def test_full_size_batched_moe_against_exact_weights_and_the_gemv_path(ops, expe
     assert torch.equal(ys2, ys * 2)
 
 
+@pytest.mark.parametrize("T,distinct", [(1, False), (2, False), (4, False), (8, False), (16, False), (20, True)])
+def test_batched_kernels_at_every_split_of_k(ops, experts, T, distinct):
+    """Few tokens through the batched kernels: the kernel that splits K over wavefronts picks its split on the device
+    from the experts that are active — 8 wavefronts per item for 8 to 32 experts (an expert's K is 8 tiles), 4 up to
+    64, 2 up to 128, and whole chains when the routing has more active experts than the host's estimate (20 tokens whose
+    160 experts are all different: the estimate for uniform routing is 119).  Every (token, slot) output of the fused
+    gate/up product and of the down product against FP64 products of the exact weights."""
+    (wg, gate), (wu, up), (wd, down) = experts
+    g = torch.Generator(device="cuda").manual_seed(300 + T)
+    x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
+    if distinct:
+        ids = torch.randperm(E, generator=g, device="cuda")[: T * TOPK].to(torch.int32).view(T, TOPK).contiguous()
+    else:
+        _, ids = ops.router_topk(torch.randn((T, E), generator=g, device="cuda"), TOPK)
+    src1, dst, bounds = ops.mm_ids_route(ids, E, False)
+    a = ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.float32, routes=(src1, dst, bounds))
+    a16 = a.to(torch.bfloat16)
+    ys = ops.moe_mm_ids(a16, ids, down, E, routes=(dst, dst, bounds))
+    for t in range(T):
+        xe = x[t].double()
+        for s in range(TOPK):
+            e = int(ids[t, s])
+            gg, uu = wg[e * N:(e + 1) * N].double() @ xe, wu[e * N:(e + 1) * N].double() @ xe
+            want = uu * silu64(gg)
+            assert torch.all((a[t, s].double() - want).abs() <= 1e-3 * want.abs() + 1e-5), (t, s)
+            h = a16[t, s].double()
+            wde = wd[e * K:(e + 1) * K].double()
+            err = (ys[t, s].double() - wde @ h).abs()
+            assert torch.all(err <= 1e-5 * (wde.abs() @ h.abs())), (t, s)
+
+
 # ---- the benchmark configurations at their stated sizes ---------------------------------------------------------------
 
 def upload_policy(ops, w, n_matrices=1):
