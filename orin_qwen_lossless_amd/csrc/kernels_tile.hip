@@ -463,18 +463,34 @@ __device__ __forceinline__ void ks_items(const bf16n_weight & w, const bf16n_wei
     const int groups = c.groups, per_expert = c.per_expert, n_items = c.n_items, spw = c.slabs / WPI;
     const w64_ptrs q0 = w64p(w), q1 = w64p(GLU ? w_up : w);
     uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
-    for (int base = blockIdx.x * IPB; base < n_items; base += gridDim.x * IPB) {
+    // When the launch holds every item at once (always, unless WPI is 1) the items are dealt out evenly over all
+    // blocks, fewer than IPB to a block if need be: a block's wavefronts share its SIMDs, and the decode is VALU work
+    // (33 active experts: 2 or 3 items on each of 256 CUs instead of 4 on 132 of them).  Else IPB per block, in rounds.
+    const int64_t per_round = (int64_t) gridDim.x * IPB;
+    const bool dealt = n_items <= per_round - gridDim.x; // (only where that lowers the most items of a block)
+    for (int64_t r0 = 0; r0 < n_items; r0 += per_round) {
+        int base, cnt;
+        if (dealt) {
+            base = (int) ((int64_t) blockIdx.x * n_items / gridDim.x);
+            cnt = (int) ((int64_t) (blockIdx.x + 1) * n_items / gridDim.x) - base;
+        } else {
+            base = (int) (r0 + (int64_t) blockIdx.x * IPB);
+            cnt = n_items - base < IPB ? n_items - base : IPB;
+        }
+        if (cnt <= 0) { // (the same in every thread of the block)
+            continue;
+        }
         int maxn = 0;
 #pragma unroll
         for (int k = 0; k < IPB; k++) {
-            if (base + k < n_items) {
+            if (k < cnt) {
                 const int ek = (int) uniform(act[(base + k) / per_expert]);
                 const int nk = a.bounds[ek + 1] - a.bounds[ek];
                 maxn = nk > maxn ? nk : maxn;
             }
         }
         const int item = base + is;
-        const bool valid = item < n_items;
+        const bool valid = is < cnt;
         const int e = valid ? (int) uniform(act[item / per_expert]) : 0, p = valid ? item % per_expert : 0;
         const int j0 = a.bounds[e], n = valid ? a.bounds[e + 1] - j0 : 0;
         const int g0 = GLU ? p : 2 * p;
@@ -591,8 +607,10 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     while (wpi > 1 && (c.slabs % wpi != 0 || (int64_t) c.n_items * wpi > (int64_t) gridDim.x * KS_WAVES)) {
         wpi >>= 1;
     }
-    if ((int64_t) blockIdx.x * (KS_WAVES / wpi) >= c.n_items) {
-        return; // (the same in every thread of the block)
+    const int ipb = KS_WAVES / wpi;
+    if (c.n_items <= (int) gridDim.x * (ipb - 1) ? (int64_t) (blockIdx.x + 1) * c.n_items / gridDim.x == (int64_t) blockIdx.x * c.n_items / gridDim.x
+                                                  : (int64_t) blockIdx.x * ipb >= c.n_items) {
+        return; // no item for this block (the same in every thread of the block)
     }
     ((uint4 *) c.lut)[threadIdx.x] = t0;
     if (GLU) {
