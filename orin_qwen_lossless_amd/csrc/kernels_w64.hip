@@ -75,16 +75,21 @@ template <int C> struct geom {
 };
 
 // One decode chain of a wave: a contiguous range of units with its own stream ring, plane pointer and row counter.
-template <int NB>
+// HINT: as in w64_dec_t, for the plane bytes and the stream blocks alike.
+template <int NB, int HINT = -1>
 struct chain {
-    w64_dec dec;
+    w64_dec_t<HINT> dec;
     range_t plane;         // the plane bytes of the chain's units
     uint32_t off;          // byte offset of this lane's 16 bytes in the next step to load
     uint4 sm[NB];          // plane bytes of the body's steps
     int64_t row;           // output row of the next body, relative to the product
     bool once;             // the launch reads the plane bytes once (see load_once)
     __device__ __forceinline__ uint4 load_step(int) const { // past the end of the chain: dropped, reads as zeros
-        return range_load16(plane, off, once);
+        if constexpr (HINT < 0) {
+            return range_load16(plane, off, once);
+        } else {
+            return range_load16<HINT == 1>(plane, off);
+        }
     }
     // first / end: the stream words of units [gu0, gu0 + n_units) (unit bases, read by the caller ahead of time)
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t gu0, int64_t n_units, int64_t row0, int R, int K,
@@ -111,8 +116,8 @@ struct chain {
 // other one issues.
 // GLU (N = 2, NC = 1): chain 0 decodes a unit of the gate matrix, chain 1 the same unit of the up matrix (its table
 // LUT_WORDS behind the first), and the rows come out as silu(gate x) * (up x).
-template <typename TX, int C, int NC, int N, bool GLU = false>
-__device__ __forceinline__ void unit_pass(chain<geom<C>::NB> (&ch)[2], const uint32_t * lut, const xchunk<TX> (&xr)[NC][geom<C>::XS],
+template <typename TX, int C, int NC, int N, bool GLU = false, int HINT = -1>
+__device__ __forceinline__ void unit_pass(chain<geom<C>::NB, HINT> (&ch)[2], const uint32_t * lut, const xchunk<TX> (&xr)[NC][geom<C>::XS],
                                           const cols & p, const col_view & cv, int R, int lane) {
     using G = geom<C>;
     const int l32 = lane & 31, half = lane >> 5;
@@ -232,7 +237,7 @@ constexpr int x_regs() { return NC * geom<C>::XS * (sizeof(TX) == 2 ? 8 : 16); }
 // eight chunks per row (they spilled at 128); these run in blocks of at most eight wavefronts
 constexpr bool wide_regs(int xr, bool x_bf16, int C) { return xr > 64 || (xr == 64 && (!x_bf16 || C == 8)); }
 
-template <typename TX, int C, int NC, int NCH>
+template <typename TX, int C, int NC, int NCH, int HINT = -1>
 __global__ void __launch_bounds__(wide_regs(x_regs<TX, C, NC>(), sizeof(TX) == 2, C) ? 512 : 1024) k_w64_mmv(const bf16n_weight w, const cols p, int units_per_wave) {
     using G = geom<C>;
     constexpr int K = C * CHUNK;
@@ -265,7 +270,7 @@ __global__ void __launch_bounds__(wide_regs(x_regs<TX, C, NC>(), sizeof(TX) == 2
     if (!live) {
         return;
     }
-    chain<G::NB> ch[2];
+    chain<G::NB, HINT> ch[2];
     uint32_t * ring = rings + wave * (NCH * WAVE_LDS_WORDS);
     ch[0].start(ring, q, gu0, nA, u_begin * R, R, K, lane, b0, b1, p.plane_once, p.stream_once);
     if (NCH == 2 && nB > 0) {
@@ -273,9 +278,9 @@ __global__ void __launch_bounds__(wide_regs(x_regs<TX, C, NC>(), sizeof(TX) == 2
     }
     for (int64_t i = 0; i < nA; i++) {
         if (NCH == 2 && i < nB) {
-            unit_pass<TX, C, NC, 2>(ch, lut, xr, p, cv, R, lane);
+            unit_pass<TX, C, NC, 2, false, HINT>(ch, lut, xr, p, cv, R, lane);
         } else {
-            unit_pass<TX, C, NC, 1>(ch, lut, xr, p, cv, R, lane);
+            unit_pass<TX, C, NC, 1, false, HINT>(ch, lut, xr, p, cv, R, lane);
         }
     }
 }
@@ -435,15 +440,28 @@ constexpr int max_group() {
 template <typename TX, int C, int NC>
 constexpr bool two_chains() { return x_regs<TX, C, NC>() <= 16; }
 
-template <typename TX, int C, int NC>
-void mmv_launch(dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
+// the load policy of plane and stream as a compile-time choice of the instance
+template <typename TX, int C, int NC, int HINT>
+void mmv_launch_hint(dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
     if constexpr (two_chains<TX, C, NC>()) {
         if (upw >= 2) {
-            hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 2>), grid, dim3(nt), w64_shm(2 * wpb), stream, w, p, upw);
+            hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 2, HINT>), grid, dim3(nt), w64_shm(2 * wpb), stream, w, p, upw);
             return;
         }
     }
-    hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 1>), grid, dim3(nt), w64_shm(wpb), stream, w, p, upw);
+    hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 1, HINT>), grid, dim3(nt), w64_shm(wpb), stream, w, p, upw);
+}
+template <typename TX, int C, int NC>
+void mmv_launch(dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
+    if (p.plane_once == p.stream_once) { // (what launch_w64_mmv sets; the run-time form stays for other callers)
+        if (p.plane_once) {
+            mmv_launch_hint<TX, C, NC, 1>(grid, nt, wpb, stream, w, p, upw);
+        } else {
+            mmv_launch_hint<TX, C, NC, 0>(grid, nt, wpb, stream, w, p, upw);
+        }
+        return;
+    }
+    mmv_launch_hint<TX, C, NC, -1>(grid, nt, wpb, stream, w, p, upw);
 }
 
 template <typename TX, int C>
