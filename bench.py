@@ -480,7 +480,7 @@ def main() -> None:
         "roofline": {"bound": "hbm", "achieved": round(algo_bytes / (kern_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": traffic, "traffic_source": TRAFFIC_PROFILE if traffic is not None else None,
-                     "kernel": "k_w64_mmv<bf16_t, 4, 1, 2>", "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 2),
+                     "kernel": "k_w64_mmv<bf16_t, 4, 1, 2, 1>", "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 2),
                      "median_launch_us": round(float(np.median(durs)) * 1e3, 2)},
         "extra": {"pct_of_hbm_peak_compressed": round(100 * comp_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
                   "us_per_matrix": round(ms * 1e3, 2), "block_us_per_step_min_max": [round(min(blocks) / args.steps * 1e3, 2), round(max(blocks) / args.steps * 1e3, 2)],
