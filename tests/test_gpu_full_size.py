@@ -458,6 +458,28 @@ def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, mode, wan
     assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y4))
 
 
+@pytest.mark.parametrize("rows,k", [(5120, 2048), (2048, 4096)])
+def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, rows, k):
+    """A 4-bit matrix large enough to fill the GPU with one column decodes a (row, chunk) once for 2 or 4 columns of a
+    batch: every column of every batch size up to 9 has the bits of its single-column product, escapes included."""
+    from orin_qwen_lossless_amd import synth
+
+    wb = synth.weights(rows, k, 900 + rows % 89)
+    wb[::5, ::131] = np.uint16(0x4500)  # exponents outside a row's window: escape records
+    plane, aux, fmt, _ = ops.encode_bits(wb, 1, 0)
+    assert fmt == 1
+    ta = torch.from_numpy(aux)
+    enc = ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
+    xb = synth.activations(9, k, 78)
+    x = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16).cuda()
+    single = torch.cat([ops.mmv(x[t: t + 1], enc) for t in range(9)])
+    for T in (2, 3, 4, 5, 8, 9):
+        assert torch.equal(ops.mmv(x[:T], enc), single[:T]), T
+    xf = x.float()
+    single_f = torch.cat([ops.mmv(xf[t: t + 1], enc) for t in range(4)])
+    assert torch.equal(ops.mmv(xf[:4], enc), single_f)
+
+
 # ---- the decode step (40 x [qkv, o, router, top-8, 256 experts + shared, glue]): two layers of it at real size ------------
 
 @pytest.fixture(scope="module")
