@@ -155,7 +155,9 @@ template <int NT, int W> struct mt_shape {
     static constexpr int TPT = STAGERS / TOK;                      // of them per token
     static constexpr int CPT = MT_HK / TPT;                        // columns each: 8 per uint4
     static constexpr int VPT = CPT / 8;
-    static constexpr int DEPTH = NT == 1 ? 2 : 4;                  // steps of plane bytes held ahead per chain
+    // steps of plane bytes held ahead per chain: two in every shape (a step of the 128-token shape takes about 2 us,
+    // longer than a load; four ahead took 18 more registers and ran the down product 6 % slower at 2048 tokens)
+    static constexpr int DEPTH = 2;
 };
 
 // the V uint4s a thread stages per block of activations, in named registers (under this kernel's register pressure
