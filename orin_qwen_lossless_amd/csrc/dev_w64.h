@@ -151,10 +151,22 @@ struct w64_dec_t {
     }
     // two pair codes; afterwards lanes whose position passed a word boundary request the next stream words in lane order
     __device__ __forceinline__ void two(const uint32_t * lut, uint32_t & e0, uint32_t & e1) {
+        two_with([lut](uint32_t off) { return lds_entry(lut, off); }, e0, e1);
+    }
+    // the same with the table at LDS byte address `lut_addr`, a compile-time value at the call (kernels whose only LDS
+    // is the dynamic segment keep their tables at its start, address 0): the address of an entry is then the masked
+    // stream bits themselves plus an immediate, where a pointer into the dynamic segment costs an add per lookup
+    __device__ __forceinline__ void two_at(uint32_t lut_addr, uint32_t & e0, uint32_t & e1) {
+        two_with([lut_addr](uint32_t off) {
+            return *(const __attribute__((address_space(3))) uint32_t *) (uintptr_t) (lut_addr + off);
+        }, e0, e1);
+    }
+    template <typename L>
+    __device__ __forceinline__ void two_with(L entry, uint32_t & e0, uint32_t & e1) {
         const uint32_t W = __builtin_amdgcn_alignbit(w1, w0, P);
-        e0 = lds_entry(lut, W & 0x3FFCu);
+        e0 = entry(W & 0x3FFCu);
         const uint32_t W2 = W >> (e0 & 31u);
-        e1 = lds_entry(lut, W2 & 0x3FFCu);
+        e1 = entry(W2 & 0x3FFCu);
         // entry bits 5 and 6 are zero and P < 32: bits 0..5 of the sum are exact (the exponent fields only add above)
         const uint32_t t = (P + e0 + e1) & 63u;
         const uint64_t m = lanes_lt(31u, t);

@@ -76,7 +76,8 @@ template <int D, bool ONCE = false> struct tchain_t {
 typedef tchain_t<4> tchain;
 
 // one step of N chains, instruction streams interleaved; lut of chain k at lut + k * lut_stride
-template <int N, int D, bool ONCE = false>
+// ABS: the tables sit at the start of the kernel's LDS (address 0): see w64_dec_t::two_at
+template <int N, int D, bool ONCE = false, bool ABS = false>
 __device__ __forceinline__ void tile_step(tchain_t<D, ONCE> * ch, const uint32_t * lut, int lut_stride, int s, uint32_t (&wp)[N][8]) {
     uint32_t smw[N][4];
 #pragma unroll
@@ -88,7 +89,11 @@ __device__ __forceinline__ void tile_step(tchain_t<D, ONCE> * ch, const uint32_t
 #pragma unroll
         for (int k = 0; k < N; k++) {
             uint32_t e0, e1;
-            ch[k].dec.two(lut + k * lut_stride, e0, e1);
+            if constexpr (ABS) {
+                ch[k].dec.two_at((uint32_t) (k * lut_stride * 4), e0, e1);
+            } else {
+                ch[k].dec.two(lut + k * lut_stride, e0, e1);
+            }
             wp[k][2 * j] = merge(spread_lo(smw[k][j]), e0);
             wp[k][2 * j + 1] = merge(spread_hi(smw[k][j]), e1);
         }
@@ -120,7 +125,7 @@ __device__ __forceinline__ void tile_step_mm(tchain_t<D, ONCE> * ch, const uint3
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 uint32_t e0, e1;
-                ch[k].dec.two(lut + k * lut_stride, e0, e1);
+                ch[k].dec.two_at((uint32_t) (k * lut_stride * 4), e0, e1); // (its callers keep the tables at LDS address 0)
                 wq[2 * j] = merge(spread_lo(smw[k][2 * kb + j]), e0);
                 wq[2 * j + 1] = merge(spread_hi(smw[k][2 * kb + j]), e1);
             }
@@ -349,7 +354,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
                                          [&](int kb) { return *(const bf16x8_t *) (bp + 16 * kb); }, acc[0][0], acc[1][0]);
                         } else {
                             uint32_t wp[2][8];
-                            tile_step<2, S::DEPTH, NT == 1>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
+                            tile_step<2, S::DEPTH, NT == 1, true>(ch, lut, GLU ? LUT_WORDS : 0, s, wp);
                             ch[0].reload(s, lane);
                             ch[1].reload(s, lane);
                             bf16x8_t av[2][2]; // [chain][16-column block]
@@ -835,19 +840,24 @@ bool is_tile_layout(const bf16n_weight & w) {
     return w.format == FMT_HUFPAIR && (w.flags & FLAG_WAVE64) && !(w.flags & FLAG_CHUNK_MAJOR) && w.R == TILE_R;
 }
 
-template <bool GLU, int NT, int W> void mt_attr() {
-    (void) hipFuncSetAttribute((const void *) k_mm_tile<GLU, NT, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<NT, W>(GLU));
+// The batched kernels address their tables by LDS address (two_at), which holds as long as the dynamic segment, whose
+// first words the tables are, starts at address 0: the kernel must have no static LDS.  Checked once per kernel here.
+void lds_attr(const void * kernel, size_t dynamic_bytes) {
+    hipFuncAttributes fa;
+    if (hipFuncGetAttributes(&fa, kernel) == hipSuccess && fa.sharedSizeBytes != 0) {
+        throw std::logic_error("bf16n: a batched tile kernel has static LDS in front of its tables");
+    }
+    (void) hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) dynamic_bytes);
 }
-template <bool GLU> void ks_attr() {
-    (void) hipFuncSetAttribute((const void *) k_mm_tile_ks<GLU>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) ks_shm(GLU));
-}
+template <bool GLU, int NT, int W> void mt_attr() { lds_attr((const void *) k_mm_tile<GLU, NT, W>, mt_shm<NT, W>(GLU)); }
+template <bool GLU> void ks_attr() { lds_attr((const void *) k_mm_tile_ks<GLU>, ks_shm(GLU)); }
 
 void tile_init() {
     mt_attr<true, 4, 8>();
     mt_attr<false, 4, 8>();
     mt_attr<true, 1, 16>();
     mt_attr<false, 1, 16>();
-    (void) hipFuncSetAttribute((const void *) k_mm_tile<false, 1, 16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) mt_shm<1, 16>(false));
+    lds_attr((const void *) k_mm_tile<false, 1, 16, true>, mt_shm<1, 16>(false));
     ks_attr<true>(); ks_attr<false>();
 }
 
