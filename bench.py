@@ -218,7 +218,7 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4), n_laye
 
     sets, raw, nbytes = D.make_layer_sets(ops, gen, n_sets, True)
     head_bytes = head.plane.numel() + head.aux.numel()
-    res = {"layers": n_layers, "weight_sets": n_sets, "launches_per_layer": 8,
+    res = {"layers": n_layers, "weight_sets": n_sets,
            "bf16_comparator": "the same graph on uncompressed BF16 weights: torch linear / bmm (hipBLASLt) for every product, the "
                               "experts a token selects gathered by index_select (the routing is decided on the device), "
                               "the same glue and top-k launches"}
@@ -243,7 +243,8 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4), n_laye
         bf16_bytes = 2 * (n_layers * (sum(r * k for n_, (r, k, m) in D.SHAPES.items() if m == 1)
                                       + (min(T * D.TOPK, D.E) + 1) * 3 * D.N_MID * K) + head_bf16.numel())
         t = entry["bf16n"]
-        res[f"batch{T}"] = {"us": round(t, 1), "compressed_bytes_touched_upper_bound": int(touched), "GBps": round(touched / t / 1e3, 1),
+        gemv_path = T * (D.TOPK + 1) <= max(ops.MOE_GEMV_MIN_PAIRS, ops.MOE_GEMV_PAIRS_PER_EXPERT[0] * D.EA)
+        res[f"batch{T}"] = {"us": round(t, 1), "launches_per_layer": 8 if gemv_path else 9, "compressed_bytes_touched_upper_bound": int(touched), "GBps": round(touched / t / 1e3, 1),
                             "frac_of_hbm_peak": round(touched / t / 1e3 / HBM_PEAK_GBS, 4), "tokens_per_s": round(T / t * 1e6, 1),
                             "bf16_us": round(entry["bf16"], 1), "speedup_vs_bf16": round(entry["bf16"] / t, 2),
                             "bf16_bytes_touched": int(bf16_bytes), "bf16_us_at_hbm_peak": round(bf16_bytes / HBM_PEAK_GBS / 1e3, 1),

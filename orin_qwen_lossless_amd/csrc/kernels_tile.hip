@@ -219,12 +219,15 @@ struct mm_args {
 // blocks share out the work items of these only, so that a call with few active experts keeps its blocks equally loaded
 // instead of leaving some with several items and others with none.  Every wavefront of the block takes 64 experts at
 // a time (one read of their bounds for the whole block), the counts meet in LDS behind the list.  Ends with a barrier.
-__device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, int wave, int lane, int n_waves) {
+// span (optional, [MT_MAX_LISTED]): first routed pair and number of pairs of every listed expert, so that the items need
+// not read the bounds again.
+__device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, int wave, int lane, int n_waves, int2 * span = nullptr) {
     int * cnt = (int *) (act + MT_MAX_LISTED + 8); // [n_waves], n_waves <= 16
     int total = 0;
     for (int e0 = 0; e0 < a.n_experts; e0 += 64 * n_waves) {
         const int e = e0 + 64 * wave + lane;
-        const bool on = e < a.n_experts && a.bounds[e + 1] > a.bounds[e];
+        const int b0 = e < a.n_experts ? a.bounds[e] : 0, b1 = e < a.n_experts ? a.bounds[e + 1] : 0;
+        const bool on = b1 > b0;
         const uint64_t m = __ballot(on);
         if (lane == 0) {
             cnt[wave] = __builtin_popcountll(m);
@@ -237,7 +240,11 @@ __device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, in
             all += c;
         }
         if (on) {
-            act[before + __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u))] = (uint16_t) e;
+            const int at = before + (int) __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
+            act[at] = (uint16_t) e;
+            if (span) {
+                span[at] = make_int2(b0, b1 - b0);
+            }
         }
         total += all;
         __syncthreads();
@@ -454,7 +461,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
 constexpr int KS_WAVES = 16;
 
 struct ks_ctx {
-    uint32_t * lut, * rings; uint16_t * act;
+    uint32_t * lut, * rings; uint16_t * act; const int2 * span;
     int n_items, per_expert, groups, slabs;
 };
 
@@ -491,15 +498,15 @@ __device__ __forceinline__ void ks_items(const bf16n_weight & w, const bf16n_wei
 #pragma unroll
         for (int k = 0; k < IPB; k++) {
             if (k < cnt) {
-                const int ek = (int) uniform(act[(base + k) / per_expert]);
-                const int nk = a.bounds[ek + 1] - a.bounds[ek];
+                const int nk = (int) uniform((uint32_t) c.span[(base + k) / per_expert].y);
                 maxn = nk > maxn ? nk : maxn;
             }
         }
         const int item = base + is;
         const bool valid = is < cnt;
-        const int e = valid ? (int) uniform(act[item / per_expert]) : 0, p = valid ? item % per_expert : 0;
-        const int j0 = a.bounds[e], n = valid ? a.bounds[e + 1] - j0 : 0;
+        const int at = valid ? item / per_expert : 0, p = valid ? item % per_expert : 0;
+        const int e = (int) uniform(act[at]);
+        const int j0 = (int) uniform((uint32_t) c.span[at].x), n = valid ? (int) uniform((uint32_t) c.span[at].y) : 0;
         const int g0 = GLU ? p : 2 * p;
         const bool has1 = GLU || g0 + 1 < groups;
         const int g1 = has1 && !GLU ? g0 + 1 : g0;
@@ -599,6 +606,8 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     c.lut = shm;
     c.rings = shm + NM * LUT_WORDS;
     c.act = (uint16_t *) (c.rings + KS_WAVES * 2 * WAVE_LDS_WORDS);
+    int2 * span = (int2 *) (c.act + MT_MAX_LISTED + 8 + 2 * 16); // behind the list and its 16 counters
+    c.span = span;
     const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6);
     // the tables are requested first (one 16-byte load per thread and table) and stored once the block knows that it
     // has work: their way from memory overlaps the listing of the active experts
@@ -608,7 +617,7 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     c.groups = (int) (a.rows / TILE_R);
     c.per_expert = GLU ? c.groups : (c.groups + 1) / 2;       // items per expert
     c.slabs = (int) (w.K / TILE_K);
-    c.n_items = list_active(c.act, a, wave, lane, KS_WAVES) * c.per_expert;
+    c.n_items = list_active(c.act, a, wave, lane, KS_WAVES, span) * c.per_expert;
     // the most wavefronts per item for which the launch's blocks hold every item at once
     int wpi = KS_WAVES;
     while (wpi > 1 && (c.slabs % wpi != 0 || (int64_t) c.n_items * wpi > (int64_t) gridDim.x * KS_WAVES)) {
@@ -633,8 +642,9 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     }
 }
 
-size_t ks_shm(bool glu) {
-    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_LISTED + 8) * 2 + 16 * 4;
+size_t ks_shm(bool glu) { // tables, rings, list of active experts + counters, their spans
+    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_LISTED + 8) * 2 + 16 * 4 +
+           (size_t) MT_MAX_LISTED * 8;
 }
 
 template <int NT, int W> size_t mt_shm(bool glu) {
