@@ -62,6 +62,12 @@ __device__ __forceinline__ uint64_t lanes_lt(uint32_t a, uint32_t b) {
     asm("v_cmp_lt_u32_e64 %0, %1, %2" : "=s"(m) : "v"(a), "v"(b));
     return m;
 }
+// lane mask of (a != b)
+__device__ __forceinline__ uint64_t lanes_ne(uint32_t a, uint32_t b) {
+    uint64_t m;
+    asm("v_cmp_ne_u32_e64 %0, %1, %2" : "=s"(m) : "v"(a), "v"(b));
+    return m;
+}
 // lane-wise m ? b : a
 __device__ __forceinline__ uint32_t pick(uint32_t a, uint32_t b, uint64_t m) {
     uint32_t d;
@@ -78,7 +84,10 @@ __device__ __forceinline__ int64_t uniform64(int64_t v) { // an offset the compi
 // prefetched block between registers at its end: 2.5 % of the 248320 x 2048 GEMV).
 template <int HINT = -1>
 struct w64_dec_t {
-    uint32_t w0, w1, w2, P; // per lane: three stream words and the bit position in w0 (< 32)
+    uint32_t w0, w1, w2;    // per lane: three stream words
+    uint32_t P;             // per lane: bits consumed since the unit began, in its low seven bits (the bits above are
+                            // scraps of table entries); P mod 32 is the position in w0, which is all the funnel shift reads
+    uint32_t P5;            // bit 5 of P at the last check: a change of that bit is a word boundary passed
     uint32_t nw;            // the word requested at the last check (becomes w2 where took is set)
     uint64_t took;          // lanes that requested a word at the last check
     uint32_t cons;          // words consumed, relative to src
@@ -145,6 +154,7 @@ struct w64_dec_t {
         w1 = p[1];
         w2 = p[2];
         P = 0;
+        P5 = 0;
         took = 0;
         nw = 0;
         cons = uniform(cons + 192);
@@ -167,9 +177,12 @@ struct w64_dec_t {
         e0 = entry(W & 0x3FFCu);
         const uint32_t W2 = W >> (e0 & 31u);
         e1 = entry(W2 & 0x3FFCu);
-        // entry bits 5 and 6 are zero and P < 32: bits 0..5 of the sum are exact (the exponent fields only add above)
-        const uint32_t t = (P + e0 + e1) & 63u;
-        const uint64_t m = lanes_lt(31u, t);
+        // entry bits 5 and 6 are zero: the low seven bits of the running sum are exact (the exponent fields only add
+        // above them), and two pair codes are at most 24 bits, so bit 5 changes exactly when a word boundary is passed
+        P = P + e0 + e1;
+        const uint32_t p5 = P & 32u;
+        const uint64_t m = lanes_ne(p5, P5);
+        P5 = p5;
         const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
         const uint32_t req = ring[(cons & (RING - 1)) + rank];
         // the word requested one check ago has arrived by now: it is this lane's w2
@@ -178,7 +191,6 @@ struct w64_dec_t {
         w1 = pick(w1, w2, m);
         nw = req;
         took = m;
-        P = t & 31u;
         cons = uniform(cons + (uint32_t) __builtin_popcountll(m));
     }
     // the 16 weights of this lane in one step as 8 BF16 pairs: wp[2j], wp[2j+1] = columns 128j + 4(lane%32) + {0,1}, {2,3}
