@@ -376,11 +376,27 @@ __global__ void __launch_bounds__(NT) k_nib_rows(const bf16n_weight w, const cha
         const int64_t gr = row0 + (ids ? (int64_t) * (const int32_t *) (ids + i * ids_s0) : i);
         char * o = dst + i * dst_s1;
         const uint4 T = *(const uint4 *) (q.table + gr * 16);
+        const uint32_t e0 = q.esc_off[gr], e1 = q.esc_off[gr + 1];
         for (int c = 0; c < C; c++) {
             const uint4 sm = *((const uint4 *) (q.plane + gr * K + c * CHUNK) + l32);
             const uint2 cd = *((const uint2 *) (q.codes + gr * (K / 2) + c * 256) + l32);
             uint32_t wp[8];
             nib_chunk(sm, cd, T, wp);
+            // the row's escapes go into the registers of the lane that holds their column: every element is stored once
+            for (uint32_t e = e0; e < e1; e++) {
+                const uint32_t rec = q.esc[e];
+                const int rel = (int) (rec & 0xFFFu) - c * CHUNK;
+                if (rel >= 0 && rel < CHUNK && ((rel & 127) >> 2) == l32) {
+                    const int at = (rel >> 7) * 2 + ((rel & 3) >> 1);
+                    const uint32_t b = esc_bits(rec);
+#pragma unroll
+                    for (int i2 = 0; i2 < 8; i2++) {
+                        if (i2 == at) {
+                            wp[i2] = (rel & 1) ? (wp[i2] & 0xFFFFu) | (b << 16) : (wp[i2] & 0xFFFF0000u) | b;
+                        }
+                    }
+                }
+            }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int col = c * CHUNK + 128 * j + 4 * l32;
@@ -390,17 +406,6 @@ __global__ void __launch_bounds__(NT) k_nib_rows(const bf16n_weight w, const cha
                     *(float4 *) (o + 4 * col) = make_float4(bf16_bits_to_f32(wp[2 * j] & 0xFFFFu), __uint_as_float(wp[2 * j] & 0xFFFF0000u),
                                                             bf16_bits_to_f32(wp[2 * j + 1] & 0xFFFFu), __uint_as_float(wp[2 * j + 1] & 0xFFFF0000u));
                 }
-            }
-        }
-        // the dense stores of this half-wave must land before its escape stores to the same row
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        __builtin_amdgcn_wave_barrier();
-        for (uint32_t e = q.esc_off[gr] + l32; e < q.esc_off[gr + 1]; e += 32) {
-            const uint32_t rec = q.esc[e];
-            if (BF) {
-                ((uint16_t *) o)[rec & 0xFFFu] = (uint16_t) esc_bits(rec);
-            } else {
-                ((float *) o)[rec & 0xFFFu] = bf16_bits_to_f32(esc_bits(rec));
             }
         }
     }
