@@ -244,7 +244,7 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4), n_laye
                                       + (min(T * D.TOPK, D.E) + 1) * 3 * D.N_MID * K) + head_bf16.numel())
         t = entry["bf16n"]
         gemv_path = T * (D.TOPK + 1) <= max(ops.MOE_GEMV_MIN_PAIRS, ops.MOE_GEMV_PAIRS_PER_EXPERT[0] * D.EA)
-        res[f"batch{T}"] = {"us": round(t, 1), "launches_per_layer": 8 if gemv_path else 9, "compressed_bytes_touched_upper_bound": int(touched), "GBps": round(touched / t / 1e3, 1),
+        res[f"batch{T}"] = {"us": round(t, 1), "launches_per_layer": 8 if gemv_path or T <= ops.TOPK_ROUTE_ONE_LAUNCH_TOKENS else 9, "compressed_bytes_touched_upper_bound": int(touched), "GBps": round(touched / t / 1e3, 1),
                             "frac_of_hbm_peak": round(touched / t / 1e3 / HBM_PEAK_GBS, 4), "tokens_per_s": round(T / t * 1e6, 1),
                             "bf16_us": round(entry["bf16"], 1), "speedup_vs_bf16": round(entry["bf16"] / t, 2),
                             "bf16_bytes_touched": int(bf16_bytes), "bf16_us_at_hbm_peak": round(bf16_bytes / HBM_PEAK_GBS / 1e3, 1),

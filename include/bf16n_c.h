@@ -133,6 +133,15 @@ int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, in
  * shared expert stacked behind them) keeps their ids and weights in the columns from k on */
 int bf16n_router_topk_strided(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
                               int32_t * ids, float * weights, int64_t out_stride, void * stream);
+/* bf16n_router_topk_strided and bf16n_mm_ids_route (launch.cu:458-471) in one launch for few tokens: after the top-k the
+ * same block sorts the first n_slots columns (k <= n_slots <= out_stride: the k chosen here, then the columns the caller
+ * keeps filled) of the id rows into the lists bf16n_mm_ids_route writes for them, over n_listed >= n_experts experts
+ * (bounds: n_listed + 1 entries; ids_src1, ids_dst: n_tok * n_slots).  Limits, bf16n_router_topk_route_fits: n_tok <= 16,
+ * n_tok * n_slots <= 1024, n_listed <= 1024.  Ids outside [0, n_listed) in the caller's columns are left out of the lists. */
+int bf16n_router_topk_route_fits(int n_tok, int n_slots, int n_listed);
+int bf16n_router_topk_route(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
+                            int32_t * ids, float * weights, int64_t out_stride, int n_slots, int n_listed,
+                            int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds, int nchannels_y, int sis1, void * stream);
 
 /* Read-bandwidth probe (the reference's bench/micro/bwprobe.cu:23-60 as a library call): a kernel that only reads
  * `bytes` (rounded down to whole KiB) from src, for the memory rate this GPU gives a pure streaming read.  pattern 0:

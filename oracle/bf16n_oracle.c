@@ -668,11 +668,14 @@ void orc_moe_combine(const float *ys, const float *w, float *y, int n_tok, int n
 
 void orc_route(const int32_t *ids, int64_t ids_stride, int n_experts, int n_tok, int n_used, int nchannels_y, int sis1,
                int32_t *ids_src1, int32_t *ids_dst, int32_t *bounds) {
-    int j = 0;
+    int listed = 0;
     for (int e = 0; e < n_experts; e++) {
+        int j = 0; /* the expert's list starts behind every naming of a lower expert (nex_prev, mmid_helper.cu:66-68) */
+        for (int t = 0; t < n_tok; t++)
+            for (int k = 0; k < n_used; k++) j += ids[t * ids_stride + k] < e;
         bounds[e] = j;
         for (int t = 0; t < n_tok; t++) {
-            int used = -1; /* the last slot of the token naming e (mmid_helper.cu:66-71) */
+            int used = -1; /* the last slot of the token naming e (mmid_helper.cu:69-71) */
             for (int k = 0; k < n_used; k++)
                 if (ids[t * ids_stride + k] == e) used = k;
             if (used >= 0) {
@@ -681,8 +684,9 @@ void orc_route(const int32_t *ids, int64_t ids_stride, int n_experts, int n_tok,
                 j++;
             }
         }
+        listed = j;
     }
-    bounds[n_experts] = j;
+    bounds[n_experts] = listed; /* mmid_helper.cu:134 */
 }
 
 void orc_router_topk(const float *logits, int n, int k, int32_t *ids, float *weights) {

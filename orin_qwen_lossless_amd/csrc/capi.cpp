@@ -531,6 +531,29 @@ int bf16n_router_topk_strided(const float * logits, int64_t logits_stride, int n
     });
 }
 
+int bf16n_router_topk_route_fits(int n_tok, int n_slots, int n_listed) {
+    return n_tok > 0 && n_slots > 0 && n_listed > 0 && dev::router_topk_route_fits(n_tok, n_slots, n_listed) ? 1 : 0;
+}
+
+int bf16n_router_topk_route(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
+                            int32_t * ids, float * weights, int64_t out_stride, int n_slots, int n_listed,
+                            int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds, int nchannels_y, int sis1, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        require(n_tok > 0 && n_experts > 0 && k > 0 && k <= n_experts && k <= 64, "router_topk: need 0 < k <= min(n_experts, 64)");
+        require(n_experts <= 1024, "router_topk: at most 1024 experts");
+        require(n_slots >= k && out_stride >= n_slots, "router_topk_route: need k <= n_slots <= out_stride");
+        require(n_listed >= n_experts, "router_topk_route: the lists must cover the router's experts");
+        require(bf16n_router_topk_route_fits(n_tok, n_slots, n_listed) != 0,
+                "router_topk_route: at most 16 tokens, 1024 (token, slot) pairs and 1024 listed experts");
+        require(logits && ids && weights && ids_src1 && ids_dst && bounds, "null pointer");
+        require(nchannels_y > 0, "routing sizes out of range");
+        dev::launch_router_topk_route(logits, logits_stride, n_tok, n_experts, k, renorm != 0, ids, weights, out_stride, n_slots,
+                                      n_listed, ids_src1, ids_dst, bounds, nchannels_y, sis1, (hipStream_t) stream);
+        launch_check("router_topk_route");
+    });
+}
+
 int bf16n_router_topk(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
                       int32_t * ids, float * weights, void * stream) {
     return bf16n_router_topk_strided(logits, logits_stride, n_tok, n_experts, k, renorm, ids, weights, k, stream);

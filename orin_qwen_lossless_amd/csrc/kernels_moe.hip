@@ -167,10 +167,8 @@ __global__ void __launch_bounds__(ROUTE_THREADS) k_route(const char * __restrict
 // ever returns an index below n_experts that was not taken before, whatever the values are: the ids feed address
 // arithmetic in the kernels that follow.
 template <int NQ>
-__global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ logits, int64_t stride, int n_experts, int k, bool renorm,
-                                                    int32_t * __restrict__ ids, float * __restrict__ weights, int64_t out_stride) {
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const float * lg = logits + (int64_t) t * stride;
+__device__ __forceinline__ void topk_token(const float * __restrict__ lg, int n_experts, int k, bool renorm, int32_t * ids_row,
+                                           float * weights_row, int lane, int * ids_copy = nullptr) {
     float val[NQ];
     bool open[NQ]; // a real expert that has not been taken yet
     float mx = -INFINITY;
@@ -207,7 +205,10 @@ __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ l
         top += pj;
         if (lane == (j & 63)) {
             mine = pj; // k <= 64
-            ids[(int64_t) t * out_stride + j] = (int32_t) bi;
+            ids_row[j] = (int32_t) bi;
+            if (ids_copy) {
+                ids_copy[j] = (int) bi;
+            }
         }
 #pragma unroll
         for (int q = 0; q < NQ; q++) {
@@ -215,7 +216,102 @@ __global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ l
         }
     }
     if (lane < k) {
-        weights[(int64_t) t * out_stride + lane] = renorm ? mine / top : mine;
+        weights_row[lane] = renorm ? mine / top : mine;
+    }
+}
+
+template <int NQ>
+__global__ void __launch_bounds__(64) k_router_topk(const float * __restrict__ logits, int64_t stride, int n_experts, int k, bool renorm,
+                                                    int32_t * __restrict__ ids, float * __restrict__ weights, int64_t out_stride) {
+    const int t = blockIdx.x;
+    topk_token<NQ>(logits + (int64_t) t * stride, n_experts, k, renorm, ids + (int64_t) t * out_stride, weights + (int64_t) t * out_stride,
+                   (int) threadIdx.x);
+}
+
+// The router's top-k of up to TOPK_ROUTE_TOKENS tokens and the expert-sorted lists of k_route over the first n_slots
+// columns of their id rows (the k chosen here, then columns the caller has filled: experts every token uses), in one
+// launch of one block: wavefront t selects for token t, then the block sorts the (token, slot) pairs.  The lists are
+// those k_route writes for the same ids (entries of an expert in token order; of an expert that a token names twice
+// the last slot counts, and bounds count every naming); ids outside [0, n_listed) are left out.
+constexpr int TOPK_ROUTE_TOKENS = 16, TOPK_ROUTE_MAX = 1024; // wavefronts of the block; pairs and listed experts
+template <int NQ>
+__global__ void __launch_bounds__(TOPK_ROUTE_TOKENS * 64) k_router_topk_route(
+        const float * __restrict__ logits, int64_t stride, int n_experts, int k, bool renorm, int32_t * ids, float * __restrict__ weights,
+        int64_t out_stride, int n_tok, int n_slots, int n_listed, int32_t * __restrict__ ids_src1, int32_t * __restrict__ ids_dst,
+        int32_t * __restrict__ bounds, int nchannels_y, int sis1) {
+    __shared__ int named[TOPK_ROUTE_MAX];  // namings of an expert, then the start of its list
+    __shared__ int listed[TOPK_ROUTE_MAX]; // entries of its list
+    __shared__ int named_by[TOPK_ROUTE_MAX]; // expert a pair names
+    __shared__ int key[TOPK_ROUTE_MAX];    // expert of a pair that enters a list, else -1
+    __shared__ int wave_total[TOPK_ROUTE_TOKENS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int pairs = n_tok * n_slots;
+    const int t = tid / n_slots, s = tid - t * n_slots;
+    int given = -1; // a column the caller filled
+    if (tid < pairs && s >= k) {
+        given = ids[(int64_t) t * out_stride + s];
+    }
+    named[tid] = 0;
+    listed[tid] = 0;
+    if (wave < n_tok) {
+        topk_token<NQ>(logits + (int64_t) wave * stride, n_experts, k, renorm, ids + (int64_t) wave * out_stride,
+                       weights + (int64_t) wave * out_stride, lane, named_by + wave * n_slots);
+    }
+    if (tid < pairs && s >= k) {
+        named_by[tid] = given;
+    }
+    __syncthreads();
+    int mine = -1;
+    if (tid < pairs) {
+        const int v = named_by[tid];
+        if (v >= 0 && v < n_listed) {
+            bool last = true;
+            for (int s2 = s + 1; s2 < n_slots; s2++) {
+                last &= named_by[tid - s + s2] != v;
+            }
+            atomicAdd(&named[v], 1);
+            if (last) {
+                atomicAdd(&listed[v], 1);
+                mine = v;
+            }
+        }
+    }
+    key[tid] = mine;
+    __syncthreads();
+    // exclusive prefix of the namings over the experts
+    const int c = named[tid]; // 0 from n_listed on
+    int scan = c;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(scan, o, 64);
+        scan += lane >= o ? up : 0;
+    }
+    if (lane == 63) {
+        wave_total[wave] = scan;
+    }
+    __syncthreads();
+    int start = scan - c;
+#pragma unroll
+    for (int w2 = 0; w2 < TOPK_ROUTE_TOKENS; w2++) {
+        start += w2 < wave ? wave_total[w2] : 0;
+    }
+    named[tid] = start;
+    if (tid < n_listed) {
+        bounds[tid] = start;
+        if (tid == n_listed - 1) {
+            bounds[n_listed] = start + listed[tid];
+        }
+    }
+    __syncthreads();
+    if (mine >= 0) {
+        int rank = 0; // pairs are numbered token by token: the earlier entries of this expert's list
+#pragma unroll 8
+        for (int j = 0; j < tid; j++) {
+            rank += key[j] == mine;
+        }
+        const int j = named[mine] + rank;
+        ids_dst[j] = t * n_slots + s;
+        ids_src1[j] = t * sis1 + s % nchannels_y;
     }
 }
 
@@ -345,6 +441,23 @@ void launch_router_topk_strided(const float * logits, int64_t stride, int n_tok,
         hipLaunchKernelGGL(k_router_topk<4>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights, out_stride);
     } else {
         hipLaunchKernelGGL(k_router_topk<16>, dim3(n_tok), dim3(64), 0, stream, logits, stride, n_experts, k, renorm, ids, weights, out_stride);
+    }
+}
+bool router_topk_route_fits(int n_tok, int n_slots, int n_listed) {
+    return n_tok <= TOPK_ROUTE_TOKENS && (int64_t) n_tok * n_slots <= TOPK_ROUTE_MAX && n_listed <= TOPK_ROUTE_MAX;
+}
+void launch_router_topk_route(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
+                              float * weights, int64_t out_stride, int n_slots, int n_listed, int32_t * ids_src1, int32_t * ids_dst,
+                              int32_t * bounds, int nchannels_y, int sis1, hipStream_t stream) {
+    if (!router_topk_route_fits(n_tok, n_slots, n_listed)) {
+        throw std::invalid_argument("router_topk_route: at most 16 tokens, 1024 (token, slot) pairs and 1024 listed experts");
+    }
+    if (n_experts <= 256) {
+        hipLaunchKernelGGL(k_router_topk_route<4>, dim3(1), dim3(TOPK_ROUTE_TOKENS * 64), 0, stream, logits, stride, n_experts, k, renorm,
+                           ids, weights, out_stride, n_tok, n_slots, n_listed, ids_src1, ids_dst, bounds, nchannels_y, sis1);
+    } else {
+        hipLaunchKernelGGL(k_router_topk_route<16>, dim3(1), dim3(TOPK_ROUTE_TOKENS * 64), 0, stream, logits, stride, n_experts, k, renorm,
+                           ids, weights, out_stride, n_tok, n_slots, n_listed, ids_src1, ids_dst, bounds, nchannels_y, sis1);
     }
 }
 void launch_router_topk(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,

@@ -63,6 +63,11 @@ struct add_norm_args {
 void launch_add_rmsnorm(const add_norm_args & a, int n_tok, hipStream_t stream);
 void launch_router_topk_strided(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
                                 float * weights, int64_t out_stride, hipStream_t stream);
+// top-k and the routing lists of launch_route over the first n_slots columns of the id rows in one launch (few tokens)
+bool router_topk_route_fits(int n_tok, int n_slots, int n_listed);
+void launch_router_topk_route(const float * logits, int64_t stride, int n_tok, int n_experts, int k, bool renorm, int32_t * ids,
+                              float * weights, int64_t out_stride, int n_slots, int n_listed, int32_t * ids_src1, int32_t * ids_dst,
+                              int32_t * bounds, int nchannels_y, int sis1, hipStream_t stream);
 
 // read-bandwidth probe (kernels_probe.hip)
 void launch_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, int cus, hipStream_t stream);

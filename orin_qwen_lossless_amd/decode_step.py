@@ -78,8 +78,12 @@ class Bf16nStep:
     def experts(self, w, x2):
         """(ys [T, 9, K] FP32 per-slot outputs, wts [T, 9], ids [T, 9])."""
         ops = self.ops
-        wts, ids = ops.router_topk(ops.mmv(x2, w["router"]), TOPK, out=self.routing)
-        return ops.moe_experts_rows(x2, w["gate"], w["up"], w["down"], ids, EA), wts, ids
+        logits, routes = ops.mmv(x2, w["router"]), None
+        if ops.moe_experts_batched(x2.shape[0], TOPK + 1, w["gate"], w["up"], w["down"], EA):
+            wts, ids, routes = ops.router_topk_routes(logits, TOPK, EA, out=self.routing)  # one launch up to 16 tokens
+        else:
+            wts, ids = ops.router_topk(logits, TOPK, out=self.routing)
+        return ops.moe_experts_rows(x2, w["gate"], w["up"], w["down"], ids, EA, routes), wts, ids
 
     def layer(self, w, h, x1):
         ops = self.ops

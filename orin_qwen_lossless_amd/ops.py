@@ -593,6 +593,45 @@ def router_topk(logits: torch.Tensor, k: int, renorm: bool = True, out: tuple[to
     return wts, ids
 
 
+# router_topk_routes: tokens up to which one block that selects and sorts beats the two launches (its one CU runs a
+# wavefront per token: 7.7 / 8.6 / 12.4 us at 4 / 8 / 16 tokens against 4.6 + 5.4 us and the gap between two launches)
+TOPK_ROUTE_ONE_LAUNCH_TOKENS = 8
+
+
+def router_topk_routes(logits: torch.Tensor, k: int, n_listed: int, renorm: bool = True,
+                       out: tuple[torch.Tensor, torch.Tensor] | None = None):
+    """router_topk followed by mm_ids_route(ids, n_listed, False) over every column of the id rows: (weights, ids,
+    (ids_src1, ids_dst, bounds)).  One launch (bf16n_router_topk_route) up to TOPK_ROUTE_ONE_LAUNCH_TOKENS tokens, two
+    beyond."""
+    if out is not None and not (out[1].dim() == 2 and out[1].shape[1] >= k):
+        raise ValueError("bf16n.router_topk_routes: out must be (f32, int32) [tokens, m >= k] tensors")
+    T = logits.shape[0] if logits.dim() == 2 else 0
+    n_slots = out[1].shape[1] if out is not None else k
+    L = _lib.lib()
+    if T == 0 or T > TOPK_ROUTE_ONE_LAUNCH_TOKENS or not L.bf16n_router_topk_route_fits(T, n_slots, n_listed):
+        wts, ids = router_topk(logits, k, renorm, out)
+        return wts, ids, mm_ids_route(ids, n_listed, False)
+    if not (logits.is_cuda and logits.dtype == torch.float32 and logits.stride(1) == 1):
+        raise ValueError("bf16n.router_topk: logits must be f32 [tokens, n_experts], contiguous along experts")
+    dev = logits.device
+    if out is None:
+        ids = torch.empty((T, k), dtype=torch.int32, device=dev)
+        wts = torch.empty((T, k), dtype=torch.float32, device=dev)
+    else:
+        wts, ids = out
+        if not (wts.dtype == torch.float32 and ids.dtype == torch.int32 and wts.shape == ids.shape and wts.shape[0] == T
+                and wts.is_contiguous() and ids.is_contiguous() and wts.device == dev and ids.device == dev):
+            raise ValueError("bf16n.router_topk: out must be contiguous (f32, int32) [tokens, m >= k] tensors on the logits' device")
+    src1 = torch.empty(T * n_slots, dtype=torch.int32, device=dev)
+    dst = torch.empty(T * n_slots, dtype=torch.int32, device=dev)
+    bounds = torch.empty(n_listed + 1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(L.bf16n_router_topk_route(logits.data_ptr(), logits.stride(0), T, logits.shape[1], k, int(renorm), ids.data_ptr(),
+                                             wts.data_ptr(), n_slots, n_slots, n_listed, src1.data_ptr(), dst.data_ptr(),
+                                             bounds.data_ptr(), 1, 1, _stream()))
+    return wts, ids, (src1, dst, bounds)
+
+
 _probe_sink: dict = {}
 
 
@@ -616,10 +655,10 @@ def glu2_supported(gate: Weight, up: Weight) -> bool:
             and (not g.wave64 or g.K in (512, 1024, 2048, 4096)))
 
 
-def _experts_batched(x, gate, up, down, topk_ids, n_experts):
+def _experts_batched(x, gate, up, down, topk_ids, n_experts, routes=None):
     """Per-pair FP32 outputs of the routed experts through the batched kernels: one routing pass serves both products
     (with one activation row per (token, slot), as down takes them, the source row of a pair is its destination row)."""
-    src1, dst, bounds = mm_ids_route(topk_ids, n_experts, False)
+    src1, dst, bounds = routes if routes is not None else mm_ids_route(topk_ids, n_experts, False)
     hidden = moe_mm_ids(x, topk_ids, gate, n_experts, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
     return moe_mm_ids(hidden, topk_ids, down, n_experts, out_dtype=torch.float32, routes=(dst, dst, bounds))
 
@@ -631,10 +670,22 @@ def _experts_gemv_hidden(x, gate, up, topk_ids, n_mid):
     return swiglu(mmv(x, gate, topk_ids, n_mid), mmv(x, up, topk_ids, n_mid))
 
 
-def moe_experts_rows(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_ids: torch.Tensor, n_experts: int
-                     ) -> torch.Tensor:
+def moe_experts_batched(n_tokens: int, n_used: int, gate: Weight, up: Weight, down: Weight, n_experts: int) -> bool:
+    """Whether moe_experts_rows runs these experts through the batched kernels (then it takes routing lists) rather than
+    through one GEMV column per (token, slot); the thresholds are explained there."""
+    tiles = all(m.meta.wave64 and m.meta.R == 32 for m in (gate, up, down))
+    if tiles:
+        gemv = n_tokens * n_used <= max(MOE_GEMV_MIN_PAIRS, MOE_GEMV_PAIRS_PER_EXPERT[0] * n_experts)
+    else:
+        gemv = n_tokens <= max(GEMV_MAX_TOKENS, int(MOE_GEMV_PAIRS_PER_EXPERT[1] * n_experts) // n_used)
+    return not gemv and mm_ids_supported(gate, up) and mm_ids_supported(down)
+
+
+def moe_experts_rows(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, topk_ids: torch.Tensor, n_experts: int,
+                     routes=None) -> torch.Tensor:
     """The per-(token, slot) outputs down_e(silu(gate_e x) * (up_e x)) of the routed experts, FP32 [T, n_used, H]:
     moe_experts before the weighted sum (callers that fold the sum into their own next launch, add_rmsnorm, stop here).
+    routes: mm_ids_route(topk_ids, n_experts, False) if the caller has it (router_topk_routes), used by the batched kernels.
 
     The reference switches from expert GEMVs to the batched kernels above 8 tokens.  Here the GEMVs stay ahead only
     while the routed pairs are few against the experts (each pair decodes one expert matrix in its own GEMV column; the
@@ -646,13 +697,8 @@ def moe_experts_rows(x: torch.Tensor, gate: Weight, up: Weight, down: Weight, to
     n_tokens, n_used = x.shape[0], max(int(topk_ids.shape[1]), 1)
     n_mid, n_out = gate.meta.rows // n_experts, down.meta.rows // n_experts
     x = x.contiguous()
-    tiles = all(m.meta.wave64 and m.meta.R == 32 for m in (gate, up, down))
-    if tiles:
-        gemv = n_tokens * n_used <= max(MOE_GEMV_MIN_PAIRS, MOE_GEMV_PAIRS_PER_EXPERT[0] * n_experts)
-    else:
-        gemv = n_tokens <= max(GEMV_MAX_TOKENS, int(MOE_GEMV_PAIRS_PER_EXPERT[1] * n_experts) // n_used)
-    if not gemv and mm_ids_supported(gate, up) and mm_ids_supported(down):
-        return _experts_batched(x, gate, up, down, topk_ids, n_experts)
+    if moe_experts_batched(n_tokens, n_used, gate, up, down, n_experts):
+        return _experts_batched(x, gate, up, down, topk_ids, n_experts, routes)
     # one GEMV column per (token, slot), FP32 between the products
     return mmv(_experts_gemv_hidden(x, gate, up, topk_ids, n_mid), down, topk_ids, n_out)
 

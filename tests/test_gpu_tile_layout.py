@@ -303,3 +303,51 @@ def test_router_topk_into_wider_rows(ops):
     assert bool((ids[:, 8] == 256).all()) and bool((wts[:, 8] == 1.0).all())
     with pytest.raises(ValueError):
         ops.router_topk(lg, 8, out=(wts[:, :4].contiguous(), ids[:, :4].contiguous()))
+
+
+@pytest.mark.parametrize("T,E,k,extra", [(1, 256, 8, 1), (4, 256, 8, 1), (16, 256, 8, 1), (7, 64, 4, 0), (16, 1000, 64, 0),
+                                         (3, 300, 8, 3), (17, 256, 8, 1)])
+def test_router_topk_and_routing_lists_in_one_launch(ops, oracle, T, E, k, extra, monkeypatch):
+    """router_topk_routes against router_topk followed by mm_ids_route, and the lists against the oracle's: bit for
+    bit, with stacked always-on experts in the columns behind the k routed ones, logits with ties, a token that names an
+    expert twice (the last slot counts) and, above 16 tokens, the two-launch form it falls back to."""
+    monkeypatch.setattr(ops, "TOPK_ROUTE_ONE_LAUNCH_TOKENS", 16)  # every size the kernel takes
+    g = torch.Generator().manual_seed(T * 1000 + E)
+    lg = torch.randn((T, E), generator=g).cuda()
+    lg[:, : E // 4] = lg[:, : E // 4].round()  # ties
+    n_listed, n_slots = E + extra, k + extra
+
+    def rows():
+        wts = torch.full((T, n_slots), 1.0, device="cuda")
+        ids = torch.full((T, n_slots), 0, dtype=torch.int32, device="cuda")
+        for j in range(extra):
+            ids[:, k + j] = E + j
+        if extra >= 3:
+            ids[:, k + 2] = E + 1  # slot k + 2 names the expert of slot k + 1 again
+        return wts, ids
+
+    def listed(ids, bounds):
+        """positions of the lists that hold entries (a token naming an expert twice leaves a gap behind its list)"""
+        ids, bounds = ids.cpu().numpy(), bounds.cpu().numpy()
+        pos = [bounds[e] + j for e in range(n_listed) for j in range(int((ids == e).any(axis=1).sum()))]
+        return torch.tensor(pos, dtype=torch.long, device="cuda")
+
+    w1, i1, (s1, d1, b1) = ops.router_topk_routes(lg, k, n_listed, out=rows())
+    w2, i2 = ops.router_topk(lg, k, out=rows())
+    s2, d2, b2 = ops.mm_ids_route(i2, n_listed, False)
+    assert torch.equal(i1, i2) and torch.equal(w1, w2)
+    at = listed(i2, b2)
+    assert len(at) == T * (n_slots - (extra >= 3))
+    assert torch.equal(b1, b2) and torch.equal(s1[at], s2[at]) and torch.equal(d1[at], d2[at])
+    os1, od, ob = oracle.route(i2.cpu().numpy(), n_listed, nchannels_y=1, sis1=1)
+    assert np.array_equal(ob, b1.cpu().numpy()) and np.array_equal(od[at.cpu().numpy()], d1[at].cpu().numpy())
+    assert np.array_equal(os1[at.cpu().numpy()], s1[at].cpu().numpy())
+    if extra == 0:  # dense rows of k
+        w3, i3, (s3, d3, b3) = ops.router_topk_routes(lg, k, n_listed)
+        assert torch.equal(i3, i2) and torch.equal(b3, b2) and torch.equal(d3, d2)
+    # a second call with other logits
+    lg2 = torch.randn((T, E), generator=g).cuda()
+    _, i4, (s4, d4, b4) = ops.router_topk_routes(lg2, k, n_listed, out=rows())
+    s5, d5, b5 = ops.mm_ids_route(i4, n_listed, False)
+    at = listed(i4, b5)
+    assert torch.equal(b4, b5) and torch.equal(d4[at], d5[at]) and torch.equal(s4[at], s5[at])

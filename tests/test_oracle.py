@@ -258,6 +258,10 @@ def test_swiglu_combine_route_router(oracle):
     assert [int(v) for v in src1] == [t * k + s for _, t, s in pairs]
     assert [int(v) for v in oracle.route(ids, E, 1, 1)[0]] == [t for _, t, _ in pairs]  # one row per token
     assert [int(v) for v in bounds] == [sum(1 for e, _, _ in pairs if e < b) for b in range(E + 1)]
+    # a token that names an expert twice: the last slot is listed, and later lists start behind every naming
+    # (mmid_helper.cu:66-71 counts namings, not list entries), worked by hand for ids [[0, 0], [1, 2]]
+    _, dst2, bounds2 = oracle.route(np.array([[0, 0], [1, 2]], dtype=np.int32), 3, 2, 2)
+    assert [int(v) for v in bounds2] == [0, 2, 3, 4] and [int(dst2[j]) for j in (0, 2, 3)] == [1, 2, 3]
     # router: closed forms only (no reference counterpart)
     lg = rng.standard_normal(256).astype(np.float32)
     rid, rw = oracle.router_topk(lg, 8)
