@@ -481,12 +481,16 @@ __device__ __forceinline__ void ks_items(const bf16n_weight & w, const bf16n_wei
     // blocks, fewer than IPB to a block if need be: a block's wavefronts share its SIMDs, and the decode is VALU work
     // (33 active experts: 2 or 3 items on each of 256 CUs instead of 4 on 132 of them).  Else IPB per block, in rounds.
     const int64_t per_round = (int64_t) gridDim.x * IPB;
-    const bool dealt = n_items <= per_round - gridDim.x; // (only where that lowers the most items of a block)
-    for (int64_t r0 = 0; r0 < n_items; r0 += per_round) {
+    // More items than one round holds: dealt out evenly as well, every block taking its share IPB at a time, so that
+    // the last round has a few items on every CU rather than full blocks on a few CUs.
+    const bool dealt = n_items <= per_round - gridDim.x || n_items > per_round; // (only where that lowers the most items of a block)
+    const int first = (int) ((int64_t) blockIdx.x * n_items / gridDim.x);
+    const int share = (int) ((int64_t) (blockIdx.x + 1) * n_items / gridDim.x) - first;
+    for (int64_t r0 = 0, r = 0; r0 < n_items; r0 += per_round, r++) {
         int base, cnt;
         if (dealt) {
-            base = (int) ((int64_t) blockIdx.x * n_items / gridDim.x);
-            cnt = (int) ((int64_t) (blockIdx.x + 1) * n_items / gridDim.x) - base;
+            base = first + (int) r * IPB;
+            cnt = share - (int) r * IPB < IPB ? share - (int) r * IPB : IPB;
         } else {
             base = (int) (r0 + (int64_t) blockIdx.x * IPB);
             cnt = n_items - base < IPB ? n_items - base : IPB;
@@ -888,17 +892,21 @@ void mt_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & 
     }
 }
 
-// Passes of 32 tokens.  While the experts that can be active are few enough that K may be split over wavefronts
-// (k_mm_tile_ks: one block per CU, the split chosen on the device from the experts that are active), that kernel; else
-// whole experts (or 32 row groups) per block of sixteen wavefronts with the activations staged in LDS.  The estimate of
-// the active experts is the expectation for uniform routing; when it is too low the K-split kernel runs unsplit, which
-// measured up to a quarter behind the staged kernel at 32 tokens, and never runs a second round of blocks.
+// Passes of 32 tokens.  While the experts that can be active give at most a round of items to the kernel that may
+// split K over wavefronts (k_mm_tile_ks: one block per CU, the split chosen on the device from the experts that are
+// active), that kernel; else whole experts (or 32 row groups) per block of sixteen wavefronts with the activations
+// staged in LDS, which keeps only as many CUs busy as experts are active.  The estimate of the active experts is the
+// expectation for uniform routing; when it is too low the K-split kernel runs further rounds, dealt out evenly.
 void mt_launch_small(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int64_t n_pairs, int cus, hipStream_t stream) {
     const int slabs = (int) (w.K / TILE_K), groups = (int) (a.rows / TILE_R);
     const double e = (double) a.n_experts;
     const double active = std::min((double) n_pairs, e * (1.0 - std::pow(1.0 - 1.0 / e, (double) n_pairs)));
     const double items = active * (up ? groups : (groups + 1) / 2);
-    const bool split = a.bounds && a.n_experts <= MT_MAX_LISTED && slabs % 2 == 0 && items * 2 <= (double) cus * KS_WAVES;
+    // (a product without the fusion has short items, K / 256 = 2 tiles in the MoE down product, and runs a second
+    // round of them well: 130 / 159 / 203 / 227 active experts of 256 took 56 / 60 / 74 / 85 us against 70 / 74 / 80 /
+    // 84 us of the staged kernel; the fused gate / up product at one wavefront per item is level with it beyond a round)
+    const double rounds = up ? 1.0 : 1.5;
+    const bool split = a.bounds && a.n_experts <= MT_MAX_LISTED && slabs % 2 == 0 && items <= rounds * (double) cus * KS_WAVES;
     if (split) {
         if (up) {
             hipLaunchKernelGGL((k_mm_tile_ks<true>), dim3((unsigned) cus), dim3(KS_WAVES * 64), ks_shm(true), stream, w, *up, a);

@@ -257,13 +257,16 @@ def test_full_size_batched_moe_against_exact_weights_and_the_gemv_path(ops, expe
     assert torch.equal(ys2, ys * 2)
 
 
-@pytest.mark.parametrize("T,distinct", [(1, False), (2, False), (4, False), (8, False), (16, False), (20, True)])
+@pytest.mark.parametrize("T,distinct", [(1, False), (2, False), (4, False), (8, False), (16, False), (20, True), (28, False),
+                                        (30, True)])
 def test_batched_kernels_at_every_split_of_k(ops, experts, T, distinct):
     """Few tokens through the batched kernels: the kernel that splits K over wavefronts picks its split on the device
     from the experts that are active — 8 wavefronts per item for 8 to 32 experts (an expert's K is 8 tiles), 4 up to
     64, 2 up to 128, and whole chains when the routing has more active experts than the host's estimate (20 tokens whose
-    160 experts are all different: the estimate for uniform routing is 119).  Every (token, slot) output of the fused
-    gate/up product and of the down product against FP64 products of the exact weights."""
+    160 experts are all different: the estimate for uniform routing is 119).  More than 128 active experts give the down
+    product (32 items per expert) more items than the launch holds at once: a second round, dealt out evenly over the
+    blocks (28 tokens; 30 tokens whose 240 experts are all different).  Every (token, slot) output of the fused gate/up
+    product and of the down product against FP64 products of the exact weights."""
     (wg, gate), (wu, up), (wd, down) = experts
     g = torch.Generator(device="cuda").manual_seed(300 + T)
     x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
