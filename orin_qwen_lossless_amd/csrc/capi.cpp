@@ -259,7 +259,7 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
             require(dev::w64_mmv_supported(*w, a->x_bf16 != 0), "no wave64 GEMV kernel for this K / R (K in {512, 1024, 2048, 4096})");
             dev::launch_w64_mmv(*w, p, a->ncols, a->x_bf16 != 0, multi_col != 0, g_cus, (hipStream_t) stream);
         } else {
-            dev::launch_compat_mmv(*w, nullptr, 0, p, a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
+            dev::launch_compat_mmv(*w, nullptr, 0, p, a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream, multi_col != 0);
         }
         launch_check("mmv");
     });
@@ -280,6 +280,11 @@ int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
             // a large matrix in wave64 units: two launches of eight columns per decode (2 x 302 us on 248320 x 2048)
             // still beat writing and re-reading the whole matrix as BF16 (dequant + GEMM: 820 us)
             *out = 16;
+        } else if (w->format == FMT_NIBBLE) {
+            // the 4-bit code has no decode chain: batches go through the matrix cores, 32 tokens per decode of the
+            // matrix (5120 x 2048: 11-13 us up to 32 tokens, 20 us up to 64, where dequant + GEMM takes 20-21 us;
+            // 2048 x 4096: 17-21 us against 22-28 us)
+            *out = 64;
         } else {
             *out = 8;
         }

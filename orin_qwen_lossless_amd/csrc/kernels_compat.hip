@@ -15,6 +15,7 @@ namespace dev {
 namespace {
 
 constexpr int NT = 256;          // threads per block
+constexpr int NIB_MM_MIN_COLS = 5; // dense NIBBLE batches of BF16 columns go through the matrix cores from this many on at the earliest
 constexpr int HALVES = NT / 32;  // units (rows) per block
 
 template <typename TX>
@@ -365,6 +366,109 @@ __global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16
     }
 }
 
+// Dense NIBBLE products through the matrix cores: y[t] = W x[t] for BF16 token columns, 32 per block (gridDim.y blocks
+// of tokens; columns past the last repeat it and are not stored).  The 4-bit code has no decode chain, so one decode of
+// the matrix serves 32 tokens at the cost of one.  A block is one group of 32 rows with K / 256 wavefronts; wavefront v
+// takes half a chunk: the slots [16 (v & 1), +16) of chunk v / 2.  Lane (row r, half h) decodes two adjacent slots of
+// its row per step, 16 (v & 1) + 4n + 2h and the next (n = 0..3): 32 weights, which are eight adjacent columns
+// 128 j + 64 (v & 1) + 16 n + 8 h + [0, 8) in each of the chunk's four column blocks j — the A operands of four matrix
+// instructions (k positions 8h + [0, 8) of instruction j) — and lane (token t, half h) supplies the same columns of its
+// token's activations as B operands, one 16-byte load each: which columns an instruction's k positions stand for is
+// free as long as both operands agree.  (The activations staged through LDS by loads that take a token's 128 bytes
+// with eight adjacent lanes measured the same for K = 2048 and, in two turns of eight wavefronts, slower for K = 4096:
+// a launch is a few serial latencies, not the rate of its loads.)  BF16 products are exact in FP32; the partial sums of
+// the wavefronts are added in K order through LDS, the products of escaped weights (decoded as +0) last, and the sum
+// is rounded once.
+typedef __bf16 nm_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float nm_f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t nm_u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int NM_WAVES = 8; // per block: K / 256 half chunks in one turn each, K > 2048 in two
+
+// TURNS: half chunks per wavefront (wavefront v takes v TURNS + [0, TURNS)).  Every load of a wavefront is issued before
+// the first is used: a launch is a few serial latencies long, and eight wavefronts per block leave the registers for it.
+template <int TURNS>
+__global__ void __launch_bounds__(NM_WAVES * 64) k_nib_mm(const bf16n_weight w, const cols p, const int ncols) {
+    extern __shared__ __align__(16) float nm_part[]; // [wavefront][accumulator register][lane]
+    const nib_ptrs q = nibp(w, 0);
+    const int K = (int) w.K;
+    const int lane = threadIdx.x & 63, r = lane & 31, h = lane >> 5, wave = (int) (threadIdx.x >> 6), n_waves = (int) (blockDim.x >> 6);
+    const int64_t g0 = (int64_t) blockIdx.x * 32;
+    const int64_t row = p.row0 + (g0 + r < p.nrows ? g0 + r : p.nrows - 1);
+    const int t0 = (int) blockIdx.y * 32;
+    const char * x = p.x + (int64_t) (t0 + r < ncols ? t0 + r : ncols - 1) * p.x_tok;
+    const uint4 T = *(const uint4 *) (q.table + row * 16);
+    // the sums this thread finishes at the end are (token, row) = (e / 32, e % 32) for e = thread, thread + block size:
+    // one row (the block size is a multiple of 32), whose escape range is requested now
+    const int64_t my_row = g0 + (threadIdx.x & 31);
+    const int64_t my_gr = p.row0 + (my_row < p.nrows ? my_row : p.nrows - 1);
+    const uint32_t esc0 = q.esc_off[my_gr], esc1 = q.esc_off[my_gr + 1];
+    uint4 sm0[TURNS][4], sm1[TURNS][4], cdv[TURNS][4], b[TURNS][4][4];
+#pragma unroll
+    for (int turn = 0; turn < TURNS; turn++) {
+        // a last wavefront with a half chunk too few (K / 256 odd) repeats its first
+        const int hc = (wave * TURNS + turn) * 256 < K ? wave * TURNS + turn : wave * TURNS;
+        const int c = hc >> 1, s0 = 16 * (hc & 1) + 2 * h; // this lane's first slot
+        const uint8_t * pl = q.plane + row * K + c * CHUNK + 16 * s0;
+        const uint8_t * cd = q.codes + row * (K / 2) + c * (CHUNK / 2) + 8 * s0;
+        const char * xb = x + 2 * (c * CHUNK + 4 * s0);
+#pragma unroll
+        for (int n = 0; n < 4; n++) {
+            sm0[turn][n] = *(const uint4 *) (pl + 64 * n);
+            sm1[turn][n] = *(const uint4 *) (pl + 64 * n + 16);
+            cdv[turn][n] = *(const uint4 *) (cd + 32 * n);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                b[turn][n][j] = *(const uint4 *) (xb + 32 * n + 256 * j);
+            }
+        }
+    }
+    nm_f32x16_t acc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        acc[i] = 0.f;
+    }
+#pragma unroll
+    for (int turn = 0; turn < TURNS; turn++) {
+        if ((wave * TURNS + turn) * 256 < K) {
+#pragma unroll
+            for (int n = 0; n < 4; n++) {
+                uint32_t w0[8], w1[8];
+                nib_chunk(sm0[turn][n], make_uint2(cdv[turn][n].x, cdv[turn][n].y), T, w0);
+                nib_chunk(sm1[turn][n], make_uint2(cdv[turn][n].z, cdv[turn][n].w), T, w1);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const nm_u32x4_t a = {w0[2 * j], w0[2 * j + 1], w1[2 * j], w1[2 * j + 1]};
+                    const nm_u32x4_t bv = {b[turn][n][j].x, b[turn][n][j].y, b[turn][n][j].z, b[turn][n][j].w};
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(nm_bf16x8_t, a), __builtin_bit_cast(nm_bf16x8_t, bv), acc, 0, 0, 0);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        nm_part[(wave * 16 + i) * 64 + lane] = acc[i];
+    }
+    __syncthreads();
+    // accumulator register i of lane l: row 8 (i / 4) + 4 (l / 32) + i % 4 of the group, token l % 32.  A thread per
+    // (token, row), rows adjacent in a wavefront: a token's 32 outputs are stored side by side.
+    for (int e = (int) threadIdx.x; e < 1024; e += (int) blockDim.x) {
+        const int tok = e >> 5, rr = e & 31;
+        const int i = 4 * (rr >> 3) + (rr & 3), l = tok + 32 * ((rr >> 2) & 1);
+        float v = 0.f;
+        for (int k = 0; k < n_waves; k++) {
+            v += nm_part[(k * 16 + i) * 64 + l];
+        }
+        if (g0 + rr < p.nrows && t0 + tok < ncols) {
+            const char * xt = p.x + (int64_t) (t0 + tok) * p.x_tok;
+            for (uint32_t k = esc0; k < esc1; k++) {
+                const uint32_t rec = q.esc[k];
+                v = fmaf(bf16_bits_to_f32(esc_bits(rec)), x_at<bf16_t>(xt, (int) (rec & 0xFFFu)), v);
+            }
+            store_y(p.y + (int64_t) (t0 + tok) * p.y_tok, p.y_bf16, g0 + rr, v);
+        }
+    }
+}
+
 // exact rows of a NIBBLE matrix: FP32 or BF16, to out + i * stride (bytes); row index from ids (gather) or row0 + i
 template <bool BF>
 __global__ void __launch_bounds__(NT) k_nib_rows(const bf16n_weight w, const char * __restrict__ ids, int64_t ids_s0, int64_t n,
@@ -421,10 +525,26 @@ int grid_for(int64_t work, int ncols, int cus) {
 } // namespace
 
 void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,
-                       int cus, hipStream_t stream) {
+                       int cus, hipStream_t stream, bool matrix_cores) {
     const bf16n_weight & wu = up ? *up : w;
     const int64_t work = w.format == FMT_NIBBLE ? p.nrows : p.nrows / w.R;
     const dim3 grid(grid_for(work, ncols, cus), ncols);
+    // the matrix cores from nine BF16 columns on, and from five where the row groups give at least half of the CUs a
+    // block (5120 x 2048: 11.0-13.0 us for 5-32 columns against 9.6 / 17.9 us for 4 / 8 GEMV columns and 20 us for
+    // dequant + GEMM; 2048 x 4096, 64 blocks: 18.3-22.8 us against 8.6 / 15.4 us and 24-28 us)
+    const int64_t nm_blocks = (p.nrows + 31) / 32;
+    if (matrix_cores && w.format == FMT_NIBBLE && !p.ids && glu == 0 && x_bf16 && w.K % CHUNK == 0 && w.K / 256 <= 2 * NM_WAVES &&
+        (ncols > 8 || (ncols >= NIB_MM_MIN_COLS && nm_blocks * 2 >= cus)) && ((uintptr_t) p.x & 15) == 0 && p.x_tok % 16 == 0) {
+        const int halves = (int) (w.K / 256), turns = halves > NM_WAVES ? 2 : 1, waves = (halves + turns - 1) / turns;
+        const dim3 grid((unsigned) nm_blocks, (unsigned) ((ncols + 31) / 32));
+        const size_t shm = (size_t) waves * 16 * 64 * sizeof(float);
+        if (turns == 2) {
+            hipLaunchKernelGGL(k_nib_mm<2>, grid, dim3(waves * 64), shm, stream, w, p, ncols);
+        } else {
+            hipLaunchKernelGGL(k_nib_mm<1>, grid, dim3(waves * 64), shm, stream, w, p, ncols);
+        }
+        return;
+    }
     if (w.format == FMT_NIBBLE) {
         const int rpb = HALVES / (int) (w.K / CHUNK);
         // dense batches: four (two) columns share one decode of the matrix once there are columns enough to keep at

@@ -13,7 +13,7 @@ namespace dev {
 
 // 32-lane layouts (kernels_compat.hip). glu: 0 plain, 1 merged [gate; up] NIBBLE matrix, 2 separate gate / up matrices
 void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,
-                       int cus, hipStream_t stream);
+                       int cus, hipStream_t stream, bool matrix_cores = true);
 void launch_compat_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream);
 void launch_compat_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
                             int64_t dst_s1, int64_t row0, hipStream_t stream);

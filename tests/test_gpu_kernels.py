@@ -55,9 +55,9 @@ def test_gemv_dense(ops, oracle, K, fmt, R, cm, w64):
     assert np.array_equal(bits(y16), rne_bf16(y_bf))
     # multi-column launches give each column the single-column result
     y1 = np.stack([ops.mmv(tbf16(xb[t: t + 1]), w).cpu().numpy()[0] for t in range(3)])
-    assert np.array_equal(y1, y_bf)
     y_sc = ops.mmv(tbf16(xb), w, multi_col=False).cpu().numpy()
-    assert np.array_equal(y_sc, y_bf)
+    assert np.array_equal(y_sc, y1)
+    assert np.array_equal(y1, y_bf)
 
 
 @pytest.mark.parametrize("K", [512, 1024, 2048, 4096])
@@ -87,6 +87,8 @@ def test_wave64_column_groups_equal_single_columns(ops, oracle, K, R):
 def test_nibble_column_groups_equal_single_columns(ops, oracle, K):
     # dense NIBBLE batches of 8 and more columns decode a (row, chunk) once for two or four columns; every column keeps
     # the bits of its single-column launch, plain and with the fused SwiGLU, BF16 and FP32 activations, ragged tails
+    # (the plain product of BF16 activations runs on the matrix cores from nine columns on: the same bits at every
+    # such batch size, within the oracle's bounds)
     rows = 2 * 88
     wb = synth.weights(rows, K, 5 * K)
     wb[3, 7] = 0x4000                                          # 2.0: an exponent outside the row table, an escape
@@ -97,8 +99,10 @@ def test_nibble_column_groups_equal_single_columns(ops, oracle, K):
         y1 = torch.cat([ops.mmv(x[t: t + 1], w) for t in range(19)])
         g1 = torch.cat([ops.mmv_glu(x[t: t + 1], w) for t in range(19)])
         check_gemv(oracle, y1[:4].cpu().numpy(), wb, xf[:4])
+        y19 = ops.mmv(x, w)
+        check_gemv(oracle, y19[[0, 7, 18]].cpu().numpy(), wb, xf[[0, 7, 18]])
         for T in (8, 9, 15, 16, 17, 19):
-            assert torch.equal(ops.mmv(x[:T], w), y1[:T]), (T, x.dtype)
+            assert torch.equal(ops.mmv(x[:T], w), y1[:T] if x.dtype == torch.float32 or T <= 8 else y19[:T]), (T, x.dtype)
             assert torch.equal(ops.mmv_glu(x[:T], w), g1[:T]), (T, x.dtype)
 
 
