@@ -146,6 +146,8 @@ __device__ __forceinline__ void tile_step_mm(tchain_t<D, ONCE> * ch, const uint3
 
 constexpr int MT_SMALL_PAIRS = 16;  // routed pairs per expert up to which the 32-token shape is used
 constexpr int MT_MAX_LISTED = 1024; // experts up to which a block lists the active ones
+constexpr int MT_MAX_UNITS = 2 * MT_MAX_LISTED; // listed (expert, pass of 32 tokens) units: one per active expert and one
+                                                // more per 32 routed pairs, of which the 32-token shape takes 16 per expert
 constexpr int MT_HK = 128;         // activation columns staged at a time (half a tile)
 constexpr int MT_BSTRIDE = 136;    // BF16 elements per staged token row: 272 bytes spread 16 lanes over all banks
 
@@ -215,22 +217,34 @@ struct mm_args {
     int n_experts, n_tok;
 };
 
-// The experts that have tokens, in order, listed in LDS (act[MT_MAX_LISTED]: their number, which is returned): the
-// blocks share out the work items of these only, so that a call with few active experts keeps its blocks equally loaded
-// instead of leaving some with several items and others with none.  Every wavefront of the block takes 64 experts at
-// a time (one read of their bounds for the whole block), the counts meet in LDS behind the list.  Ends with a barrier.
-// span (optional, [MT_MAX_LISTED]): first routed pair and number of pairs of every listed expert, so that the items need
-// not read the bounds again.
-__device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, int wave, int lane, int n_waves, int2 * span = nullptr) {
-    int * cnt = (int *) (act + MT_MAX_LISTED + 8); // [n_waves], n_waves <= 16
+// The work of a call with routing lists, listed in LDS: one unit per active expert and pass of 32 of its tokens, in
+// expert order (unit[MT_MAX_UNITS]: expert | pass << 16; their number is returned).  The blocks share out the work
+// items of these only, so that a call with few active experts keeps its blocks equally loaded instead of leaving some
+// with several items and others with none, and the passes of an expert with more than 32 tokens (one that every token
+// uses, say) run side by side on different blocks instead of one after the other on one.  Every wavefront of the block
+// takes 64 experts at a time (one read of their bounds for the whole block), the counts meet in LDS behind the list.
+// Ends with a barrier.  span (optional, [MT_MAX_UNITS]): first routed pair and number of pairs of every unit.
+__device__ __forceinline__ int list_units(uint32_t * unit, const mm_args & a, int wave, int lane, int n_waves, int2 * span = nullptr) {
+    int * cnt = (int *) (unit + MT_MAX_UNITS); // [n_waves], n_waves <= 16
     int total = 0;
     for (int e0 = 0; e0 < a.n_experts; e0 += 64 * n_waves) {
         const int e = e0 + 64 * wave + lane;
         const int b0 = e < a.n_experts ? a.bounds[e] : 0, b1 = e < a.n_experts ? a.bounds[e + 1] : 0;
-        const bool on = b1 > b0;
-        const uint64_t m = __ballot(on);
-        if (lane == 0) {
-            cnt[wave] = __builtin_popcountll(m);
+        const int np = b1 > b0 ? (b1 - b0 + 31) >> 5 : 0;
+        int scan; // inclusive prefix of the passes over the lanes
+        if (__ballot(np > 1) == 0) { // (nearly always: no expert of these 64 has more than 32 tokens)
+            const uint64_t m = __ballot(np > 0);
+            scan = (int) __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u)) + np;
+        } else {
+            scan = np;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(scan, o, 64);
+                scan += lane >= o ? up : 0;
+            }
+        }
+        if (lane == 63) {
+            cnt[wave] = scan;
         }
         __syncthreads();
         int before = total, all = 0;
@@ -239,17 +253,17 @@ __device__ __forceinline__ int list_active(uint16_t * act, const mm_args & a, in
             before += k < wave ? c : 0;
             all += c;
         }
-        if (on) {
-            const int at = before + (int) __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u));
-            act[at] = (uint16_t) e;
+        const int at = before + scan - np;
+        for (int k = 0; k < np && at + k < MT_MAX_UNITS; k++) {
+            unit[at + k] = (uint32_t) e | ((uint32_t) k << 16);
             if (span) {
-                span[at] = make_int2(b0, b1 - b0);
+                span[at + k] = make_int2(b0 + 32 * k, b1 - b0 - 32 * k < 32 ? b1 - b0 - 32 * k : 32);
             }
         }
         total += all;
         __syncthreads();
     }
-    return (int) uniform((uint32_t) total);
+    return (int) uniform((uint32_t) (total < MT_MAX_UNITS ? total : MT_MAX_UNITS));
 }
 
 // A work item is (expert, slab of row groups): every wavefront owns two decode chains, gate and up of one row group
@@ -281,15 +295,18 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
     // this thread's share of a staged block: CPT columns of one token (NT = 1: the upper wavefronts stage nothing)
     const bool stager = S::STAGERS == S::THREADS || wave < S::STAGERS / 64;
     const int b_tok = stager ? tid / S::TPT : 0, b_part = tid % S::TPT;
-    uint16_t * act = (uint16_t *) (bbuf + 2 * S::TOK * MT_BSTRIDE);
+    uint32_t * unit = (uint32_t *) (bbuf + 2 * S::TOK * MT_BSTRIDE);
     // (passes of 128 tokens are for calls with many tokens per expert: every expert is active)
     const bool listed = NT == 1 && a.bounds != nullptr && a.n_experts <= MT_MAX_LISTED;
-    const int n_act = listed ? list_active(act, a, wave, lane, S::WAVES) : a.n_experts;
+    const int n_act = listed ? list_units(unit, a, wave, lane, S::WAVES) : a.n_experts;
     __syncthreads();
     for (int item = blockIdx.x; item < n_act * slabs_per_expert; item += gridDim.x) {
         // (read from LDS: the same in every lane, and kept in a scalar register like the arithmetic form)
-        const int e = listed ? (int) uniform(act[item / slabs_per_expert]) : item / slabs_per_expert, sl = item % slabs_per_expert;
-        const int j0 = a.bounds ? a.bounds[e] : 0, n = a.bounds ? a.bounds[e + 1] - j0 : a.n_tok;
+        const uint32_t un = listed ? uniform(unit[item / slabs_per_expert]) : (uint32_t) (item / slabs_per_expert);
+        const int e = listed ? (int) (un & 0xFFFFu) : (int) un, sl = item % slabs_per_expert;
+        // a listed unit is one pass of 32 tokens of its expert
+        const int first = a.bounds ? a.bounds[e] : 0, j0 = listed ? first + 32 * (int) (un >> 16) : first;
+        const int left_e = a.bounds ? a.bounds[e + 1] - j0 : a.n_tok, n = listed && left_e > 32 ? 32 : left_e;
         // this wavefront's row groups (inside the expert); a missing second group repeats the first and is dropped
         const int g0 = GLU ? sl * GPI + wave : sl * GPI + 2 * wave;
         const bool live = g0 < groups, has1 = GLU || g0 + 1 < groups;
@@ -461,7 +478,7 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
 constexpr int KS_WAVES = 16;
 
 struct ks_ctx {
-    uint32_t * lut, * rings; uint16_t * act; const int2 * span;
+    uint32_t * lut, * rings, * unit; const int2 * span;
     int n_items, per_expert, groups, slabs;
 };
 
@@ -471,7 +488,7 @@ __device__ __forceinline__ void ks_items(const bf16n_weight & w, const bf16n_wei
     uint32_t * lut = c.lut;
     uint32_t * rings = c.rings;
     float * part = (float *) rings;                           // [wavefront][register][lane], 6 KB apart
-    uint16_t * act = c.act;
+    const uint32_t * unit = c.unit;
     const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
     const int is = wave / WPI, kw = wave % WPI;               // item of the block, K part
     const int groups = c.groups, per_expert = c.per_expert, n_items = c.n_items, spw = c.slabs / WPI;
@@ -509,7 +526,7 @@ __device__ __forceinline__ void ks_items(const bf16n_weight & w, const bf16n_wei
         const int item = base + is;
         const bool valid = is < cnt;
         const int at = valid ? item / per_expert : 0, p = valid ? item % per_expert : 0;
-        const int e = (int) uniform(act[at]);
+        const int e = (int) (uniform(unit[at]) & 0xFFFFu);
         const int j0 = (int) uniform((uint32_t) c.span[at].x), n = valid ? (int) uniform((uint32_t) c.span[at].y) : 0;
         const int g0 = GLU ? p : 2 * p;
         const bool has1 = GLU || g0 + 1 < groups;
@@ -609,8 +626,8 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     ks_ctx c;
     c.lut = shm;
     c.rings = shm + NM * LUT_WORDS;
-    c.act = (uint16_t *) (c.rings + KS_WAVES * 2 * WAVE_LDS_WORDS);
-    int2 * span = (int2 *) (c.act + MT_MAX_LISTED + 8 + 2 * 16); // behind the list and its 16 counters
+    c.unit = c.rings + KS_WAVES * 2 * WAVE_LDS_WORDS;
+    int2 * span = (int2 *) (c.unit + MT_MAX_UNITS + 16); // behind the list and its 16 counters
     c.span = span;
     const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6);
     // the tables are requested first (one 16-byte load per thread and table) and stored once the block knows that it
@@ -621,7 +638,7 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     c.groups = (int) (a.rows / TILE_R);
     c.per_expert = GLU ? c.groups : (c.groups + 1) / 2;       // items per expert
     c.slabs = (int) (w.K / TILE_K);
-    c.n_items = list_active(c.act, a, wave, lane, KS_WAVES, span) * c.per_expert;
+    c.n_items = list_units(c.unit, a, wave, lane, KS_WAVES, span) * c.per_expert;
     // the most wavefronts per item for which the launch's blocks hold every item at once
     int wpi = KS_WAVES;
     while (wpi > 1 && (c.slabs % wpi != 0 || (int64_t) c.n_items * wpi > (int64_t) gridDim.x * KS_WAVES)) {
@@ -647,14 +664,14 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
 }
 
 size_t ks_shm(bool glu) { // tables, rings, list of active experts + counters, their spans
-    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_LISTED + 8) * 2 + 16 * 4 +
-           (size_t) MT_MAX_LISTED * 8;
+    return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_UNITS + 16) * 4 +
+           (size_t) MT_MAX_UNITS * 8;
 }
 
 template <int NT, int W> size_t mt_shm(bool glu) {
     using S = mt_shape<NT, W>;
     return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) S::WAVES * 2 * WAVE_LDS_WORDS * 4 + (size_t) 2 * S::TOK * MT_BSTRIDE * 2 +
-           (MT_MAX_LISTED + 8) * 2 + 16 * 4;
+           (MT_MAX_UNITS + 16) * 4;
 }
 
 // ---------------------------------------------------------------- GEMV
@@ -904,8 +921,9 @@ void mt_launch_small(const bf16n_weight & w, const bf16n_weight * up, const mm_a
     const double items = active * (up ? groups : (groups + 1) / 2);
     // (a product without the fusion has short items, K / 256 = 2 tiles in the MoE down product, and runs a second
     // round of them well: 130 / 159 / 203 / 227 active experts of 256 took 56 / 60 / 74 / 85 us against 70 / 74 / 80 /
-    // 84 us of the staged kernel; the fused gate / up product at one wavefront per item is level with it beyond a round)
-    const double rounds = up ? 1.0 : 1.5;
+    // 84 us of the staged kernel; the fused gate / up product at one wavefront per item, eight tiles per chain, is ahead
+    // of it up to two thirds of a round, level at 0.8 and far behind at 0.9: 107 / 294 us at 173 / 230 active experts)
+    const double rounds = up ? 0.75 : 1.5;
     const bool split = a.bounds && a.n_experts <= MT_MAX_LISTED && slabs % 2 == 0 && items <= rounds * (double) cus * KS_WAVES;
     if (split) {
         if (up) {

@@ -258,22 +258,28 @@ def test_full_size_batched_moe_against_exact_weights_and_the_gemv_path(ops, expe
 
 
 @pytest.mark.parametrize("T,distinct", [(1, False), (2, False), (4, False), (8, False), (16, False), (20, True), (28, False),
-                                        (30, True)])
+                                        (30, True), (40, "popular"), (70, "popular")])
 def test_batched_kernels_at_every_split_of_k(ops, experts, T, distinct):
     """Few tokens through the batched kernels: the kernel that splits K over wavefronts picks its split on the device
     from the experts that are active — 8 wavefronts per item for 8 to 32 experts (an expert's K is 8 tiles), 4 up to
     64, 2 up to 128, and whole chains when the routing has more active experts than the host's estimate (20 tokens whose
     160 experts are all different: the estimate for uniform routing is 119).  More than 128 active experts give the down
     product (32 items per expert) more items than the launch holds at once: a second round, dealt out evenly over the
-    blocks (28 tokens; 30 tokens whose 240 experts are all different).  Every (token, slot) output of the fused gate/up
-    product and of the down product against FP64 products of the exact weights."""
+    blocks (28 tokens; 30 tokens whose 240 experts are all different).  An expert that every token uses has more than
+    the 32 tokens of a pass: its passes are listed as work of their own and run on different blocks (40 and 70 tokens:
+    two and three passes, the last one ragged).  Every (token, slot) output of the fused gate/up product and of the
+    down product against FP64 products of the exact weights."""
     (wg, gate), (wu, up), (wd, down) = experts
     g = torch.Generator(device="cuda").manual_seed(300 + T)
     x = torch.randn((T, K), generator=g, device="cuda").to(torch.bfloat16)
-    if distinct:
+    if distinct is True:
         ids = torch.randperm(E, generator=g, device="cuda")[: T * TOPK].to(torch.int32).view(T, TOPK).contiguous()
     else:
-        _, ids = ops.router_topk(torch.randn((T, E), generator=g, device="cuda"), TOPK)
+        logits = torch.randn((T, E), generator=g, device="cuda")
+        if distinct == "popular":
+            logits[:, 7] = 50.0  # every token's first choice
+        _, ids = ops.router_topk(logits, TOPK)
+        assert distinct != "popular" or bool((ids[:, 0] == 7).all())
     src1, dst, bounds = ops.mm_ids_route(ids, E, False)
     a = ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.float32, routes=(src1, dst, bounds))
     a16 = a.to(torch.bfloat16)
@@ -461,10 +467,14 @@ def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, mode, wan
     assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y4))
 
 
-@pytest.mark.parametrize("rows,k", [(5120, 2048), (2048, 4096)])
-def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, rows, k):
-    """A 4-bit matrix large enough to fill the GPU with one column decodes a (row, chunk) once for 2 or 4 columns of a
-    batch: every column of every batch size up to 9 has the bits of its single-column product, escapes included."""
+@pytest.mark.parametrize("rows,k", [(5120, 2048), (2048, 4096), (1000, 512)])
+def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, oracle, rows, k):
+    """Dense batches on a 4-bit matrix, escapes included.  Few BF16 columns (and FP32 columns) share decodes on the VALU
+    and have the bits of their single-column products.  From nine BF16 columns on — from five where the matrix has row
+    groups for half of the CUs — the product runs on the matrix cores, 32 tokens per decode: there a column has the same
+    bits at every batch size and at every position (a token's sum never meets another token's), within the FP64 bound
+    of the GEMV.  Rows that are no multiple of 32 and batches that are no multiple of 32 tokens leave a ragged last
+    block."""
     from orin_qwen_lossless_amd import synth
 
     wb = synth.weights(rows, k, 900 + rows % 89)
@@ -473,14 +483,27 @@ def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, rows, k):
     assert fmt == 1
     ta = torch.from_numpy(aux)
     enc = ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
-    xb = synth.activations(9, k, 78)
+    xb = synth.activations(70, k, 78)
     x = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16).cuda()
     single = torch.cat([ops.mmv(x[t: t + 1], enc) for t in range(9)])
-    for T in (2, 3, 4, 5, 8, 9):
-        assert torch.equal(ops.mmv(x[:T], enc), single[:T]), T
-    xf = x.float()
+    first = 5 if (rows + 31) // 32 * 2 >= torch.cuda.get_device_properties(0).multi_processor_count else 9
+    y70 = ops.mmv(x, enc)
+    for T in (2, 3, 4, 5, 8, 9, 31, 32, 33, 64):
+        assert torch.equal(ops.mmv(x[:T], enc), single[:T] if T < first else y70[:T]), T
+    assert torch.equal(ops.mmv(x[37:50], enc), y70[37:50])  # other positions in the block of 32
+    assert not torch.equal(y70[:9], single)                 # (the two paths do differ: another order of summation)
+    y70n = y70.cpu().numpy()
+    for t in (0, 2, 31, 32, 69):
+        y64, bound = oracle.gemv_f64(wb, synth.bf16_bits_to_f32(xb[t]))
+        assert np.all(np.abs(y70n[t] - y64) <= 1e-5 * bound), t
+        if t < 9:
+            assert np.all(np.abs(single[t].cpu().numpy() - y64) <= 1e-5 * bound), t
+    # BF16 out: the one rounding of the FP32 sums
+    y16 = ops.mmv(x[:12], enc, out_dtype=torch.bfloat16)
+    assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y70n[:12]))
+    xf = x[:4].float()
     single_f = torch.cat([ops.mmv(xf[t: t + 1], enc) for t in range(4)])
-    assert torch.equal(ops.mmv(xf[:4], enc), single_f)
+    assert torch.equal(ops.mmv(xf, enc), single_f)
 
 
 # ---- the decode step (40 x [qkv, o, router, top-8, 256 experts + shared, glue]): two layers of it at real size ------------
