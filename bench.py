@@ -207,7 +207,7 @@ def cpu_baseline(wbits, K: int, xf, sample_rows: int, budget_s: float):
 
 # ---------------------------------------------------------------- the other configurations of the path
 
-def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4), n_layers: int = 40, n_sets: int = 4) -> dict:
+def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4, 16), n_layers: int = 40, n_sets: int = 4) -> dict:
     """The 40-layer decode step as one HIP graph on BF16N weights and on uncompressed BF16 weights with stock kernels
     (orin_qwen_lossless_amd/decode_step.py), output projection included.  n_sets distinct weight sets are used in turn;
     every layer's input is the previous layer's output, so layers that share a set route to other experts."""
@@ -240,12 +240,14 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4), n_laye
             entry[name] = float(np.median(time_kernel(replay, 12, 3))) * 1e3
             del graph
         touched = n_layers * D.layer_bytes(nbytes, T) + head_bytes
+        expected = n_layers * D.layer_bytes(nbytes, T, expected=True) + head_bytes  # (the rates below: on these)
         bf16_bytes = 2 * (n_layers * (sum(r * k for n_, (r, k, m) in D.SHAPES.items() if m == 1)
                                       + (min(T * D.TOPK, D.E) + 1) * 3 * D.N_MID * K) + head_bf16.numel())
         t = entry["bf16n"]
         gemv_path = T * (D.TOPK + 1) <= max(ops.MOE_GEMV_MIN_PAIRS, ops.MOE_GEMV_PAIRS_PER_EXPERT[0] * D.EA)
-        res[f"batch{T}"] = {"us": round(t, 1), "launches_per_layer": 8 if gemv_path or T <= ops.TOPK_ROUTE_ONE_LAUNCH_TOKENS else 9, "compressed_bytes_touched_upper_bound": int(touched), "GBps": round(touched / t / 1e3, 1),
-                            "frac_of_hbm_peak": round(touched / t / 1e3 / HBM_PEAK_GBS, 4), "tokens_per_s": round(T / t * 1e6, 1),
+        res[f"batch{T}"] = {"us": round(t, 1), "launches_per_layer": 8 if gemv_path or T <= ops.TOPK_ROUTE_ONE_LAUNCH_TOKENS else 9, "compressed_bytes_touched_upper_bound": int(touched),
+                            "compressed_bytes_touched_expected": int(expected), "GBps": round(expected / t / 1e3, 1),
+                            "frac_of_hbm_peak": round(expected / t / 1e3 / HBM_PEAK_GBS, 4), "tokens_per_s": round(T / t * 1e6, 1),
                             "bf16_us": round(entry["bf16"], 1), "speedup_vs_bf16": round(entry["bf16"] / t, 2),
                             "bf16_bytes_touched": int(bf16_bytes), "bf16_us_at_hbm_peak": round(bf16_bytes / HBM_PEAK_GBS / 1e3, 1),
                             "eager_equals_graph": True}

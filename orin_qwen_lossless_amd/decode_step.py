@@ -53,11 +53,13 @@ def make_layer_sets(ops, gen_weights, n_sets: int, keep_bf16: bool):
     return enc_sets, raw_sets, nbytes
 
 
-def layer_bytes(nbytes: dict, tokens: int) -> int:
-    """Compressed bytes one layer touches for `tokens` tokens (upper bound: every token picks other experts)."""
-    experts = min(tokens * TOPK, E) + 1  # + the shared expert
+def layer_bytes(nbytes: dict, tokens: int, expected: bool = False) -> int:
+    """Compressed bytes one layer touches for `tokens` tokens: the upper bound (every token picks other experts), or the
+    expectation for uniform routing (tokens share experts: 102 distinct ones of 256 for 16 tokens' 128 picks)."""
+    routed = E * (1.0 - (1.0 - TOPK / E) ** tokens) if expected else min(tokens * TOPK, E)
+    experts = routed + 1  # + the shared expert
     dense = sum(nbytes[k] for k in ("qkv", "o", "router"))
-    return dense + (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * experts // EA
+    return dense + int((nbytes["gate"] + nbytes["up"] + nbytes["down"]) * experts) // EA
 
 
 def routing_buffers(n_tok: int, device) -> tuple[torch.Tensor, torch.Tensor]:

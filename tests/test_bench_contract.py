@@ -55,7 +55,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     for key in ("lm_head_batch4", "gemv_512x2048", "gemv_2048x512", "moe_layer_batch1_graph", "moe_prefill_T2048", "moe_prefill_T8192",
                 "decode_step"):
         assert key in cf, key
-    for b in ("batch1", "batch4"):
+    for b in ("batch1", "batch4", "batch16"):
         e = cf["decode_step"][b]
         assert e["us"] > 0 and e["bf16_us"] > 0 and e["eager_equals_graph"] and 0 < e["frac_of_hbm_peak"] < 1
         assert abs(e["speedup_vs_bf16"] - e["bf16_us"] / e["us"]) < 0.02
