@@ -251,6 +251,26 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4, 16), n_
                             "bf16_us": round(entry["bf16"], 1), "speedup_vs_bf16": round(entry["bf16"] / t, 2),
                             "bf16_bytes_touched": int(bf16_bytes), "bf16_us_at_hbm_peak": round(bf16_bytes / HBM_PEAK_GBS / 1e3, 1),
                             "eager_equals_graph": True}
+    # the same step with the expert stacks in the 4-bit code (the policy's nibble mode for them): no decode chain
+    # in the routed GEMVs, 7 % more expert bytes
+    sets4, _, nbytes4 = D.make_layer_sets(ops, gen, n_sets, False, expert_mode="nibble")
+    res["experts_4bit_code"] = {"expert_bytes_vs_tiles": round(nbytes4["gate"] / nbytes["gate"], 4)}
+    for T in (1, 4):
+        xin = [synth.activations_torch(T, K, 300 + i, "cuda") for i in range(4)]
+        hbuf = xin[0].clone()
+        graph, _ = D.capture(D.Bf16nStep(ops, sets4, head, n_layers, T), hbuf)
+
+        def replay4(i):
+            hbuf.copy_(xin[i & 3])
+            graph.replay()
+
+        t = float(np.median(time_kernel(replay4, 12, 3))) * 1e3
+        expected = n_layers * D.layer_bytes(nbytes4, T, expected=True) + head_bytes
+        res["experts_4bit_code"][f"batch{T}"] = {"us": round(t, 1), "vs_policy_layout": round(res[f"batch{T}"]["us"] / t, 3),
+                                                   "compressed_bytes_touched_expected": int(expected),
+                                                   "frac_of_hbm_peak": round(expected / t / 1e3 / HBM_PEAK_GBS, 4)}
+        del graph
+    del sets4
     res["layer_sets"] = sets
     res["nbytes"] = nbytes
     return res

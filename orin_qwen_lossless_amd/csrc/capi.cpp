@@ -418,7 +418,10 @@ int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x
         require(x_bf16 && dst && ids_src1 && ids_dst && bounds, "null pointer");
         require(((uintptr_t) x_bf16 & 15) == 0 && x_row % 8 == 0, "activations must be 16-byte aligned with 16-byte row strides");
         require(((uintptr_t) dst & 15) == 0 && dst_col % 4 == 0, "dst must be 16-byte aligned with a column stride that is a multiple of 4");
-        if (dev::is_tile_layout(*w)) {
+        if (w->format == FMT_NIBBLE) {
+            dev::launch_nib_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts,
+                                   (int64_t) n_tok * n_used, g_cus, (hipStream_t) stream);
+        } else if (dev::is_tile_layout(*w)) {
             dev::launch_tile_mm_ids(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts,
                                     (int64_t) n_tok * n_used, g_cus, (hipStream_t) stream);
         } else {
@@ -455,7 +458,10 @@ int bf16n_moe_mm_ids_static(const bf16n_weight * w, const bf16n_weight * up, con
         dev::launch_route(ids, ids_i64 != 0, ids_row_stride, r->src1, r->dst, r->bounds, n_experts, n_tok, n_used, nch, nch,
                           (hipStream_t) stream);
         launch_check("mm_ids_route");
-        if (dev::is_tile_layout(*w)) {
+        if (w->format == FMT_NIBBLE) {
+            dev::launch_nib_mm_ids(*w, up, x_bf16, x_row, r->src1, r->dst, r->bounds, dst, dst_bf16 != 0, dst_col, n_experts,
+                                   (int64_t) n_tok * n_used, g_cus, (hipStream_t) stream);
+        } else if (dev::is_tile_layout(*w)) {
             dev::launch_tile_mm_ids(*w, up, x_bf16, x_row, r->src1, r->dst, r->bounds, dst, dst_bf16 != 0, dst_col, n_experts,
                                     (int64_t) n_tok * n_used, g_cus, (hipStream_t) stream);
         } else {

@@ -195,33 +195,6 @@ __global__ void __launch_bounds__(NT) k_hp_get_rows(const bf16n_weight w, const 
 
 // ---------------------------------------------------------------- NIBBLE
 
-// 4 exponents of 4 adjacent columns from 4 nibble codes (16 bits) and the row's 16-byte table, as bytes e0..e3
-__device__ __forceinline__ uint32_t nib_lookup4(const uint4 T, uint32_t codes16) {
-    uint32_t s = (codes16 | (codes16 << 8)) & 0x00FF00FFu;
-    s = (s | (s << 4)) & 0x0F0F0F0Fu; // one code per byte
-    const uint32_t lo = __builtin_amdgcn_perm(T.y, T.x, s & 0x07070707u);
-    const uint32_t hi = __builtin_amdgcn_perm(T.w, T.z, s & 0x07070707u);
-    const uint32_t pick_hi = ((s >> 3) & 0x01010101u) * 0xFFu;
-    return (hi & pick_hi) | (lo & ~pick_hi);
-}
-
-// the 16 weights of one lane in one NIBBLE chunk
-__device__ __forceinline__ void nib_chunk(const uint4 sm, const uint2 cd, const uint4 T, uint32_t (&wp)[8]) {
-    const uint32_t smw[4] = {sm.x, sm.y, sm.z, sm.w};
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const uint32_t c16 = ((j & 2) ? cd.y : cd.x) >> ((j & 1) * 16) & 0xFFFFu;
-        const uint32_t e4 = nib_lookup4(T, c16);
-        wp[2 * j] = merge(spread_lo(smw[j]), __builtin_amdgcn_perm(0, e4, 0x0c010c00u) << 7);
-        wp[2 * j + 1] = merge(spread_hi(smw[j]), __builtin_amdgcn_perm(0, e4, 0x0c030c02u) << 7);
-    }
-}
-
-__device__ __forceinline__ uint32_t esc_bits(uint32_t rec) { // BF16 bits of an escape record col | sm << 12 | exponent << 20
-    const uint32_t smb = (rec >> 12) & 0xFFu, ex = rec >> 20;
-    return ((smb & 0x80u) << 8) | (ex << 7) | (smb & 0x7Fu);
-}
-
 // the 16 activations one lane meets in a 512-column chunk (columns 128 j + 4 l + 0..3), as FP32
 template <typename TX>
 __device__ __forceinline__ void x_chunk16(const char * x, int col0, float (&xv)[16]);

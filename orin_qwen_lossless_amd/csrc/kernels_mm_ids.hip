@@ -416,6 +416,9 @@ void mm_ids_init() {
 // the reference's rule (launch.cu:446-456) restated for the layouts this build encodes: gate / up in chunk-major
 // R = 8 units of K = 2048 (alone or fused with SwiGLU), down in row-major R = 16 units of K = 512
 bool mm_ids_shape_ok(const bf16n_weight & w, const bf16n_weight * up) {
+    if (w.format == FMT_NIBBLE) { // kernels_tile.hip: experts in the 4-bit code
+        return nib_mm_ids_ok(w, up);
+    }
     if (is_tile_layout(w)) { // kernels_tile.hip: any K, gate / up of the same shape
         return !up || (is_tile_layout(*up) && up->rows == w.rows && up->K == w.K);
     }

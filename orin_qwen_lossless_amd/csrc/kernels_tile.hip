@@ -11,6 +11,7 @@
 //     one row over the whole tile, so a tile ends with one cross-half add instead of a reduction per row.
 //   * k_tile_dequant, k_tile_get_rows: exact BF16 rows (launch.cu:367-443).
 #include "dev_common.h"
+#include "dev_compat.h"
 #include "dev_w64.h"
 #include "launchers.h"
 
@@ -224,15 +225,16 @@ struct mm_args {
 // uses, say) run side by side on different blocks instead of one after the other on one.  Every wavefront of the block
 // takes 64 experts at a time (one read of their bounds for the whole block), the counts meet in LDS behind the list.
 // Ends with a barrier.  span (optional, [MT_MAX_UNITS]): first routed pair and number of pairs of every unit.
+template <int TOK = 32>
 __device__ __forceinline__ int list_units(uint32_t * unit, const mm_args & a, int wave, int lane, int n_waves, int2 * span = nullptr) {
     int * cnt = (int *) (unit + MT_MAX_UNITS); // [n_waves], n_waves <= 16
     int total = 0;
     for (int e0 = 0; e0 < a.n_experts; e0 += 64 * n_waves) {
         const int e = e0 + 64 * wave + lane;
         const int b0 = e < a.n_experts ? a.bounds[e] : 0, b1 = e < a.n_experts ? a.bounds[e + 1] : 0;
-        const int np = b1 > b0 ? (b1 - b0 + 31) >> 5 : 0;
+        const int np = b1 > b0 ? (b1 - b0 + TOK - 1) / TOK : 0;
         int scan; // inclusive prefix of the passes over the lanes
-        if (__ballot(np > 1) == 0) { // (nearly always: no expert of these 64 has more than 32 tokens)
+        if (__ballot(np > 1) == 0) { // (nearly always: no expert of these 64 has more than a pass of tokens)
             const uint64_t m = __ballot(np > 0);
             scan = (int) __builtin_amdgcn_mbcnt_hi((uint32_t) (m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t) m, 0u)) + np;
         } else {
@@ -257,7 +259,7 @@ __device__ __forceinline__ int list_units(uint32_t * unit, const mm_args & a, in
         for (int k = 0; k < np && at + k < MT_MAX_UNITS; k++) {
             unit[at + k] = (uint32_t) e | ((uint32_t) k << 16);
             if (span) {
-                span[at + k] = make_int2(b0 + 32 * k, b1 - b0 - 32 * k < 32 ? b1 - b0 - 32 * k : 32);
+                span[at + k] = make_int2(b0 + TOK * k, b1 - b0 - TOK * k < TOK ? b1 - b0 - TOK * k : TOK);
             }
         }
         total += all;
@@ -663,6 +665,213 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
     }
 }
 
+// ---------------------------------------------------------------- batched products of experts in the 4-bit code
+//
+// Experts stored in the reference's NIBBLE layout (rows of all experts stacked) have no decode chain: a wavefront decodes
+// any 32 rows x 256 columns it likes, which makes the batched product a plain tiled one.  A block of eight wavefronts
+// takes a work item (expert, pass of 32 NT of its tokens, slab of row groups: eight groups with the fused gate / up
+// product, sixteen without) and walks K in half chunks of 256 columns.  Wavefront v owns one row group of gate and the
+// same of up (or two row groups of the matrix) and their 2 x NT accumulator blocks; per step lane (row r, half h)
+// decodes two adjacent slots of its row in each matrix — eight adjacent columns in each of the chunk's four column
+// blocks, the A operands of four matrix instructions (k_nib_mm explains the order) — and the B operands come from the
+// pass's activations of these 256 columns, staged in LDS by the whole block (double buffered: one barrier per half
+// chunk) in a token-major layout padded so that sixteen tokens meet all banks.  No table and no ring in LDS, so the
+// staged activations may take it all.  Escaped weights (decoded as +0) add their exact products before the SwiGLU.
+constexpr int NB_WAVES = 8;
+constexpr int NB_PAIRS_32 = 12, NB_PAIRS_64 = 40; // routed pairs per expert up to which passes are 32 / 64 tokens long
+constexpr int NB_TOK_BYTES = 4 * 128 + 16; // a staged token: four runs of 64 columns, padded
+template <int NT> constexpr int nb_stage_bytes() { return 32 * NT * NB_TOK_BYTES; }
+template <int NT> size_t nb_shm() { return (size_t) 2 * nb_stage_bytes<NT>() + (size_t) 32 * NT * 4 + (MT_MAX_UNITS + 16) * 4; }
+
+template <bool GLU, int NT>
+__global__ void __launch_bounds__(NB_WAVES * 64, NT == 1 ? 2 : 1) k_nib_mm_ids(const bf16n_weight w, const bf16n_weight w_up, const mm_args a) {
+    constexpr int TOK = 32 * NT, STAGE = nb_stage_bytes<NT>();
+    constexpr int GPI = GLU ? NB_WAVES : 2 * NB_WAVES; // row groups per work item
+    constexpr int SV = TOK * 32 / (NB_WAVES * 64);      // uint4 a thread stages per half chunk: 32 per token
+    constexpr int AHEAD = NT == 4 ? 1 : 2;              // steps the weight loads run ahead (registers: 24 per step)
+    extern __shared__ __align__(16) char nb_lds[];
+    char * stage = nb_lds;                              // [2][TOK][NB_TOK_BYTES]
+    int * tok_row = (int *) (nb_lds + 2 * STAGE);       // [TOK]: the activation row of every token of the pass
+    uint32_t * unit = (uint32_t *) (tok_row + TOK);
+    const nib_ptrs q0 = nibp(w, 0), q1 = nibp(GLU ? w_up : w, 0);
+    const int K = (int) w.K, halves = K / 256;
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, h = lane >> 5, wave = (int) uniform(tid >> 6);
+    const int groups = (int) (a.rows / 32), slabs = (groups + GPI - 1) / GPI;
+    const int n_units = list_units<TOK>(unit, a, wave, lane, NB_WAVES);
+    for (int item = blockIdx.x; item < n_units * slabs; item += gridDim.x) {
+        const uint32_t un = uniform(unit[item / slabs]);
+        const int e = (int) (un & 0xFFFFu), sl = item % slabs;
+        const int j0 = a.bounds[e] + TOK * (int) (un >> 16);
+        const int left = a.bounds[e + 1] - j0, n = left < TOK ? left : TOK, nt = (n + 31) >> 5;
+        __syncthreads(); // the item before is done with tok_row and the staging buffers
+        if (tid < TOK) {
+            tok_row[tid] = a.ids_src1[j0 + (tid < n ? tid : n - 1)];
+        }
+        __syncthreads();
+        const int g0 = GLU ? sl * GPI + wave : sl * GPI + 2 * wave;
+        const bool live = g0 < groups, has1 = GLU || g0 + 1 < groups;
+        const int g1 = GLU || !has1 ? g0 : g0 + 1;
+        const int64_t row0 = (int64_t) e * a.rows + (live ? g0 : 0) * 32 + r, row1 = (int64_t) e * a.rows + (live ? g1 : 0) * 32 + r;
+        const uint4 T0 = *(const uint4 *) (q0.table + row0 * 16), T1 = *(const uint4 *) (q1.table + row1 * 16);
+        const uint8_t * pl0 = q0.plane + row0 * K + 32 * h, * pl1 = q1.plane + row1 * K + 32 * h;
+        const uint8_t * cd0 = q0.codes + row0 * (K / 2) + 16 * h, * cd1 = q1.codes + row1 * (K / 2) + 16 * h;
+        // staging: uint4 v of this thread is part (index % 8) of column block (index / 8 % 4) of token index / 32
+        const char * sx[SV];
+        int so[SV];
+#pragma unroll
+        for (int v = 0; v < SV; v++) {
+            const int idx = tid + NB_WAVES * 64 * v, tok = idx >> 5, jb = (idx >> 3) & 3, part = idx & 7;
+            sx[v] = (const char *) (a.x + (int64_t) tok_row[tok] * a.x_row) + 256 * jb + 16 * part;
+            so[v] = tok * NB_TOK_BYTES + 128 * jb + 16 * part;
+        }
+        f32x16_t acc[2][NT];
+#pragma unroll
+        for (int m = 0; m < 2; m++) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    acc[m][t][i] = 0.f;
+                }
+            }
+        }
+        // the weights of the first steps (a step's: two slots of 16 plane bytes and their 16 code bytes, per matrix)
+        uint4 pa[AHEAD][6];
+#pragma unroll
+        for (int q = 0; q < AHEAD; q++) {
+            pa[q][0] = *(const uint4 *) (pl0 + 64 * q);
+            pa[q][1] = *(const uint4 *) (pl0 + 64 * q + 16);
+            pa[q][2] = *(const uint4 *) (cd0 + 32 * q);
+            pa[q][3] = *(const uint4 *) (pl1 + 64 * q);
+            pa[q][4] = *(const uint4 *) (pl1 + 64 * q + 16);
+            pa[q][5] = *(const uint4 *) (cd1 + 32 * q);
+        }
+        {   // the first half chunk's activations
+            uint4 f[SV];
+#pragma unroll
+            for (int v = 0; v < SV; v++) {
+                f[v] = *(const uint4 *) sx[v];
+            }
+#pragma unroll
+            for (int v = 0; v < SV; v++) {
+                *(uint4 *) (stage + so[v]) = f[v];
+            }
+        }
+        __syncthreads();
+#pragma unroll 1
+        for (int hc = 0; hc < halves; hc++) {
+            const char * bcur = stage + (hc & 1) * STAGE;
+            // the next half chunk's activations: requested now, stored after this one's steps (after the last half
+            // chunk the same one again, into the buffer nobody reads any more)
+            const int nx = hc + 1 < halves ? hc + 1 : hc;
+            uint4 f[SV];
+#pragma unroll
+            for (int v = 0; v < SV; v++) {
+                f[v] = *(const uint4 *) (sx[v] + 2 * ((nx >> 1) * 512 + 64 * (nx & 1)));
+            }
+            if (live) {
+#pragma unroll
+                for (int s4 = 0; s4 < 4; s4++) {
+                    // step q = 4 hc + s4 takes the plane bytes [64 q, +64) and the code bytes [32 q, +32) of the row (two
+                    // lanes); its loads were issued AHEAD steps ago, and those of step q + AHEAD go out now
+                    const int q = 4 * hc + s4;
+                    const uint4 c00 = pa[s4 % AHEAD][0], c01 = pa[s4 % AHEAD][1], ck0 = pa[s4 % AHEAD][2];
+                    const uint4 c10 = pa[s4 % AHEAD][3], c11 = pa[s4 % AHEAD][4], ck1 = pa[s4 % AHEAD][5];
+                    const int qn = q + AHEAD < 4 * halves ? q + AHEAD : q; // past the end: this step's again, unused
+                    pa[s4 % AHEAD][0] = *(const uint4 *) (pl0 + 64 * qn);
+                    pa[s4 % AHEAD][1] = *(const uint4 *) (pl0 + 64 * qn + 16);
+                    pa[s4 % AHEAD][2] = *(const uint4 *) (cd0 + 32 * qn);
+                    pa[s4 % AHEAD][3] = *(const uint4 *) (pl1 + 64 * qn);
+                    pa[s4 % AHEAD][4] = *(const uint4 *) (pl1 + 64 * qn + 16);
+                    pa[s4 % AHEAD][5] = *(const uint4 *) (cd1 + 32 * qn);
+                    uint32_t wa[2][8], wb[2][8]; // [matrix]: the lane's first and second slot
+                    nib_chunk(c00, make_uint2(ck0.x, ck0.y), T0, wa[0]);
+                    nib_chunk(c01, make_uint2(ck0.z, ck0.w), T0, wb[0]);
+                    nib_chunk(c10, make_uint2(ck1.x, ck1.y), T1, wa[1]);
+                    nib_chunk(c11, make_uint2(ck1.z, ck1.w), T1, wb[1]);
+#pragma unroll
+                    for (int jb = 0; jb < 4; jb++) {
+                        const u32x4_t a0 = {wa[0][2 * jb], wa[0][2 * jb + 1], wb[0][2 * jb], wb[0][2 * jb + 1]};
+                        const u32x4_t a1 = {wa[1][2 * jb], wa[1][2 * jb + 1], wb[1][2 * jb], wb[1][2 * jb + 1]};
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            if (t == 0 || t < nt) {
+                                const bf16x8_t bv = *(const bf16x8_t *) (bcur + (32 * t + r) * NB_TOK_BYTES + 128 * jb + 32 * s4 + 16 * h);
+                                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), bv, acc[0][t], 0, 0, 0);
+                                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), bv, acc[1][t], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+            }
+            char * bn = stage + ((hc + 1) & 1) * STAGE;
+#pragma unroll
+            for (int v = 0; v < SV; v++) {
+                *(uint4 *) (bn + so[v]) = f[v];
+            }
+            __syncthreads();
+        }
+        if (!live) {
+            continue;
+        }
+        // the exact products of escaped weights; accumulator element i of a lane: row 8 (i / 4) + 4 h + i % 4, token 32 t + r
+#pragma unroll
+        for (int m = 0; m < 2; m++) {
+            const nib_ptrs & q = m ? q1 : q0;
+            const int64_t gr0 = (int64_t) e * a.rows + (m && !GLU ? g1 : g0) * 32;
+            if (uniform(q.esc_off[gr0 + 32] - q.esc_off[gr0]) == 0) {
+                continue;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int64_t gr = gr0 + 8 * (i >> 2) + 4 * h + (i & 3);
+                for (uint32_t k = q.esc_off[gr]; k < q.esc_off[gr + 1]; k++) {
+                    const uint32_t rec = q.esc[k];
+                    const float wv = bf16_bits_to_f32(esc_bits(rec));
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        if (t < nt) {
+                            const uint16_t xv = a.x[(int64_t) tok_row[32 * t + r] * a.x_row + (rec & 0xFFFu)];
+                            acc[m][t][i] = fmaf(wv, bf16_bits_to_f32(xv), acc[m][t][i]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int tk = 32 * t + r;
+            if (t < nt && tk < n) {
+                const int64_t col = (int64_t) a.ids_dst[j0 + tk] * a.dst_col;
+#pragma unroll
+                for (int m = 0; m < (GLU ? 1 : 2); m++) {
+                    if (m == 1 && !has1) {
+                        continue;
+                    }
+                    const int64_t rbase = (int64_t) (m ? g1 : g0) * 32 + 4 * h;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        float v[4];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const float pv = acc[m][t][4 * g + i];
+                            v[i] = GLU ? acc[1][t][4 * g + i] * silu(pv) : pv;
+                        }
+                        const int64_t o = col + rbase + 8 * g;
+                        if (a.dst_bf16) {
+                            *(uint2 *) ((uint16_t *) a.dst + o) =
+                                make_uint2(f32_to_bf16_rne(v[0]) | ((uint32_t) f32_to_bf16_rne(v[1]) << 16),
+                                           f32_to_bf16_rne(v[2]) | ((uint32_t) f32_to_bf16_rne(v[3]) << 16));
+                        } else {
+                            *(float4 *) ((float *) a.dst + o) = make_float4(v[0], v[1], v[2], v[3]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 size_t ks_shm(bool glu) { // tables, rings, list of active experts + counters, their spans
     return (size_t) (glu ? 2 : 1) * LUT_WORDS * 4 + (size_t) KS_WAVES * 2 * WAVE_LDS_WORDS * 4 + (MT_MAX_UNITS + 16) * 4 +
            (size_t) MT_MAX_UNITS * 8;
@@ -883,7 +1092,12 @@ void lds_attr(const void * kernel, size_t dynamic_bytes) {
 template <bool GLU, int NT, int W> void mt_attr() { lds_attr((const void *) k_mm_tile<GLU, NT, W>, mt_shm<NT, W>(GLU)); }
 template <bool GLU> void ks_attr() { lds_attr((const void *) k_mm_tile_ks<GLU>, ks_shm(GLU)); }
 
+template <bool GLU, int NT> void nb_attr() {
+    (void) hipFuncSetAttribute((const void *) k_nib_mm_ids<GLU, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) nb_shm<NT>());
+}
+
 void tile_init() {
+    nb_attr<true, 1>(); nb_attr<false, 1>(); nb_attr<true, 2>(); nb_attr<false, 2>(); nb_attr<true, 4>(); nb_attr<false, 4>();
     mt_attr<true, 4, 8>();
     mt_attr<false, 4, 8>();
     mt_attr<true, 1, 16>();
@@ -953,6 +1167,45 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
         mt_launch_small(w, up, a, n_pairs, cus, stream);
     } else {
         mt_launch<4, 8>(w, up, a, cus, stream);
+    }
+}
+
+// Experts in the 4-bit code (NIBBLE, the rows of all experts stacked): passes of 32, 64 or 128 tokens by the routed pairs
+// per expert; blocks stay on their CU and take items in turn (how many there are is known on the device only).
+bool nib_mm_ids_ok(const bf16n_weight & w, const bf16n_weight * up) {
+    return w.format == FMT_NIBBLE && w.K % 512 == 0 && (!up || (up->format == FMT_NIBBLE && up->rows == w.rows && up->K == w.K));
+}
+
+template <int NT>
+void nb_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int cus, hipStream_t stream) {
+    const int per_cu = (int) (160 * 1024 / nb_shm<NT>()) < 3 ? (int) (160 * 1024 / nb_shm<NT>()) : 3;
+    const dim3 grid((unsigned) (cus * (per_cu < 1 ? 1 : per_cu)));
+    if (up) {
+        hipLaunchKernelGGL((k_nib_mm_ids<true, NT>), grid, dim3(NB_WAVES * 64), nb_shm<NT>(), stream, w, *up, a);
+    } else {
+        hipLaunchKernelGGL((k_nib_mm_ids<false, NT>), grid, dim3(NB_WAVES * 64), nb_shm<NT>(), stream, w, w, a);
+    }
+}
+
+void launch_nib_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
+                       const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
+                       int64_t n_pairs, int cus, hipStream_t stream) {
+    mm_args a;
+    a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
+    a.ids_src1 = ids_src1; a.ids_dst = ids_dst; a.bounds = bounds;
+    a.dst = (char *) dst; a.dst_col = dst_col; a.dst_bf16 = dst_bf16;
+    a.rows = w.rows / n_experts; a.n_experts = n_experts; a.n_tok = 0;
+    if (a.rows % 32 != 0 || n_experts > MT_MAX_LISTED) {
+        throw std::invalid_argument("bf16n: batched 4-bit-code experts need rows per expert in multiples of 32 and at most 1024 experts");
+    }
+    // a pass decodes the expert's rows again: long passes where the experts have many tokens.  The units listed are at
+    // most one per expert and one per full pass: within MT_MAX_UNITS for up to 32 pairs per expert with the shortest.
+    if (n_pairs <= (int64_t) NB_PAIRS_32 * n_experts) {
+        nb_launch<1>(w, up, a, cus, stream);
+    } else if (n_pairs <= (int64_t) NB_PAIRS_64 * n_experts) {
+        nb_launch<2>(w, up, a, cus, stream);
+    } else {
+        nb_launch<4>(w, up, a, cus, stream);
     }
 }
 

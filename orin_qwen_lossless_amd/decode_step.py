@@ -26,25 +26,27 @@ SHAPES = {"qkv": (QKV_ROWS, K_MODEL, 1), "o": (K_MODEL, ATT, 1), "router": (E, K
           "up": (EA * N_MID, K_MODEL, EA), "down": (EA * K_MODEL, N_MID, EA)}
 
 
-def encode_policy(ops, w_dev: torch.Tensor, n_matrices: int = 1):
-    """[rows, K] BF16 device tensor -> (Weight in the layout of the mi355x policy, compressed bytes)."""
+def encode_policy(ops, w_dev: torch.Tensor, n_matrices: int = 1, mode: str = "hybrid"):
+    """[rows, K] BF16 device tensor -> (Weight in the layout of the mi355x policy, compressed bytes).  mode: the policy's
+    (hybrid, huffman or nibble: the 4-bit code for everything)."""
     rows, k = w_dev.shape
-    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, k, n_matrices, engine="mi355x", expert=n_matrices > 1)
+    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, k, n_matrices, engine="mi355x", mode=mode, expert=n_matrices > 1)
     bits = w_dev.cpu().view(torch.int16).numpy().view(np.uint16)
     plane, aux, _, _ = ops.encode_bits(bits, fmt, R, cm, wave64=w64)
     ta = torch.from_numpy(aux)
     return ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), w_dev.device), plane.size + aux.size
 
 
-def make_layer_sets(ops, gen_weights, n_sets: int, keep_bf16: bool):
+def make_layer_sets(ops, gen_weights, n_sets: int, keep_bf16: bool, expert_mode: str = "hybrid"):
     """n_sets weight sets of one layer.  gen_weights(rows, K) -> BF16 device tensor.  Returns (encoded sets, BF16 sets or
-    None, compressed bytes by matrix name of one set)."""
+    None, compressed bytes by matrix name of one set).  expert_mode "nibble": the expert stacks in the 4-bit code (7 %
+    more bytes than the policy's tiles, no decode chain: the form for decode at one or two tokens)."""
     enc_sets, raw_sets, nbytes = [], [] if keep_bf16 else None, {}
     for _ in range(n_sets):
         enc, raw = {}, {}
         for name, (rows, k, nm) in SHAPES.items():
             w = gen_weights(rows, k)
-            enc[name], nbytes[name] = encode_policy(ops, w, nm)
+            enc[name], nbytes[name] = encode_policy(ops, w, nm, expert_mode if nm > 1 else "hybrid")
             if keep_bf16:
                 raw[name] = w
         enc_sets.append(enc)

@@ -59,6 +59,8 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
         e = cf["decode_step"][b]
         assert e["us"] > 0 and e["bf16_us"] > 0 and e["eager_equals_graph"] and 0 < e["frac_of_hbm_peak"] < 1
         assert abs(e["speedup_vs_bf16"] - e["bf16_us"] / e["us"]) < 0.02
+    e4 = cf["decode_step"]["experts_4bit_code"]
+    assert e4["batch1"]["us"] > 0 and e4["batch4"]["us"] > 0 and 1.0 < e4["expert_bytes_vs_tiles"] < 1.2
     for T in (2048, 8192):
         e = cf[f"moe_prefill_T{T}"]
         assert 0 < e["frac_of_bf16_mfma_peak"] < 1 and e["weight_decode_GBps"] > 0
