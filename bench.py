@@ -125,7 +125,8 @@ def graph_us(fn, n: int = 16, reps: int = 30) -> float:
     return med_us(lambda i: graph.replay(), reps, 3) / n
 
 
-def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: str = "mi355x", matrix_core_order: bool = False):
+def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: str = "mi355x", matrix_core_order: bool = False,
+                     mode: str = "hybrid"):
     """Encode a [rows, K] BF16 device tensor under the mi355x policy (n_matrices stacked experts; matrix_core_order: the
     policy's dense_frag_order option) and upload `copies` copies; returns (list of weights, compressed bytes,
     description)."""
@@ -133,7 +134,7 @@ def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: s
     import torch
 
     rows, K = w_dev.shape
-    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, K, n_matrices, engine=engine, expert=n_matrices > 1,
+    fmt, R, cm, _, w64 = ops.choose(rows // n_matrices, K, n_matrices, engine=engine, mode=mode, expert=n_matrices > 1,
                                     dense_frag_order=matrix_core_order)
     wbits = w_dev.cpu().view(torch.int16).numpy().view(np.uint16)
     plane, aux, fmt_out, _ = ops.encode_bits(wbits, fmt, R, cm, wave64=w64)
@@ -376,7 +377,7 @@ def suite(ops, w_head, head_copies, K: int) -> dict:
     return {"lm_head_batches": {"tiles": tdesc, "tiles_bytes": tbytes, "by_batch": batches}}
 
 
-def prefill_only(T: int, steps: int) -> None:
+def prefill_only(T: int, steps: int, mode: str = "hybrid") -> None:
     """Only the batched MoE kernels of one 35B-A3B-shaped layer (256 experts x (gate, up 512 x 2048; down 2048 x 512),
     top-8, experts in the mi355x policy's layout) on T tokens: routing lists once, then fused gate/up + SwiGLU (BF16)
     and down, `steps` times.  For profiling these kernels alone; prints its own JSON line."""
@@ -387,9 +388,9 @@ def prefill_only(T: int, steps: int) -> None:
     torch.cuda.set_device(0)
     ops.init()
     E, topk, N, K = 256, 8, 512, 2048
-    (gate,), gb, gdesc = encode_to_device(ops, synth.weights_torch(E * N, K, 31, "cuda"), n_matrices=E)
-    (up,), ub, _ = encode_to_device(ops, synth.weights_torch(E * N, K, 32, "cuda"), n_matrices=E)
-    (down,), db, ddesc = encode_to_device(ops, synth.weights_torch(E * K, N, 33, "cuda"), n_matrices=E)
+    (gate,), gb, gdesc = encode_to_device(ops, synth.weights_torch(E * N, K, 31, "cuda"), n_matrices=E, mode=mode)
+    (up,), ub, _ = encode_to_device(ops, synth.weights_torch(E * N, K, 32, "cuda"), n_matrices=E, mode=mode)
+    (down,), db, ddesc = encode_to_device(ops, synth.weights_torch(E * K, N, 33, "cuda"), n_matrices=E, mode=mode)
     x = synth.activations_torch(T, K, 34, "cuda")
     _, ids = ops.router_topk(synth.normal_torch(T * E, 35, "cuda").view(T, E), topk)
     src1, dst, bounds = ops.mm_ids_route(ids, E, False)
@@ -454,13 +455,14 @@ def main() -> None:
     ap.add_argument("--suite", action="store_true", help="also sweep the output projection over batch sizes in both layouts")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="run only the batched MoE kernels of one layer on T tokens (for profiling) and exit")
+    ap.add_argument("--experts-4bit", action="store_true", help="with --prefill: the expert stacks in the 4-bit code (policy mode nibble)")
     ap.add_argument("--decode-step", type=int, default=0, metavar="T",
                     help="run only the 40-layer decode step at batch T (for profiling) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path has no collective); run with --gpus 1")
     if args.prefill > 0:
-        prefill_only(args.prefill, min(args.steps, 20))
+        prefill_only(args.prefill, min(args.steps, 20), "nibble" if args.experts_4bit else "hybrid")
         return
     if args.decode_step > 0:
         decode_only(args.decode_step, min(args.steps, 20))

@@ -673,7 +673,8 @@ __global__ void __launch_bounds__(KS_WAVES * 64) k_mm_tile_ks(const bf16n_weight
 // product, sixteen without) and walks K in half chunks of 256 columns.  Wavefront v owns one row group of gate and the
 // same of up (or two row groups of the matrix) and their 2 x NT accumulator blocks; per step lane (row r, half h)
 // decodes two adjacent slots of its row in each matrix — eight adjacent columns in each of the chunk's four column
-// blocks, the A operands of four matrix instructions (k_nib_mm explains the order) — and the B operands come from the
+// blocks, the A operands of four matrix instructions (k_nib_mm explains the order; here a lane owns four adjacent
+// slots, two steps' worth, so that a row's cache line is used up at once) — and the B operands come from the
 // pass's activations of these 256 columns, staged in LDS by the whole block (double buffered: one barrier per half
 // chunk) in a token-major layout padded so that sixteen tokens meet all banks.  No table and no ring in LDS, so the
 // staged activations may take it all.  Escaped weights (decoded as +0) add their exact products before the SwiGLU.
@@ -688,7 +689,6 @@ __global__ void __launch_bounds__(NB_WAVES * 64, NT == 1 ? 2 : 1) k_nib_mm_ids(c
     constexpr int TOK = 32 * NT, STAGE = nb_stage_bytes<NT>();
     constexpr int GPI = GLU ? NB_WAVES : 2 * NB_WAVES; // row groups per work item
     constexpr int SV = TOK * 32 / (NB_WAVES * 64);      // uint4 a thread stages per half chunk: 32 per token
-    constexpr int AHEAD = NT == 4 ? 1 : 2;              // steps the weight loads run ahead (registers: 24 per step)
     extern __shared__ __align__(16) char nb_lds[];
     char * stage = nb_lds;                              // [2][TOK][NB_TOK_BYTES]
     int * tok_row = (int *) (nb_lds + 2 * STAGE);       // [TOK]: the activation row of every token of the pass
@@ -713,8 +713,11 @@ __global__ void __launch_bounds__(NB_WAVES * 64, NT == 1 ? 2 : 1) k_nib_mm_ids(c
         const int g1 = GLU || !has1 ? g0 : g0 + 1;
         const int64_t row0 = (int64_t) e * a.rows + (live ? g0 : 0) * 32 + r, row1 = (int64_t) e * a.rows + (live ? g1 : 0) * 32 + r;
         const uint4 T0 = *(const uint4 *) (q0.table + row0 * 16), T1 = *(const uint4 *) (q1.table + row1 * 16);
-        const uint8_t * pl0 = q0.plane + row0 * K + 32 * h, * pl1 = q1.plane + row1 * K + 32 * h;
-        const uint8_t * cd0 = q0.codes + row0 * (K / 2) + 16 * h, * cd1 = q1.codes + row1 * (K / 2) + 16 * h;
+        // a lane takes four adjacent slots of its row at a time, 64 plane bytes and 32 code bytes, the two halves of a
+        // row's 128-byte line in the same load instructions: taken 32 bytes at a time, a step apart, every line came from
+        // HBM twice at 2,048 tokens (FETCH_SIZE 1.92 GB for 0.83 GB of weights: neither L1 nor L2 kept it that long)
+        const uint8_t * pl0 = q0.plane + row0 * K + 64 * h, * pl1 = q1.plane + row1 * K + 64 * h;
+        const uint8_t * cd0 = q0.codes + row0 * (K / 2) + 32 * h, * cd1 = q1.codes + row1 * (K / 2) + 32 * h;
         // staging: uint4 v of this thread is part (index % 8) of column block (index / 8 % 4) of token index / 32
         const char * sx[SV];
         int so[SV];
@@ -735,16 +738,17 @@ __global__ void __launch_bounds__(NB_WAVES * 64, NT == 1 ? 2 : 1) k_nib_mm_ids(c
                 }
             }
         }
-        // the weights of the first steps (a step's: two slots of 16 plane bytes and their 16 code bytes, per matrix)
-        uint4 pa[AHEAD][6];
+        // the weights of the first pair of steps: per matrix four slots of 16 plane bytes and their 32 code bytes
+        uint4 pa[12];
 #pragma unroll
-        for (int q = 0; q < AHEAD; q++) {
-            pa[q][0] = *(const uint4 *) (pl0 + 64 * q);
-            pa[q][1] = *(const uint4 *) (pl0 + 64 * q + 16);
-            pa[q][2] = *(const uint4 *) (cd0 + 32 * q);
-            pa[q][3] = *(const uint4 *) (pl1 + 64 * q);
-            pa[q][4] = *(const uint4 *) (pl1 + 64 * q + 16);
-            pa[q][5] = *(const uint4 *) (cd1 + 32 * q);
+        for (int k = 0; k < 4; k++) {
+            pa[k] = *(const uint4 *) (pl0 + 16 * k);
+            pa[6 + k] = *(const uint4 *) (pl1 + 16 * k);
+        }
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            pa[4 + k] = *(const uint4 *) (cd0 + 16 * k);
+            pa[10 + k] = *(const uint4 *) (cd1 + 16 * k);
         }
         {   // the first half chunk's activations
             uint4 f[SV];
@@ -771,34 +775,56 @@ __global__ void __launch_bounds__(NB_WAVES * 64, NT == 1 ? 2 : 1) k_nib_mm_ids(c
             }
             if (live) {
 #pragma unroll
-                for (int s4 = 0; s4 < 4; s4++) {
-                    // step q = 4 hc + s4 takes the plane bytes [64 q, +64) and the code bytes [32 q, +32) of the row (two
-                    // lanes); its loads were issued AHEAD steps ago, and those of step q + AHEAD go out now
-                    const int q = 4 * hc + s4;
-                    const uint4 c00 = pa[s4 % AHEAD][0], c01 = pa[s4 % AHEAD][1], ck0 = pa[s4 % AHEAD][2];
-                    const uint4 c10 = pa[s4 % AHEAD][3], c11 = pa[s4 % AHEAD][4], ck1 = pa[s4 % AHEAD][5];
-                    const int qn = q + AHEAD < 4 * halves ? q + AHEAD : q; // past the end: this step's again, unused
-                    pa[s4 % AHEAD][0] = *(const uint4 *) (pl0 + 64 * qn);
-                    pa[s4 % AHEAD][1] = *(const uint4 *) (pl0 + 64 * qn + 16);
-                    pa[s4 % AHEAD][2] = *(const uint4 *) (cd0 + 32 * qn);
-                    pa[s4 % AHEAD][3] = *(const uint4 *) (pl1 + 64 * qn);
-                    pa[s4 % AHEAD][4] = *(const uint4 *) (pl1 + 64 * qn + 16);
-                    pa[s4 % AHEAD][5] = *(const uint4 *) (cd1 + 32 * qn);
-                    uint32_t wa[2][8], wb[2][8]; // [matrix]: the lane's first and second slot
-                    nib_chunk(c00, make_uint2(ck0.x, ck0.y), T0, wa[0]);
-                    nib_chunk(c01, make_uint2(ck0.z, ck0.w), T0, wb[0]);
-                    nib_chunk(c10, make_uint2(ck1.x, ck1.y), T1, wa[1]);
-                    nib_chunk(c11, make_uint2(ck1.z, ck1.w), T1, wb[1]);
+                for (int d = 0; d < 2; d++) {
+                    // pair p = 2 hc + d of steps takes the plane bytes [128 p, +128) and the code bytes [64 p, +64) of the
+                    // row (two lanes); its loads were issued a pair ago, and those of pair p + 1 go out now
+                    // (128-token passes have no registers for a pair ahead: they load the pair they are at, and the
+                    // matrix instructions of the pair before cover the wait)
+                    const int p = 2 * hc + d;
+                    uint4 cur[12];
+                    if constexpr (NT != 4) {
 #pragma unroll
-                    for (int jb = 0; jb < 4; jb++) {
-                        const u32x4_t a0 = {wa[0][2 * jb], wa[0][2 * jb + 1], wb[0][2 * jb], wb[0][2 * jb + 1]};
-                        const u32x4_t a1 = {wa[1][2 * jb], wa[1][2 * jb + 1], wb[1][2 * jb], wb[1][2 * jb + 1]};
+                        for (int k = 0; k < 12; k++) {
+                            cur[k] = pa[k];
+                        }
+                    }
+                    const int pn = NT == 4 ? p : p + 1 < 2 * halves ? p + 1 : p; // past the end: this pair's again, unused
 #pragma unroll
-                        for (int t = 0; t < NT; t++) {
-                            if (t == 0 || t < nt) {
-                                const bf16x8_t bv = *(const bf16x8_t *) (bcur + (32 * t + r) * NB_TOK_BYTES + 128 * jb + 32 * s4 + 16 * h);
-                                acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), bv, acc[0][t], 0, 0, 0);
-                                acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), bv, acc[1][t], 0, 0, 0);
+                    for (int k = 0; k < 4; k++) {
+                        pa[k] = *(const uint4 *) (pl0 + 128 * pn + 16 * k);
+                        pa[6 + k] = *(const uint4 *) (pl1 + 128 * pn + 16 * k);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 2; k++) {
+                        pa[4 + k] = *(const uint4 *) (cd0 + 64 * pn + 16 * k);
+                        pa[10 + k] = *(const uint4 *) (cd1 + 64 * pn + 16 * k);
+                    }
+                    if constexpr (NT == 4) {
+#pragma unroll
+                        for (int k = 0; k < 12; k++) {
+                            cur[k] = pa[k];
+                        }
+                    }
+#pragma unroll
+                    for (int st = 0; st < 2; st++) { // the pair's steps: slots 2 st, 2 st + 1 of the lane's four
+                        uint32_t wa[2][8], wb[2][8]; // [matrix]: the step's first and second slot
+#pragma unroll
+                        for (int m = 0; m < 2; m++) {
+                            const uint4 ck = cur[6 * m + 4 + st];
+                            nib_chunk(cur[6 * m + 2 * st], make_uint2(ck.x, ck.y), m ? T1 : T0, wa[m]);
+                            nib_chunk(cur[6 * m + 2 * st + 1], make_uint2(ck.z, ck.w), m ? T1 : T0, wb[m]);
+                        }
+#pragma unroll
+                        for (int jb = 0; jb < 4; jb++) {
+                            const u32x4_t a0 = {wa[0][2 * jb], wa[0][2 * jb + 1], wb[0][2 * jb], wb[0][2 * jb + 1]};
+                            const u32x4_t a1 = {wa[1][2 * jb], wa[1][2 * jb + 1], wb[1][2 * jb], wb[1][2 * jb + 1]};
+#pragma unroll
+                            for (int t = 0; t < NT; t++) {
+                                if (t == 0 || t < nt) {
+                                    const bf16x8_t bv = *(const bf16x8_t *) (bcur + (32 * t + r) * NB_TOK_BYTES + 128 * jb + 64 * d + 32 * h + 16 * st);
+                                    acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), bv, acc[0][t], 0, 0, 0);
+                                    acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), bv, acc[1][t], 0, 0, 0);
+                                }
                             }
                         }
                     }
