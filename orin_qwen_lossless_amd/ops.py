@@ -27,7 +27,7 @@ FLAG_CHUNK_MAJOR, FLAG_FRAG_ORDER, FLAG_WAVE64 = 1, 2, 4
 GEMV_MAX_TOKENS = 8
 # moe_experts: expert GEMVs up to this many routed (token, slot) pairs per expert (tile layout, other layouts), and in
 # the tile layout up to this many pairs whatever the number of experts
-MOE_GEMV_PAIRS_PER_EXPERT = (0.14, 0.7)
+MOE_GEMV_PAIRS_PER_EXPERT = (0.14, 0.7, 0.5)  # tiles, other wave64 / reference layouts, the 4-bit code
 MOE_GEMV_MIN_PAIRS = 24
 DEQUANT_CHUNK_BYTES = 64 << 20
 
@@ -676,6 +676,10 @@ def moe_experts_batched(n_tokens: int, n_used: int, gate: Weight, up: Weight, do
     tiles = all(m.meta.wave64 and m.meta.R == 32 for m in (gate, up, down))
     if tiles:
         gemv = n_tokens * n_used <= max(MOE_GEMV_MIN_PAIRS, MOE_GEMV_PAIRS_PER_EXPERT[0] * n_experts)
+    elif all(m.meta.format == FMT_NIBBLE for m in (gate, up, down)):
+        # the 4-bit code: its GEMV columns have no decode chain and stay ahead for longer (40 layers of 257 experts,
+        # top-8 + 1: 182 / 202 / 221 us per layer at 12 / 14 / 16 tokens against 195 / 199 / 203 batched)
+        gemv = n_tokens <= max(GEMV_MAX_TOKENS, int(MOE_GEMV_PAIRS_PER_EXPERT[2] * n_experts) // n_used)
     else:
         gemv = n_tokens <= max(GEMV_MAX_TOKENS, int(MOE_GEMV_PAIRS_PER_EXPERT[1] * n_experts) // n_used)
     return not gemv and mm_ids_supported(gate, up) and mm_ids_supported(down)

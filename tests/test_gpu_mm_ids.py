@@ -144,8 +144,10 @@ def test_mm_ids_contract(ops):
     cm = enc(ops, wb, HP, 8, True)
     with pytest.raises(ValueError, match="BF16 activations"):
         ops.moe_mm_ids(x.float(), ids, cm, 4)
-    nib = enc(ops, wb, 1)
-    assert not ops.mm_ids_supported(nib)
+    nib = enc(ops, wb, 1)                    # the 4-bit code has a batched kernel of its own (rows per expert: groups of 32)
+    assert ops.mm_ids_supported(nib)
+    with pytest.raises(ValueError, match="multiples of 32"):
+        ops.moe_mm_ids(x, ids, nib, 32)
 
 
 @pytest.mark.parametrize("cm,w64", [(True, False), (False, True)])
