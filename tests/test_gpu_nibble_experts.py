@@ -101,3 +101,15 @@ def test_moe_experts_on_the_4_bit_code_in_both_token_regimes(ops, T):
     got = ops.moe_experts(x, gate, up, down, wts, ids, E).float()
     ref = moe_layer_exact(ops, x, gate, up, down, wts, ids, E).float()
     assert torch.all((got - ref).abs() <= 2e-2 * ref.abs() + 2e-2 * ref.abs().max())
+
+
+def test_batched_kernel_limits_of_the_4_bit_code(ops):
+    """More than 1,024 experts, or rows per expert that are no multiple of 32: a clear error, no launch."""
+    w = nib(ops, synth.weights_torch(2048 * 32, 512, 71, "cuda"))
+    x = torch.zeros((4, 512), dtype=torch.bfloat16, device="cuda")
+    ids = torch.zeros((4, 1), dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="at most 1024 experts"):
+        ops.moe_mm_ids(x, ids, w, 2048)
+    with pytest.raises(ValueError, match="multiples of 32"):
+        ops.moe_mm_ids(x, ids, w, 4096)
+    assert ops.moe_mm_ids(x, ids, w, 1024).shape == (4, 1, 64)
