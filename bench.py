@@ -271,6 +271,7 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4, 16), n_
                                                    "compressed_bytes_touched_expected": int(expected),
                                                    "frac_of_hbm_peak": round(expected / t / 1e3 / HBM_PEAK_GBS, 4)}
         del graph
+    res["layer_sets_4bit"] = sets4[:1]
     del sets4
     res["layer_sets"] = sets
     res["nbytes"] = nbytes
@@ -304,7 +305,7 @@ def configs(ops, w_head, head_copies, comp_bytes: int, K: int) -> dict:
         out[f"gemv_{r}x{k}"] = {"layout": desc, "us": round(t, 2), "GBps": round(nb / t / 1e3, 1), "timing": "16 launches per HIP graph replay"}
     # decode step (builds the layer sets that the MoE layer and the prefill configurations reuse)
     step = decode_step_config(ops, gen, head_copies[0], w_head, K)
-    sets, nbytes = step.pop("layer_sets"), step.pop("nbytes")
+    sets, nbytes, sets4 = step.pop("layer_sets"), step.pop("nbytes"), step.pop("layer_sets_4bit")
     out["decode_step"] = step
     # MoE decode layer, batch 1: router GEMV, top-8 on the device, 8 routed + the shared expert, weighted sum + norm
     st = D.Bf16nStep(ops, sets, None, 1, 1)
@@ -360,6 +361,10 @@ def configs(ops, w_head, head_copies, comp_bytes: int, K: int) -> dict:
         out[f"moe_prefill_T{T}"] = {"us": round(t, 1), "TFLOPs": round(flops / t / 1e6, 1),
                                     "frac_of_bf16_mfma_peak": round(flops / t / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
                                     "weight_decode_GBps": round(wbytes / t / 1e3, 1), "tokens_per_s": round(T / t * 1e6, 0)}
+        w, keep = sets4[0], w  # the same with the expert stacks in the 4-bit code
+        t4 = med_us(prefill, 10, 2)
+        w = keep
+        out[f"moe_prefill_T{T}"]["experts_4bit_code"] = {"us": round(t4, 1), "frac_of_bf16_mfma_peak": round(flops / t4 / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
     return out
 
 
