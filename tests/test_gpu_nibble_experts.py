@@ -117,17 +117,17 @@ def test_batched_kernel_limits_of_the_4_bit_code(ops):
 
 def test_which_token_counts_take_the_batched_kernels(ops):
     """moe_experts_batched for 256 experts with nine slots per token: the tiles leave the expert GEMVs above 0.14 routed
-    pairs per expert (35.8: 3 tokens), the 4-bit code above 0.5 pairs per expert (14 tokens: its GEMV has no decode chain), other layouts
+    pairs per expert (35.8: 3 tokens), the 4-bit code above 0.5 (14 tokens: its GEMV has no decode chain), other layouts
     with a batched kernel above 0.7 (19 tokens)."""
-    E, rows, K = 256, 32, 512
-    wb = synth.weights(E * rows, K, 91)
+    E, rows = 256, 32
 
-    def enc(fmt, R, w64):
-        plane, aux, _, _ = ops.encode_bits(wb, fmt, R, False, wave64=w64)
+    def enc(K, fmt, R, w64):
+        plane, aux, _, _ = ops.encode_bits(synth.weights(E * rows, K, 91 + K), fmt, R, False, wave64=w64)
         ta = torch.from_numpy(aux)
         return ops.upload(torch.from_numpy(plane), ta, ops.parse_header(ta), "cuda")
 
-    for w, last_gemv in ((enc(3, 32, True), 3), (enc(1, 0, False), 14), (enc(3, 4, True), 19)):
-        assert ops.mm_ids_supported(w, w)
-        got = [T for T in range(1, 40) if not ops.moe_experts_batched(T, 9, w, w, w, E)]
-        assert got == list(range(1, last_gemv + 1)), (w.meta.format, w.meta.R, got)
+    for fmt, R, w64, last_gemv in ((3, 32, True, 3), (1, 0, False, 14), (3, 4, True, 19)):
+        gate_up, down = enc(2048, fmt, R, w64), enc(512, fmt, R, w64)
+        assert ops.mm_ids_supported(gate_up, gate_up) and ops.mm_ids_supported(down)
+        got = [T for T in range(1, 40) if not ops.moe_experts_batched(T, 9, gate_up, gate_up, down, E)]
+        assert got == list(range(1, last_gemv + 1)), (fmt, R, got)
