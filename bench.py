@@ -377,7 +377,8 @@ def suite(ops, w_head, head_copies, K: int) -> dict:
     for T in (1, 2, 4, 8, 16, 32, 128):
         xT = synth.activations_torch(T, K, 700 + T, "cuda")
         base = graph_us(lambda i: ops.mmv(xT, head_copies[i & 1]), 4, 10) if T <= 8 else med_us(lambda i: ops.linear(xT, head_copies[i & 1]), 10, 2)
-        batches[str(T)] = {"units_of_16_rows_us": round(base, 1), "path": "gemv" if T <= 8 else "dequant + BF16 GEMM",
+        batches[str(T)] = {"units_of_16_rows_us": round(base, 1),
+                           "path": "gemv" if T <= 8 else "gemv, two launches" if T <= ops.gemv_max_tokens(head_copies[0]) else "dequant + BF16 GEMM",
                            "tiles_us": round(graph_us(lambda i: ops.mmv(xT, tiles[i & 1]), 4, 10), 1)}
     return {"lm_head_batches": {"tiles": tdesc, "tiles_bytes": tbytes, "by_batch": batches}}
 
