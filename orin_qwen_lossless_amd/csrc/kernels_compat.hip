@@ -502,12 +502,17 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
     const bf16n_weight & wu = up ? *up : w;
     const int64_t work = w.format == FMT_NIBBLE ? p.nrows : p.nrows / w.R;
     const dim3 grid(grid_for(work, ncols, cus), ncols);
-    // the matrix cores from nine BF16 columns on, and from five where the row groups give at least half of the CUs a
-    // block (5120 x 2048: 11.0-13.0 us for 5-32 columns against 9.6 / 17.9 us for 4 / 8 GEMV columns and 20 us for
-    // dequant + GEMM; 2048 x 4096, 64 blocks: 18.3-22.8 us against 8.6 / 15.4 us and 24-28 us)
+    // the matrix cores where the row groups of 32 give enough CUs a block: from five BF16 columns on with blocks for half
+    // of the CUs, from nine with a quarter, from 25 with an eighth (5120 x 2048, 160 blocks: 11.0-13.0 us for 5-32
+    // columns against 9.6 / 17.9 us for 4 / 8 GEMV columns and 20 us for dequant + GEMM; 2048 x 4096, 64 blocks: 16.7-20.7
+    // us against 8.6 / 15.4 us and 24-28 us; 1024 x 2048, 32 blocks: 10.6-12.8 us against 7.8 / 9.5 / 14.9 / 25.5 us in
+    // GEMV columns at 9 / 16 / 32 / 64).  Smaller matrices stay with the GEMV columns, which run side by side on idle CUs
+    // (256 x 2048: 4.9-9.5 us for 9-64 columns against 10.5-12.6 us here).
     const int64_t nm_blocks = (p.nrows + 31) / 32;
+    const bool nm_pays = (ncols >= NIB_MM_MIN_COLS && nm_blocks * 2 >= cus) || (ncols > 8 && nm_blocks * 4 >= cus) ||
+                         (ncols > 24 && nm_blocks * 8 >= cus);
     if (matrix_cores && w.format == FMT_NIBBLE && !p.ids && glu == 0 && x_bf16 && w.K % CHUNK == 0 && w.K / 256 <= 2 * NM_WAVES &&
-        (ncols > 8 || (ncols >= NIB_MM_MIN_COLS && nm_blocks * 2 >= cus)) && ((uintptr_t) p.x & 15) == 0 && p.x_tok % 16 == 0) {
+        nm_pays && ((uintptr_t) p.x & 15) == 0 && p.x_tok % 16 == 0) {
         const int halves = (int) (w.K / 256), turns = halves > NM_WAVES ? 2 : 1, waves = (halves + turns - 1) / turns;
         const dim3 grid((unsigned) nm_blocks, (unsigned) ((ncols + 31) / 32));
         const size_t shm = (size_t) waves * 16 * 64 * sizeof(float);

@@ -471,7 +471,8 @@ def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, mode, wan
 def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, oracle, rows, k):
     """Dense batches on a 4-bit matrix, escapes included.  Few BF16 columns (and FP32 columns) share decodes on the VALU
     and have the bits of their single-column products.  From nine BF16 columns on — from five where the matrix has row
-    groups for half of the CUs — the product runs on the matrix cores, 32 tokens per decode: there a column has the same
+    groups for half of the CUs, from 25 where for an eighth only, never with fewer — the product runs on the matrix
+    cores, 32 tokens per decode: there a column has the same
     bits at every batch size and at every position (a token's sum never meets another token's), within the FP64 bound
     of the GEMV.  Rows that are no multiple of 32 and batches that are no multiple of 32 tokens leave a ragged last
     block."""
@@ -486,11 +487,12 @@ def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, oracle, rows,
     xb = synth.activations(70, k, 78)
     x = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16).cuda()
     single = torch.cat([ops.mmv(x[t: t + 1], enc) for t in range(9)])
-    first = 5 if (rows + 31) // 32 * 2 >= torch.cuda.get_device_properties(0).multi_processor_count else 9
+    blocks, cus = (rows + 31) // 32, torch.cuda.get_device_properties(0).multi_processor_count
+    first = 5 if blocks * 2 >= cus else 9 if blocks * 4 >= cus else 25 if blocks * 8 >= cus else 10 ** 9
     y70 = ops.mmv(x, enc)
     for T in (2, 3, 4, 5, 8, 9, 31, 32, 33, 64):
         assert torch.equal(ops.mmv(x[:T], enc), single[:T] if T < first else y70[:T]), T
-    assert torch.equal(ops.mmv(x[37:50], enc), y70[37:50])  # other positions in the block of 32
+    assert torch.equal(ops.mmv(x[37:65], enc), y70[37:65])  # other positions in the block of 32
     assert not torch.equal(y70[:9], single)                 # (the two paths do differ: another order of summation)
     y70n = y70.cpu().numpy()
     for t in (0, 2, 31, 32, 69):
@@ -499,8 +501,8 @@ def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, oracle, rows,
         if t < 9:
             assert np.all(np.abs(single[t].cpu().numpy() - y64) <= 1e-5 * bound), t
     # BF16 out: the one rounding of the FP32 sums
-    y16 = ops.mmv(x[:12], enc, out_dtype=torch.bfloat16)
-    assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y70n[:12]))
+    y16 = ops.mmv(x[:30], enc, out_dtype=torch.bfloat16)
+    assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y70n[:30]))
     xf = x[:4].float()
     single_f = torch.cat([ops.mmv(xf[t: t + 1], enc) for t in range(4)])
     assert torch.equal(ops.mmv(xf, enc), single_f)
