@@ -421,3 +421,35 @@ def test_linear_dense_through_the_c_abi(ops, layout, T):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(yg, want), rep
+
+
+@pytest.mark.parametrize("K,rows,T,row0,nrows", [(1536, 4300, 9, 7, 4200), (2560, 8200, 33, 31, 8169), (3584, 4500, 70, 0, 4500),
+                                                 (4096, 4128, 12, 32, 4096)])
+def test_nibble_matrix_core_batches_on_row_ranges(ops, K, rows, T, row0, nrows):
+    """bf16n_mmv on a row range of a 4-bit matrix (row0, nrows of the C structure) with enough rows for the matrix-core
+    path: K that is no power of two (an odd number of half chunks: the last wavefront's second turn is empty), a range
+    that starts inside a group of 32 rows and ends ragged, escapes; against FP64 on the exact weights, and the GEMV
+    columns (multi_col = 0) beside it."""
+    import ctypes as C
+
+    from orin_qwen_lossless_amd import _lib
+
+    wb = synth.weights(rows, K, 3 * K + rows)
+    wb[::11, ::97] = 0x4500
+    w = enc(ops, wb, NIB, 0, False, False)
+    x = tbf16(synth.activations(T, K, K + T))
+
+    def product(multi_col):
+        y = torch.empty((T, nrows), dtype=torch.float32, device="cuda")
+        a = _lib.MmvArgs()
+        a.x, a.y, a.x_bf16, a.y_bf16, a.n_used, a.x_per_slot = x.data_ptr(), y.data_ptr(), 1, 0, 1, 1
+        a.ncols, a.x_tok, a.y_tok = T, x.stride(0) * 2, nrows * 4
+        a.rows_per_matrix, a.row0, a.nrows = rows, row0, nrows
+        cw = ops._cweight(w)
+        _lib.check(_lib.lib().bf16n_mmv(C.byref(cw), C.byref(a), None, multi_col))
+        return y.double()
+
+    wd = ops.dequant(w).double()[row0: row0 + nrows]
+    ref, bound = x.double() @ wd.T, x.double().abs() @ wd.abs().T
+    for multi_col in (1, 0):
+        assert torch.all((product(multi_col) - ref).abs() <= 1e-5 * bound), multi_col
