@@ -55,6 +55,11 @@ def test_batched_products_of_experts_in_the_4_bit_code(ops, E, N, K, T, topk, po
     assert torch.equal(a16, a.to(torch.bfloat16))  # BF16 out: the one rounding of the FP32 result
     ys = ops.moe_mm_ids(a16, ids, down, E, routes=(dst, dst, bounds)) if down is not None else None
     g_only = ops.moe_mm_ids(x, ids, gate, E, out_dtype=torch.float32, routes=(src1, dst, bounds))
+    # the fused product is the SwiGLU of the two plain products of the same kernel (the same accumulators), whatever the
+    # size of the sums: only the exponential differs (the kernel's fast one)
+    u_only = ops.moe_mm_ids(x, ids, up, E, out_dtype=torch.float32, routes=(src1, dst, bounds))
+    fused_from_plain = u_only * (g_only / (1 + torch.exp(-g_only)))
+    assert torch.all((a - fused_from_plain).abs() <= 2e-5 * fused_from_plain.abs() + 1e-30)
     xd = x.double()
     for e in range(E):
         tok, slot = torch.nonzero(ids == e, as_tuple=True)
