@@ -145,16 +145,31 @@ def encode_to_device(ops, w_dev, n_matrices: int = 1, copies: int = 1, engine: s
     return ws, plane.size + aux.size, desc
 
 
-def read_probe_gbs(ops, nbytes: int) -> dict:
-    """The library's read-only kernel (bf16n_read_probe) over as many bytes as the compressed matrix, two buffers in
-    turn: GB/s per access pattern (median of 30 launches each)."""
+def read_probe_gbs(nbytes: int) -> dict:
+    """A kernel that only reads (libbf16n_probe.so, built from csrc/bench_probe.hip next to the product library: the
+    yardstick of the reference's bench/micro/bwprobe.cu) over as many bytes as the compressed matrix, two buffers in
+    turn: GB/s per access pattern (median of 30 launches each).  pattern 0 / 1: a contiguous range per wavefront,
+    non-temporal / plain loads; 2 / 3: grid-stride."""
+    import ctypes as C
+
     import torch
 
+    path = os.path.join(ROOT, "orin_qwen_lossless_amd", "libbf16n_probe.so")
+    if not os.path.exists(path):
+        raise OSError(f"{path} is missing: build it with `python -m orin_qwen_lossless_amd.build`")
+    probe = C.CDLL(path).bf16n_probe_read
+    probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     bufs = [torch.randint(0, 255, (nbytes // 1024 * 1024,), dtype=torch.uint8, device="cuda") for _ in range(2)]
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def read(buf, pattern, wpc):
+        if probe(buf.data_ptr(), buf.numel(), pattern, wpc, sink.data_ptr(), torch.cuda.current_stream().cuda_stream) != 0:
+            raise RuntimeError("bf16n_probe_read failed")
+
     out = {}
     for pattern, name in ((0, "wavefront_ranges_nontemporal"), (1, "wavefront_ranges_plain"), (2, "grid_stride_nontemporal"), (3, "grid_stride_plain")):
         for wpc in (8, 16):
-            t = med_us(lambda i: ops.read_probe(bufs[i & 1], pattern, wpc), 30, 5)
+            t = med_us(lambda i: read(bufs[i & 1], pattern, wpc), 30, 5)
             out[f"{name}_{wpc}_waves_per_cu"] = round(bufs[0].numel() / t / 1e3, 1)
     return out
 
@@ -513,7 +528,7 @@ def main() -> None:
     xt = x[0].contiguous()
     blas_us = med_us(lambda i: torch.mv(w2[i & 1], xt), min(args.steps, 100), 10)
     del w2
-    probe = read_probe_gbs(ops, comp_bytes)
+    probe = read_probe_gbs(comp_bytes)
     stream_gbs = max(probe.values())
     traffic = measured_traffic(rows, K)
 

@@ -107,8 +107,10 @@ int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x
  * elements); per_slot: x holds one activation row per (token, slot) (the down product) instead of one per token.  At
  * most 65536 routed pairs (n_tok * n_used) and 1024 experts per call, EINVAL beyond.  dst gets the bits that
  * bf16n_mm_ids writes for the same arguments.  All calls on one GPU share the array: calls that can overlap on one GPU
- * (different streams, different threads) race; calls on one stream are ordered.  Call bf16n_init() on every GPU before
- * the first capture. */
+ * (different streams, different threads) race; calls on one stream are ordered.  The ids of a token must name distinct
+ * experts: a repeated naming is counted in the bounds but listed once (as in bf16n_mm_ids_route, mmid_helper.cu:66-71),
+ * and the list entry it leaves unwritten is whatever an earlier call left in the array.  Call bf16n_init() on every GPU
+ * before the first capture. */
 int bf16n_moe_mm_ids_static(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const void * ids,
                             int ids_i64, int64_t ids_row_stride, int per_slot, void * dst, int dst_bf16, int64_t dst_col,
                             int n_experts, int n_tok, int n_used, void * stream);
@@ -142,13 +144,6 @@ int bf16n_router_topk_route_fits(int n_tok, int n_slots, int n_listed);
 int bf16n_router_topk_route(const float * logits, int64_t logits_stride, int n_tok, int n_experts, int k, int renorm,
                             int32_t * ids, float * weights, int64_t out_stride, int n_slots, int n_listed,
                             int32_t * ids_src1, int32_t * ids_dst, int32_t * bounds, int nchannels_y, int sis1, void * stream);
-
-/* Read-bandwidth probe (the reference's bench/micro/bwprobe.cu:23-60 as a library call): a kernel that only reads
- * `bytes` (rounded down to whole KiB) from src, for the memory rate this GPU gives a pure streaming read.  pattern 0:
- * every wavefront walks its own contiguous range in 1 KiB pieces with non-temporal 16-byte loads, four in flight (the
- * fused GEMV's access pattern); 1: the same with plain loads; 2 / 3: grid-stride, non-temporal / plain.  waves_per_cu:
- * wavefronts per CU, 0 = 16 (the fused GEMV's occupancy).  sink: one device word (never written for ordinary data). */
-int bf16n_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, void * stream);
 
 /* ---- load-time conversion and the registry of resident tensors: the reference's llama.cpp adapter without ggml types
  * (engines/llamacpp/patches/0002-ggml-cuda-thin-BF16N-adapter-over-the-shared-core.patch).  An engine stores a converted

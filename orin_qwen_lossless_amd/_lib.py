@@ -59,7 +59,6 @@ SYMBOLS = {
     "bf16n_router_topk_strided": (_i, [_vp, _i64, _i, _i, _i, _i, _vp, _vp, _i64, _vp]),
     "bf16n_router_topk_route_fits": (_i, [_i, _i, _i]),
     "bf16n_router_topk_route": (_i, [_vp, _i64, _i, _i, _i, _i, _vp, _vp, _i64, _i, _i, _vp, _vp, _vp, _i, _i, _vp]),
-    "bf16n_read_probe": (_i, [_vp, C.c_uint64, _i, _i, _vp, _vp]),
     "bf16n_adapter_choose": (_i, [_i64, _i64, _i64, _cp, _i64, _i, _i]),
     "bf16n_adapter_convert": (_i, [_vp, _vp, _i64, _i64, _i64, _i, _i, _i, _vp, _cp, _i, C.POINTER(_i)]),
     "bf16n_verify_roundtrip": (_i, [_WP, _vp, C.POINTER(_i)]),

@@ -15,9 +15,10 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libbf16n_hip.so")
 BENCH = os.path.join(HERE, "bf16n_bench")  # stand-alone timing program (csrc/bench_mmv.cpp), linked against the library
+PROBE = os.path.join(HERE, "libbf16n_probe.so")  # read-bandwidth probe (csrc/bench_probe.hip): measurement only, loaded by the benchmarks
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "adapter.cpp", "dense.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip", "kernels_probe.hip"]
+SOURCES = ["encode.cpp", "policy.cpp", "capi.cpp", "adapter.cpp", "dense.cpp", "kernels_compat.hip", "kernels_w64.hip", "kernels_moe.hip", "kernels_mm_ids.hip", "kernels_tile.hip"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall", "-Wno-unused-function"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -47,10 +48,16 @@ def build(force: bool = False) -> str:
         if r.returncode != 0:
             sys.stderr.write(r.stdout + r.stderr)
             raise RuntimeError("link failed")
+    probe_src = os.path.join(CSRC, "bench_probe.hip")
+    if force or not os.path.exists(PROBE) or os.path.getmtime(PROBE) < os.path.getmtime(probe_src):
+        r = subprocess.run([HIPCC] + COMMON + HIP_FLAGS + ["-shared", probe_src, "-o", PROBE], capture_output=True, text=True)
+        if r.returncode != 0:
+            sys.stderr.write(r.stdout + r.stderr)
+            raise RuntimeError("building libbf16n_probe.so failed")
     bench_src = os.path.join(CSRC, "bench_mmv.cpp")
-    if force or not os.path.exists(BENCH) or os.path.getmtime(BENCH) < max(os.path.getmtime(bench_src), os.path.getmtime(LIB)):
+    if force or not os.path.exists(BENCH) or os.path.getmtime(BENCH) < max(os.path.getmtime(bench_src), os.path.getmtime(LIB), os.path.getmtime(PROBE)):
         r = subprocess.run([HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", "-I" + os.path.join(ROOT, "include"), bench_src,
-                            "-o", BENCH, "-L" + HERE, "-lbf16n_hip", "-Wl,-rpath,$ORIGIN", "-lpthread"], capture_output=True, text=True)
+                            "-o", BENCH, "-L" + HERE, "-lbf16n_hip", "-lbf16n_probe", "-Wl,-rpath,$ORIGIN", "-lpthread"], capture_output=True, text=True)
         if r.returncode != 0:
             sys.stderr.write(r.stdout + r.stderr)
             raise RuntimeError("building bf16n_bench failed")

@@ -2,8 +2,12 @@
 // the decode kernels (every wavefront walks its own contiguous range in 1 KiB pieces, one 16-byte load per lane, a fixed
 // number of loads in flight) or with the textbook grid-stride pattern.  The yardstick next to the fused GEMV's rate; the
 // counterpart of the reference's bench/micro/bwprobe.cu:23-60 (stride and per-warp chunk kernels, load-hint modes).
+//
+// Measurement only: built into libbf16n_probe.so, which the benchmark programs load next to the product library (the
+// product library exports no probe).  One C entry point, bf16n_probe_read.
 #include "dev_w64.h"
-#include "launchers.h"
+
+#include <hip/hip_runtime.h>
 
 namespace bf16n {
 namespace dev {
@@ -73,7 +77,7 @@ __global__ void __launch_bounds__(256) k_probe_stride(const uint4 * __restrict__
 
 // pattern 0: per-wavefront ranges, non-temporal loads; 1: the same with plain loads; 2 / 3: grid-stride, non-temporal
 // / plain.  bytes is rounded down to whole KiB.  waves_per_cu wavefronts per CU (0: 16, the fused GEMV's occupancy).
-void launch_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, int cus, hipStream_t stream) {
+static void launch_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, int cus, hipStream_t stream) {
     const uint64_t pieces = bytes / 1024;
     if (pattern <= 1) {
         const uint64_t waves = (uint64_t) cus * (waves_per_cu > 0 ? waves_per_cu : 16);
@@ -96,3 +100,26 @@ void launch_read_probe(const void * src, uint64_t bytes, int pattern, int waves_
 
 } // namespace dev
 } // namespace bf16n
+
+// Returns 0, or 1 for arguments out of range, or 2 for a HIP error.  src 16-byte aligned; bytes >= 1024; pattern 0..3;
+// waves_per_cu 0..32; sink: one device word (never written for ordinary data); stream: hipStream_t.
+extern "C" int bf16n_probe_read(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, void * stream) {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+            return 2;
+        }
+        cus = prop.multiProcessorCount;
+    }
+    if (!src || !sink || ((uintptr_t) src & 15) != 0 || pattern < 0 || pattern > 3 || bytes < 1024 || waves_per_cu < 0 || waves_per_cu > 32) {
+        return 1;
+    }
+    // a wavefront's range is addressed with 32-bit offsets
+    if (bytes / 1024 / ((uint64_t) cus * (waves_per_cu > 0 ? waves_per_cu : 16)) >= (1u << 21)) {
+        return 1;
+    }
+    bf16n::dev::launch_read_probe(src, bytes, pattern, waves_per_cu, sink, cus, (hipStream_t) stream);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
+}

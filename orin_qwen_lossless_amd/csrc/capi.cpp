@@ -283,8 +283,11 @@ int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
         } else if (w->format == FMT_NIBBLE) {
             // the 4-bit code has no decode chain: batches go through the matrix cores, 32 tokens per decode of the
             // matrix (5120 x 2048: 11-13 us up to 32 tokens, 20 us up to 64, where dequant + GEMM takes 20-21 us;
-            // 2048 x 4096: 17-21 us against 22-28 us)
-            *out = 64;
+            // 2048 x 4096: 17-21 us against 22-28 us), where the dispatch takes that kernel for every count from 9 to
+            // 64; matrices of up to 256 rows run their GEMV columns side by side on idle CUs (4.9-9.5 us for 9-64
+            // columns); between the two the GEMV columns lose to dequant + GEMM beyond the reference's 8
+            const bool all_counts = dev::nib_mm_pays(*w, w->rows, 9, g_cus) && dev::nib_mm_pays(*w, w->rows, 64, g_cus);
+            *out = all_counts || w->rows <= 256 ? 64 : 8;
         } else {
             *out = 8;
         }
@@ -512,20 +515,6 @@ int bf16n_swiglu(const float * g, const float * u, float * y, int64_t n, void * 
         }
         dev::launch_swiglu(g, u, y, n, g_cus, (hipStream_t) stream);
         launch_check("swiglu");
-    });
-}
-
-// bench/micro/bwprobe.cu:23-60 of the reference, as a call: a kernel that only reads
-int bf16n_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, void * stream) {
-    return guarded([&] {
-        ensure_init();
-        require(src && sink && ((uintptr_t) src & 15) == 0, "read_probe: src must be 16-byte aligned, sink non-null");
-        require(pattern >= 0 && pattern <= 3, "read_probe: pattern must be 0..3");
-        require(bytes >= 1024 && waves_per_cu >= 0 && waves_per_cu <= 32, "read_probe: sizes out of range");
-        // a wavefront's range is addressed with 32-bit offsets
-        require(bytes / 1024 / ((uint64_t) g_cus * (waves_per_cu > 0 ? waves_per_cu : 16)) < (1u << 21), "read_probe: buffer too large");
-        dev::launch_read_probe(src, bytes, pattern, waves_per_cu, sink, g_cus, (hipStream_t) stream);
-        launch_check("read_probe");
     });
 }
 

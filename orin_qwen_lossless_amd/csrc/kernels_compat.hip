@@ -497,6 +497,16 @@ int grid_for(int64_t work, int ncols, int cus) {
 
 } // namespace
 
+// Whether a dense batch of `ncols` BF16 columns over `nrows` rows of a 4-bit-code matrix goes through the matrix cores
+// (k_nib_mm): the row groups of 32 must give enough CUs a block, by column count.  The dispatch below and
+// bf16n_gemv_max_tokens share this rule.
+bool nib_mm_pays(const bf16n_weight & w, int64_t nrows, int ncols, int cus) {
+    const int64_t nm_blocks = (nrows + 31) / 32;
+    const bool enough = (ncols >= NIB_MM_MIN_COLS && nm_blocks * 2 >= cus) || (ncols > 8 && nm_blocks * 4 >= cus) ||
+                        (ncols > 24 && nm_blocks * 8 >= cus);
+    return w.format == FMT_NIBBLE && w.K % CHUNK == 0 && w.K / 256 <= 2 * NM_WAVES && enough;
+}
+
 void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,
                        int cus, hipStream_t stream, bool matrix_cores) {
     const bf16n_weight & wu = up ? *up : w;
@@ -509,10 +519,8 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
     // GEMV columns at 9 / 16 / 32 / 64).  Smaller matrices stay with the GEMV columns, which run side by side on idle CUs
     // (256 x 2048: 4.9-9.5 us for 9-64 columns against 10.5-12.6 us here).
     const int64_t nm_blocks = (p.nrows + 31) / 32;
-    const bool nm_pays = (ncols >= NIB_MM_MIN_COLS && nm_blocks * 2 >= cus) || (ncols > 8 && nm_blocks * 4 >= cus) ||
-                         (ncols > 24 && nm_blocks * 8 >= cus);
-    if (matrix_cores && w.format == FMT_NIBBLE && !p.ids && glu == 0 && x_bf16 && w.K % CHUNK == 0 && w.K / 256 <= 2 * NM_WAVES &&
-        nm_pays && ((uintptr_t) p.x & 15) == 0 && p.x_tok % 16 == 0) {
+    if (matrix_cores && !p.ids && glu == 0 && x_bf16 && nib_mm_pays(w, p.nrows, ncols, cus) && ((uintptr_t) p.x & 15) == 0 &&
+        p.x_tok % 16 == 0) {
         const int halves = (int) (w.K / 256), turns = halves > NM_WAVES ? 2 : 1, waves = (halves + turns - 1) / turns;
         const dim3 grid((unsigned) nm_blocks, (unsigned) ((ncols + 31) / 32));
         const size_t shm = (size_t) waves * 16 * 64 * sizeof(float);

@@ -1202,6 +1202,9 @@ bool nib_mm_ids_ok(const bf16n_weight & w, const bf16n_weight * up) {
     return w.format == FMT_NIBBLE && w.K % 512 == 0 && (!up || (up->format == FMT_NIBBLE && up->rows == w.rows && up->K == w.K));
 }
 
+// upper bound of the (expert, pass) units a call lists: one per expert and one per full pass
+int64_t nib_mm_ids_units_bound(int n_experts, int64_t n_pairs, int pass_tokens) { return n_experts + n_pairs / pass_tokens; }
+
 template <int NT>
 void nb_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & a, int cus, hipStream_t stream) {
     const int per_cu = (int) (160 * 1024 / nb_shm<NT>()) < 3 ? (int) (160 * 1024 / nb_shm<NT>()) : 3;
@@ -1225,7 +1228,13 @@ void launch_nib_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const vo
         throw std::invalid_argument("bf16n: batched 4-bit-code experts need rows per expert in multiples of 32 and at most 1024 experts");
     }
     // a pass decodes the expert's rows again: long passes where the experts have many tokens.  The units listed are at
-    // most one per expert and one per full pass: within MT_MAX_UNITS for up to 32 pairs per expert with the shortest.
+    // most one per expert and one per full pass: within MT_MAX_UNITS for up to 32 pairs per expert with the shortest;
+    // with the longest the bound depends on the call, and a list that does not fit would leave experts uncomputed.
+    const int pass = n_pairs <= (int64_t) NB_PAIRS_32 * n_experts ? 32 : n_pairs <= (int64_t) NB_PAIRS_64 * n_experts ? 64 : 128;
+    if (nib_mm_ids_units_bound(n_experts, n_pairs, pass) > MT_MAX_UNITS) {
+        throw std::invalid_argument("bf16n: too many routed pairs for one batched call on 4-bit-code experts (experts + pairs / 128 "
+                                    "must stay within 2048): split the tokens over several calls");
+    }
     if (n_pairs <= (int64_t) NB_PAIRS_32 * n_experts) {
         nb_launch<1>(w, up, a, cus, stream);
     } else if (n_pairs <= (int64_t) NB_PAIRS_64 * n_experts) {

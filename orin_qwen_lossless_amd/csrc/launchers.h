@@ -12,6 +12,7 @@ namespace bf16n {
 namespace dev {
 
 // 32-lane layouts (kernels_compat.hip). glu: 0 plain, 1 merged [gate; up] NIBBLE matrix, 2 separate gate / up matrices
+bool nib_mm_pays(const bf16n_weight & w, int64_t nrows, int ncols, int cus);
 void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,
                        int cus, hipStream_t stream, bool matrix_cores = true);
 void launch_compat_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream);
@@ -74,8 +75,6 @@ void launch_router_topk_route(const float * logits, int64_t stride, int n_tok, i
                               float * weights, int64_t out_stride, int n_slots, int n_listed, int32_t * ids_src1, int32_t * ids_dst,
                               int32_t * bounds, int nchannels_y, int sis1, hipStream_t stream);
 
-// read-bandwidth probe (kernels_probe.hip)
-void launch_read_probe(const void * src, uint64_t bytes, int pattern, int waves_per_cu, uint32_t * sink, int cus, hipStream_t stream);
 
 // batched MoE prefill (kernels_mm_ids.hip)
 void mm_ids_init();

@@ -632,21 +632,6 @@ def router_topk_routes(logits: torch.Tensor, k: int, n_listed: int, renorm: bool
     return wts, ids, (src1, dst, bounds)
 
 
-_probe_sink: dict = {}
-
-
-def read_probe(buf: torch.Tensor, pattern: int = 0, waves_per_cu: int = 0) -> None:
-    """One launch of the library's read-only kernel over a contiguous device buffer (bf16n_read_probe: the yardstick of
-    the reference's bench/micro/bwprobe.cu).  pattern 0 / 1: a contiguous range per wavefront, non-temporal / plain
-    loads; 2 / 3: grid-stride."""
-    if not (buf.is_cuda and buf.is_contiguous() and buf.data_ptr() % 16 == 0):
-        raise ValueError("bf16n.read_probe: a contiguous, 16-byte aligned device buffer is required")
-    sink = _probe_sink.setdefault(buf.device, torch.zeros(1, dtype=torch.int32, device=buf.device))
-    with torch.cuda.device(buf.device):
-        _lib.check(_lib.lib().bf16n_read_probe(buf.data_ptr(), buf.numel() * buf.element_size(), pattern, waves_per_cu,
-                                               sink.data_ptr(), _stream()))
-
-
 def glu2_supported(gate: Weight, up: Weight) -> bool:
     """Layouts with a fused gate / up + SwiGLU GEMV (the rule of bf16n::mmv_glu(gate, up), core launch.h:56-61, plus
     this build's wave64 units): same format, K, R and layout, not chunk-major."""

@@ -136,3 +136,29 @@ def test_which_token_counts_take_the_batched_kernels(ops):
         assert ops.mm_ids_supported(gate_up, gate_up) and ops.mm_ids_supported(down)
         got = [T for T in range(1, 40) if not ops.moe_experts_batched(T, 9, gate_up, gate_up, down, E)]
         assert got == list(range(1, last_gemv + 1)), (fmt, R, got)
+
+
+def test_a_call_whose_unit_list_would_not_fit_is_refused(ops):
+    """The batched kernel lists (expert, pass) units in LDS, 2048 at most: a call with more (experts + routed pairs / 128
+    with the longest passes) is refused on the host instead of leaving the last experts uncomputed; the largest call
+    that fits is computed, the last expert included."""
+    E, N, K, topk = 257, 32, 512, 9
+    w = synth.weights_torch(E * N, K, 77, "cuda")
+    gate = nib(ops, w)
+    T_fit = (2048 - E) * 128 // topk          # experts + pairs / 128 == 2048 at most
+    T_over = T_fit + 128
+    for T in (T_over, T_fit):
+        x = synth.activations_torch(T, K, 78, "cuda")
+        # every token names the last expert (a shared expert stacked behind the routed ones) and eight others in turn
+        base = (torch.arange(T, device="cuda", dtype=torch.int32)[:, None] * 8 + torch.arange(8, device="cuda", dtype=torch.int32)[None, :]) % (E - 1)
+        ids = torch.cat([base, torch.full((T, 1), E - 1, device="cuda", dtype=torch.int32)], 1).contiguous()
+        if T == T_over:
+            with pytest.raises(ValueError, match="too many routed pairs"):
+                ops.moe_mm_ids(x, ids, gate, E)
+            continue
+        y = ops.moe_mm_ids(x, ids, gate, E)
+        last = w[(E - 1) * N:].float()
+        for t in (0, T // 2, T - 1):   # the stacked expert's rows of the first, a middle and the last token
+            want = last.double() @ x[t].double()
+            bound = last.double().abs() @ x[t].double().abs()
+            assert torch.all((y[t, topk - 1].double() - want).abs() <= 1e-5 * bound), t

@@ -37,13 +37,16 @@ def static_call(ops, x, ids, w, n_experts, up=None, out_dtype=torch.float32):
     return y
 
 
-@pytest.mark.parametrize("layout", ["tiles", "units"])
+@pytest.mark.parametrize("layout", ["tiles", "units", "nibble"])
 def test_static_routing_lists_match_the_allocating_path(ops, layout):
     E, k, K, N = 24, 4, 2048, 512
-    r_gu, r_dn = (32, 32) if layout == "tiles" else (4, 16)
-    gate = enc(ops, synth.weights(E * N, K, 201), HP, r_gu, False, True)
-    up = enc(ops, synth.weights(E * N, K, 202), HP, r_gu, False, True)
-    down = enc(ops, synth.weights(E * K, N, 203), HP, r_dn, False, True)
+    if layout == "nibble":  # expert stacks in the 4-bit code: the third dispatch branch of the entry point
+        gate, up, down = (enc(ops, synth.weights(r, c, 201 + i), 1, 1, False) for i, (r, c) in enumerate(((E * N, K), (E * N, K), (E * K, N))))
+    else:
+        r_gu, r_dn = (32, 32) if layout == "tiles" else (4, 16)
+        gate = enc(ops, synth.weights(E * N, K, 201), HP, r_gu, False, True)
+        up = enc(ops, synth.weights(E * N, K, 202), HP, r_gu, False, True)
+        down = enc(ops, synth.weights(E * K, N, 203), HP, r_dn, False, True)
     rng = np.random.default_rng(7)
     for T in (300, 41):  # the second call is smaller: entries of the first call's lists stay behind it in the array
         x = tbf16(synth.activations(T, K, 210 + T))
