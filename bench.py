@@ -223,26 +223,39 @@ def cpu_baseline(wbits, K: int, xf, sample_rows: int, budget_s: float):
 
 # ---------------------------------------------------------------- the other configurations of the path
 
-def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4, 16), n_layers: int = 40, n_sets: int = 4) -> dict:
+def decode_step_config(ops, gen, head, head_tiles, head_bf16, K: int, batches=(1, 4, 16), n_layers: int = 40, n_sets: int = 40,
+                       n_sets_4bit: int = 8) -> dict:
     """The 40-layer decode step as one HIP graph on BF16N weights and on uncompressed BF16 weights with stock kernels
-    (orin_qwen_lossless_amd/decode_step.py), output projection included.  n_sets distinct weight sets are used in turn;
-    every layer's input is the previous layer's output, so layers that share a set route to other experts."""
+    (orin_qwen_lossless_amd/decode_step.py), output projection included.  n_sets distinct weight sets are used in turn
+    (40: every layer has weights of its own, nothing a step reads is read twice; a step's 3.4 GB also pass through the
+    256 MB last-level cache between two replays).  Batches above one token are verify steps: their output projection
+    is the one the policy gives a caller who states so (dense_frag_order: matrix-core tiles)."""
     import numpy as np
     import torch
 
     from orin_qwen_lossless_amd import decode_step as D, synth
 
+    t0 = time.perf_counter()
     sets, raw, nbytes = D.make_layer_sets(ops, gen, n_sets, True)
-    head_bytes = head.plane.numel() + head.aux.numel()
-    res = {"layers": n_layers, "weight_sets": n_sets,
-           "bf16_comparator": "the same graph on uncompressed BF16 weights: torch linear / bmm (hipBLASLt) for every product, the "
-                              "experts a token selects gathered by index_select (the routing is decided on the device), "
-                              "the same glue and top-k launches"}
+    setup_s = time.perf_counter() - t0
+    res = {"layers": n_layers, "weight_sets": n_sets, "weight_sets_setup_s": round(setup_s, 1),
+           "bf16_comparator": "the same graph on uncompressed BF16 weights with stock kernels (torch linear / bmm = hipBLASLt), the same glue "
+                              "and top-k launches.  bf16_us: the experts a token selects are gathered by index_select and multiplied "
+                              "as a batch (what a graph can capture when the routing is decided on the device).  bf16_static_ids_us: "
+                              "the expert matrices are read in place, one GEMV launch per expert and matrix, with expert ids fixed "
+                              "on the host at capture (a captured graph cannot do that with device-side routing: a lower bound for "
+                              "stock kernels).  speedup_vs_bf16 is against the faster of the two"}
     for T in batches:
         xin = [synth.activations_torch(T, K, 300 + i, "cuda") for i in range(4)]
         hbuf = xin[0].clone()
         entry = {}
-        for name, step in (("bf16n", D.Bf16nStep(ops, sets, head, n_layers, T)), ("bf16", D.Bf16Step(ops, raw, head_bf16, n_layers, T))):
+        hd = head if T == 1 else head_tiles
+        head_bytes = hd.plane.numel() + hd.aux.numel()
+        static_ids = [[(7 * t + 31 * j) % D.E for j in range(D.TOPK)] for t in range(T)] if T <= 4 else None
+        steps = [("bf16n", D.Bf16nStep(ops, sets, hd, n_layers, T)), ("bf16", D.Bf16Step(ops, raw, head_bf16, n_layers, T))]
+        if static_ids is not None:
+            steps.append(("bf16_static", D.Bf16Step(ops, raw, head_bf16, n_layers, T, static_ids=static_ids)))
+        for name, step in steps:
             graph, out = D.capture(step, hbuf)
             eager = step(hbuf).clone()
             graph.replay()
@@ -260,28 +273,34 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4, 16), n_
         bf16_bytes = 2 * (n_layers * (sum(r * k for n_, (r, k, m) in D.SHAPES.items() if m == 1)
                                       + (min(T * D.TOPK, D.E) + 1) * 3 * D.N_MID * K) + head_bf16.numel())
         t = entry["bf16n"]
+        best_bf16 = min(v for k_, v in entry.items() if k_ != "bf16n")
         gemv_path = T * (D.TOPK + 1) <= max(ops.MOE_GEMV_MIN_PAIRS, ops.MOE_GEMV_PAIRS_PER_EXPERT[0] * D.EA)
-        res[f"batch{T}"] = {"us": round(t, 1), "launches_per_layer": 8 if gemv_path or T <= ops.TOPK_ROUTE_ONE_LAUNCH_TOKENS else 9, "compressed_bytes_touched_upper_bound": int(touched),
+        res[f"batch{T}"] = {"us": round(t, 1), "launches_per_layer": D.launches_per_layer(ops, T, gemv_path),
+                            "output_projection": "16-row units" if T == 1 else "matrix-core tiles (dense_frag_order)",
+                            "compressed_bytes_touched_upper_bound": int(touched),
                             "compressed_bytes_touched_expected": int(expected), "GBps": round(expected / t / 1e3, 1),
                             "frac_of_hbm_peak": round(expected / t / 1e3 / HBM_PEAK_GBS, 4), "tokens_per_s": round(T / t * 1e6, 1),
-                            "bf16_us": round(entry["bf16"], 1), "speedup_vs_bf16": round(entry["bf16"] / t, 2),
+                            "bf16_us": round(entry["bf16"], 1),
+                            "bf16_static_ids_us": round(entry["bf16_static"], 1) if "bf16_static" in entry else None,
+                            "speedup_vs_bf16": round(best_bf16 / t, 2),
                             "bf16_bytes_touched": int(bf16_bytes), "bf16_us_at_hbm_peak": round(bf16_bytes / HBM_PEAK_GBS / 1e3, 1),
                             "eager_equals_graph": True}
     # the same step with the expert stacks in the 4-bit code (the policy's nibble mode for them): no decode chain
     # in the routed GEMVs, 7 % more expert bytes
-    sets4, _, nbytes4 = D.make_layer_sets(ops, gen, n_sets, False, expert_mode="nibble")
-    res["experts_4bit_code"] = {"expert_bytes_vs_tiles": round(nbytes4["gate"] / nbytes["gate"], 4)}
+    sets4, _, nbytes4 = D.make_layer_sets(ops, gen, n_sets_4bit, False, expert_mode="nibble")
+    res["experts_4bit_code"] = {"expert_bytes_vs_tiles": round(nbytes4["gate"] / nbytes["gate"], 4), "weight_sets": n_sets_4bit}
     for T in (1, 4):
         xin = [synth.activations_torch(T, K, 300 + i, "cuda") for i in range(4)]
         hbuf = xin[0].clone()
-        graph, _ = D.capture(D.Bf16nStep(ops, sets4, head, n_layers, T), hbuf)
+        hd = head if T == 1 else head_tiles
+        graph, _ = D.capture(D.Bf16nStep(ops, sets4, hd, n_layers, T), hbuf)
 
         def replay4(i):
             hbuf.copy_(xin[i & 3])
             graph.replay()
 
         t = float(np.median(time_kernel(replay4, 12, 3))) * 1e3
-        expected = n_layers * D.layer_bytes(nbytes4, T, expected=True) + head_bytes
+        expected = n_layers * D.layer_bytes(nbytes4, T, expected=True) + hd.plane.numel() + hd.aux.numel()
         res["experts_4bit_code"][f"batch{T}"] = {"us": round(t, 1), "vs_policy_layout": round(res[f"batch{T}"]["us"] / t, 3),
                                                    "compressed_bytes_touched_expected": int(expected),
                                                    "frac_of_hbm_peak": round(expected / t / 1e3 / HBM_PEAK_GBS, 4)}
@@ -293,7 +312,7 @@ def decode_step_config(ops, gen, head, head_bf16, K: int, batches=(1, 4, 16), n_
     return res
 
 
-def configs(ops, w_head, head_copies, comp_bytes: int, K: int) -> dict:
+def configs(ops, w_head, head_copies, comp_bytes: int, K: int, n_sets: int = 40) -> dict:
     """The other configurations, compact: batch 4 on the output projection, the two small matrices, the MoE decode
     layer as one HIP graph, the batched prefill at 2048 and 8192 tokens, the 40-layer decode step at batch 1 and 4."""
     import numpy as np
@@ -310,16 +329,34 @@ def configs(ops, w_head, head_copies, comp_bytes: int, K: int) -> dict:
 
     rows = w_head.shape[0]
     x4 = synth.activations_torch(4, K, 21, "cuda")
+    x1 = synth.activations_torch(1, K, 2, "cuda")
     t4 = graph_us(lambda i: ops.mmv(x4, head_copies[i & 1]), 8)
+    k4 = ops.last_kernel()
+    t1 = graph_us(lambda i: ops.mmv(x1, head_copies[i & 1]), 8)
     algo4 = comp_bytes + 4 * K * 2 + 4 * rows * 4
-    out["lm_head_batch4"] = {"timing": "8 launches per HIP graph replay", "us": round(t4, 2), "GBps": round(algo4 / t4 / 1e3, 1), "frac_of_hbm_peak": round(algo4 / t4 / 1e3 / HBM_PEAK_GBS, 4)}
+    # the layout the policy gives the same matrix when the caller states that it verifies several tokens per step
+    # (dense_frag_order: 32 x 256 tiles in matrix-core operand order; one decode of the matrix serves up to 32 tokens)
+    tiles, tile_bytes, tile_desc = encode_to_device(ops, w_head, copies=2, matrix_core_order=True)
+    tt4 = graph_us(lambda i: ops.mmv(x4, tiles[i & 1]), 8)
+    kt4 = ops.last_kernel()
+    tt1 = graph_us(lambda i: ops.mmv(x1, tiles[i & 1]), 8)
+    talgo4 = tile_bytes + 4 * K * 2 + 4 * rows * 4
+    out["lm_head_batch4"] = {"timing": "8 launches per HIP graph replay, two weight copies in turn",
+                             "units_of_16_rows": {"us": round(t4, 2), "batch1_us": round(t1, 2), "vs_batch1": round(t4 / t1, 3), "kernel": k4,
+                                                  "GBps": round(algo4 / t4 / 1e3, 1), "frac_of_hbm_peak": round(algo4 / t4 / 1e3 / HBM_PEAK_GBS, 4)},
+                             "matrix_core_tiles": {"layout": tile_desc, "compressed_bytes": tile_bytes, "us": round(tt4, 2), "batch1_us": round(tt1, 2),
+                                                   "vs_batch1": round(tt4 / tt1, 3), "vs_batch1_of_16_row_units": round(tt4 / t1, 3), "kernel": kt4,
+                                                   "GBps": round(talgo4 / tt4 / 1e3, 1),
+                                                   "frac_of_hbm_peak": round(talgo4 / tt4 / 1e3 / HBM_PEAK_GBS, 4)},
+                             "us": round(min(t4, tt4), 2), "policy": "dense_frag_order (the caller verifies several tokens per step) selects the tiles"}
     for r, k in ((512, 2048), (2048, 512)):
         ws, nb, desc = encode_to_device(ops, gen(r, k), copies=2)
         xx = synth.activations_torch(1, k, 22, "cuda")
         t = graph_us(lambda i: ops.mmv(xx, ws[i & 1]))
         out[f"gemv_{r}x{k}"] = {"layout": desc, "us": round(t, 2), "GBps": round(nb / t / 1e3, 1), "timing": "16 launches per HIP graph replay"}
     # decode step (builds the layer sets that the MoE layer and the prefill configurations reuse)
-    step = decode_step_config(ops, gen, head_copies[0], w_head, K)
+    step = decode_step_config(ops, gen, head_copies[0], tiles[0], w_head, K, n_sets=n_sets)
+    del tiles
     sets, nbytes, sets4 = step.pop("layer_sets"), step.pop("nbytes"), step.pop("layer_sets_4bit")
     out["decode_step"] = step
     # MoE decode layer, batch 1: router GEMV, top-8 on the device, 8 routed + the shared expert, weighted sum + norm
@@ -429,7 +466,7 @@ def prefill_only(T: int, steps: int, mode: str = "hybrid") -> None:
                       "frac_of_bf16_mfma_peak": round((flops_gu + flops_dn) / (t_gu + t_dn) / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}))
 
 
-def decode_only(T: int, steps: int) -> None:
+def decode_only(T: int, steps: int, n_sets: int = 40, expert_mode: str = "hybrid") -> None:
     """Only the 40-layer decode step on BF16N weights at batch T, `steps` graph replays (for profiling); prints its own
     JSON line."""
     import numpy as np
@@ -446,8 +483,8 @@ def decode_only(T: int, steps: int) -> None:
         seed[0] += 1
         return synth.weights_torch(rows, k, seed[0], "cuda")
 
-    sets, _, nbytes = D.make_layer_sets(ops, gen, 4, False)
-    (head,), hb, _ = encode_to_device(ops, gen(248320, K))
+    sets, _, nbytes = D.make_layer_sets(ops, gen, n_sets, False, expert_mode=expert_mode)
+    (head,), hb, _ = encode_to_device(ops, gen(248320, K), matrix_core_order=T > 1)
     xin = [synth.activations_torch(T, K, 300 + i, "cuda") for i in range(4)]
     hbuf = xin[0].clone()
     graph, _ = D.capture(D.Bf16nStep(ops, sets, head, 40, T), hbuf)
@@ -473,10 +510,11 @@ def main() -> None:
     ap.add_argument("--cpu-rows", type=int, default=16384)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU work of the baseline leg, about")
     ap.add_argument("--no-configs", action="store_true", help="only the headline kernel: skip the other configurations")
+    ap.add_argument("--weight-sets", type=int, default=40, help="distinct weight sets of the 40-layer decode step (40: one per layer)")
     ap.add_argument("--suite", action="store_true", help="also sweep the output projection over batch sizes in both layouts")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="run only the batched MoE kernels of one layer on T tokens (for profiling) and exit")
-    ap.add_argument("--experts-4bit", action="store_true", help="with --prefill: the expert stacks in the 4-bit code (policy mode nibble)")
+    ap.add_argument("--experts-4bit", action="store_true", help="with --prefill / --decode-step: the expert stacks in the 4-bit code (policy mode nibble)")
     ap.add_argument("--decode-step", type=int, default=0, metavar="T",
                     help="run only the 40-layer decode step at batch T (for profiling) and exit")
     args = ap.parse_args()
@@ -486,7 +524,7 @@ def main() -> None:
         prefill_only(args.prefill, min(args.steps, 20), "nibble" if args.experts_4bit else "hybrid")
         return
     if args.decode_step > 0:
-        decode_only(args.decode_step, min(args.steps, 20))
+        decode_only(args.decode_step, min(args.steps, 20), args.weight_sets, "nibble" if args.experts_4bit else "hybrid")
         return
 
     import numpy as np
@@ -517,6 +555,8 @@ def main() -> None:
     comp_bytes = plane.size + aux.size
     algo_bytes = comp_bytes + K * 2 + rows * 4  # weights (plane + aux incl. table, unit bases, padding) + x + y
     step = lambda i: ops.mmv(x, copies[i & 1])  # noqa: E731
+    step(0)
+    kernel_name = ops.last_kernel()  # what the library's dispatch launched for this call
     blocks, block_events = time_blocks(step, args.steps, args.warmup, SETTLE_MS, MIN_TIMED_MS)
     ms = float(np.median(blocks)) / args.steps
     # the kernel's average launch duration over the timed region: HIP events on the launch stream around each block
@@ -526,7 +566,9 @@ def main() -> None:
     # stock BF16 GEMV on the uncompressed tensor (the "vs BF16" column), same timing
     w2 = [w_dev, w_dev.clone()]
     xt = x[0].contiguous()
-    blas_us = med_us(lambda i: torch.mv(w2[i & 1], xt), min(args.steps, 100), 10)
+    blas_blocks, _ = time_blocks(lambda i: torch.mv(w2[i & 1], xt), args.steps, args.warmup, SETTLE_MS, MIN_TIMED_MS)
+    blas_us = float(np.median(blas_blocks)) / args.steps * 1e3
+    blas_single_us = med_us(lambda i: torch.mv(w2[i & 1], xt), min(args.steps, 100), 10)
     del w2
     probe = read_probe_gbs(comp_bytes)
     stream_gbs = max(probe.values())
@@ -548,18 +590,21 @@ def main() -> None:
         "roofline": {"bound": "hbm", "achieved": round(algo_bytes / (kern_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": traffic, "traffic_source": TRAFFIC_PROFILE if traffic is not None else None,
-                     "kernel": "k_w64_mmv<bf16_t, 4, 1, 2, 1>", "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 3),
+                     "kernel": kernel_name, "algorithmic_bytes": algo_bytes, "avg_launch_us": round(kern_ms * 1e3, 3),
                      "timing": f"HIP events around each block of {args.steps} back-to-back launches, median block / {args.steps}",
                      "single_launch_event_us": {"mean": round(float(np.mean(durs)) * 1e3, 2), "median": round(float(np.median(durs)) * 1e3, 2)}},
         "extra": {"pct_of_hbm_peak_compressed": round(100 * comp_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
                   "us_per_matrix": round(ms * 1e3, 2), "block_us_per_step_min_max": [round(min(blocks) / args.steps * 1e3, 2), round(max(blocks) / args.steps * 1e3, 2)],
                   "blas_bf16_gemv_us": round(blas_us, 2), "speedup_vs_blas_bf16": round(blas_us / (ms * 1e3), 3),
+                  "blas_timing": "the same blocks of back-to-back launches after the same settle time as the headline kernel (median block); "
+                                 "blas_bf16_gemv_single_launch_event_us: events around single launches, as single_launch_event_us",
+                  "blas_bf16_gemv_single_launch_event_us": round(blas_single_us, 2),
                   "plain_stream_read_GBps": round(stream_gbs, 1), "read_probe_GBps": probe,
                   "kernel_vs_plain_stream_read": round(algo_bytes / (kern_ms * 1e-3) / 1e9 / stream_gbs, 3), "tokens_per_s_lm_head_only": round(1e3 / ms, 1),
                   "host_encode_s": round(t_enc, 2), "max_err_over_sum_abs": err},
     }
     if not args.no_configs:
-        out["extra"]["configs"] = configs(ops, w_dev, copies, comp_bytes, K)
+        out["extra"]["configs"] = configs(ops, w_dev, copies, comp_bytes, K, args.weight_sets)
     if args.suite:
         out["extra"]["suite"] = suite(ops, w_dev, copies, K)
     out["extra"]["gpu_s"] = round(time.perf_counter() - t0, 1)

@@ -27,6 +27,10 @@ enum { BF16N_ENGINE_LLAMA = 0, BF16N_ENGINE_VLLM = 1, BF16N_ENGINE_MI355X = 2 };
 enum { BF16N_MODE_HYBRID = 0, BF16N_MODE_HUFFMAN = 1, BF16N_MODE_NIBBLE = 2 };
 
 const char * bf16n_last_error(void);
+/* No counterpart in the reference.  The kernel instance that the calling thread's last dense product launch chose, in
+ * the profiler's spelling ("k_w64_mmv<bf16_t, 4, 1, 2, 1>"), set by the dispatch code; "" where a path leaves no note.
+ * For measurement programs that name the kernel they time.  Valid until the thread's next call of this function. */
+const char * bf16n_last_kernel(void);
 
 /* ---- host encoder: bf16n::encode, core/include/bf16n/encode.h:12-26, core/src/encode.cpp:443-526 ----------------- */
 typedef struct bf16n_encoded bf16n_encoded; /* owns plane + aux (struct encoded, encode.h:12-17) */

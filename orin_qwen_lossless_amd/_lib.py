@@ -30,6 +30,7 @@ _i, _i64, _u32, _vp, _cp = C.c_int, C.c_int64, C.c_uint32, C.c_void_p, C.c_char_
 _WP, _AP = C.POINTER(Weight), C.POINTER(MmvArgs)
 SYMBOLS = {
     "bf16n_last_error": (_cp, []),
+    "bf16n_last_kernel": (_cp, []),
     "bf16n_encode": (_i, [_vp, _i64, _i64, _i, _i, _u32, C.POINTER(_vp)]),
     "bf16n_encoded_plane": (_vp, [_vp, C.POINTER(C.c_uint64)]),
     "bf16n_encoded_aux": (_vp, [_vp, C.POINTER(C.c_uint64)]),

@@ -24,6 +24,7 @@ struct bf16n_encoded {
 namespace {
 
 thread_local std::string g_error;
+thread_local std::string g_kernel_text;
 
 int g_cus = 0;
 int g_lds_max = 0;
@@ -170,6 +171,12 @@ void launch_check(const char * what) { hip_check(hipGetLastError(), what); }
 
 } // namespace
 
+namespace bf16n {
+namespace dev {
+thread_local kernel_note g_last_kernel = {nullptr, nullptr, 0, {0, 0, 0, 0, 0}};
+} // namespace dev
+} // namespace bf16n
+
 extern "C" {
 
 const char * bf16n_last_error(void) { return g_error.c_str(); }
@@ -268,6 +275,22 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
 // The number of BF16 token columns up to which bf16n_mmv is the faster dense path; beyond it dequant + a stock GEMM is.
 // 8 is the reference's fixed rule (core/torch/torch_bindings.cpp:195); matrices whose products run on the matrix cores
 // stay ahead for far longer (every pass of up to 128 columns decodes the matrix once).
+// The kernel instance that the calling thread's last bf16n_mmv / bf16n_mmv_glu2 launch chose, as the profiler prints it
+// ("k_w64_mmv<bf16_t, 4, 1, 2, 1>"); an empty string before the first launch or after a launch on a path that leaves
+// no note.  The pointer stays valid until the thread's next call of this function.
+const char * bf16n_last_kernel(void) {
+    const dev::kernel_note & k = dev::g_last_kernel;
+    g_kernel_text.clear();
+    if (k.name) {
+        g_kernel_text = std::string(k.name) + "<" + (k.tx ? k.tx : "");
+        for (int i = 0; i < k.n_args; i++) {
+            g_kernel_text += (i || k.tx ? ", " : "") + std::to_string(k.arg[i]);
+        }
+        g_kernel_text += ">";
+    }
+    return g_kernel_text.c_str();
+}
+
 int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
     return guarded([&] {
         ensure_init();

@@ -1142,6 +1142,7 @@ void mt_launch(const bf16n_weight & w, const bf16n_weight * up, const mm_args & 
     using S = mt_shape<NT, W>;
     const int64_t items = mt_items<W>(a, up != nullptr), slots = cus; // the LDS of a CU holds one block
     const dim3 grid((unsigned) (items < slots ? items : slots));
+    note_kernel("k_mm_tile", up ? "true" : "false", 2, NT, W);
     if (up) {
         hipLaunchKernelGGL((k_mm_tile<true, NT, W>), grid, dim3(S::THREADS), (mt_shm<NT, W>(true)), stream, w, *up, a);
     } else {

@@ -445,10 +445,12 @@ template <typename TX, int C, int NC, int HINT>
 void mmv_launch_hint(dim3 grid, int nt, int wpb, hipStream_t stream, const bf16n_weight & w, const cols & p, int upw) {
     if constexpr (two_chains<TX, C, NC>()) {
         if (upw >= 2) {
+            note_kernel("k_w64_mmv", tx_name<TX>(), 4, C, NC, 2, HINT);
             hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 2, HINT>), grid, dim3(nt), w64_shm(2 * wpb), stream, w, p, upw);
             return;
         }
     }
+    note_kernel("k_w64_mmv", tx_name<TX>(), 4, C, NC, 1, HINT);
     hipLaunchKernelGGL((k_w64_mmv<TX, C, NC, 1, HINT>), grid, dim3(nt), w64_shm(wpb), stream, w, p, upw);
 }
 template <typename TX, int C, int NC>

@@ -11,6 +11,15 @@
 namespace bf16n {
 namespace dev {
 
+// The kernel instance the calling thread's last product launcher chose: template name and its integer arguments, set
+// by the dispatch code itself (the benchmark names the kernel it timed from here instead of from a string of its own).
+struct kernel_note { const char * name; const char * tx; int n_args; int arg[5]; };
+extern thread_local kernel_note g_last_kernel;
+inline void note_kernel(const char * name, const char * tx, int n_args, int a0 = 0, int a1 = 0, int a2 = 0, int a3 = 0, int a4 = 0) {
+    g_last_kernel = {name, tx, n_args, {a0, a1, a2, a3, a4}};
+}
+template <typename TX> constexpr const char * tx_name() { return sizeof(TX) == 2 ? "bf16_t" : "float"; }
+
 // 32-lane layouts (kernels_compat.hip). glu: 0 plain, 1 merged [gate; up] NIBBLE matrix, 2 separate gate / up matrices
 bool nib_mm_pays(const bf16n_weight & w, int64_t nrows, int ncols, int cus);
 void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,

@@ -64,6 +64,13 @@ def layer_bytes(nbytes: dict, tokens: int, expected: bool = False) -> int:
     return dense + int((nbytes["gate"] + nbytes["up"] + nbytes["down"]) * experts) // EA
 
 
+def launches_per_layer(ops, tokens: int, gemv_path: bool) -> int:
+    """Kernel launches of one layer of Bf16nStep: qkv, o, glue, router, (top-k,) gate / up, down, glue."""
+    if gemv_path:
+        return 7 if getattr(ops, "TOPK_IN_EXPERT_GEMV", False) else 8
+    return 8 if tokens <= ops.TOPK_ROUTE_ONE_LAUNCH_TOKENS else 9
+
+
 def routing_buffers(n_tok: int, device) -> tuple[torch.Tensor, torch.Tensor]:
     """(weights f32, ids int32) [n_tok, 9]: columns 0..7 are written by the router's top-k in every step, column 8
     names the shared expert with weight 1."""

@@ -632,6 +632,12 @@ def router_topk_routes(logits: torch.Tensor, k: int, n_listed: int, renorm: bool
     return wts, ids, (src1, dst, bounds)
 
 
+def last_kernel() -> str:
+    """The kernel instance the calling thread's last dense product launch chose, as a profiler prints it
+    (bf16n_last_kernel; "" where the path leaves no note)."""
+    return _lib.lib().bf16n_last_kernel().decode()
+
+
 def glu2_supported(gate: Weight, up: Weight) -> bool:
     """Layouts with a fused gate / up + SwiGLU GEMV (the rule of bf16n::mmv_glu(gate, up), core launch.h:56-61, plus
     this build's wave64 units): same format, K, R and layout, not chunk-major."""
