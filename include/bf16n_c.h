@@ -95,6 +95,14 @@ int bf16n_linear_dense(const bf16n_weight * w, const uint16_t * x, int64_t x_row
                        void * scratch, uint64_t scratch_bytes, void * gemm_workspace, uint64_t gemm_workspace_bytes, void * stream);
 int bf16n_mmv_glu(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream);            /* mmv_glu merged [gate;up], launch.h:55, launch.cu:327-339 */
 int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf16n_mmv_args * a, void * stream); /* mmv_glu(gate, up), launch.h:61, launch.cu:341-365 */
+/* No counterpart in the reference (its engines run the router's softmax + top-k as a launch of their own between the
+ * router's product and the experts').  bf16n_mmv_glu2 over routed experts that selects them in its own prologue: one
+ * dependent launch fewer in a decode step.  a->ids: int32 id rows [tokens, n_used]; columns 0..k-1 are WRITTEN (the k
+ * largest of softmax(logits row), ties to the lower index, as bf16n_router_topk_strided writes them), columns from k on
+ * are read (experts every token uses).  weights: k softmax weights per token (renormalised to sum 1 if renorm) at
+ * weights + token * weights_stride.  Expert stacks in the tile layout, BF16 activations, at most 256 experts. */
+int bf16n_mmv_glu2_topk(const bf16n_weight * gate, const bf16n_weight * up, const bf16n_mmv_args * a, const float * logits,
+                        int64_t logits_stride, int n_experts, int k, int renorm, float * weights, int64_t weights_stride, void * stream);
 int bf16n_dequant(const bf16n_weight * w, int64_t row0, int64_t nrows, uint16_t * out, void * stream); /* dequant, launch.h:63, launch.cu:367-402 */
 int bf16n_get_rows(const bf16n_weight * w, const void * ids, int64_t ids_s0, int64_t n, void * dst, int dst_bf16,
                    int64_t dst_s1, void * stream, int64_t row0);                                /* get_rows, launch.h:68-69, launch.cu:404-443 */

@@ -47,6 +47,7 @@ SYMBOLS = {
     "bf16n_linear_dense": (_i, [_WP, _vp, _i64, _i, _vp, _i64, _vp, C.c_uint64, _vp, C.c_uint64, _vp]),
     "bf16n_mmv_glu": (_i, [_WP, _AP, _vp]),
     "bf16n_mmv_glu2": (_i, [_WP, _WP, _AP, _vp]),
+    "bf16n_mmv_glu2_topk": (_i, [_WP, _WP, _AP, _vp, _i64, _i, _i, _i, _vp, _i64, _vp]),
     "bf16n_dequant": (_i, [_WP, _i64, _i64, _vp, _vp]),
     "bf16n_get_rows": (_i, [_WP, _vp, _i64, _i64, _vp, _i, _i64, _vp, _i64]),
     "bf16n_mm_ids_supported": (_i, [_WP, _WP]),

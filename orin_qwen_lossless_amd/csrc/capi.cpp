@@ -4,6 +4,7 @@
 #include "bf16n_c.h"
 
 #include "encode_impl.h"
+#include "dev_topk.h"
 #include "launchers.h"
 
 #include <hip/hip_runtime.h>
@@ -272,9 +273,6 @@ int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, i
     });
 }
 
-// The number of BF16 token columns up to which bf16n_mmv is the faster dense path; beyond it dequant + a stock GEMM is.
-// 8 is the reference's fixed rule (core/torch/torch_bindings.cpp:195); matrices whose products run on the matrix cores
-// stay ahead for far longer (every pass of up to 128 columns decodes the matrix once).
 // The kernel instance that the calling thread's last bf16n_mmv / bf16n_mmv_glu2 launch chose, as the profiler prints it
 // ("k_w64_mmv<bf16_t, 4, 1, 2, 1>"); an empty string before the first launch or after a launch on a path that leaves
 // no note.  The pointer stays valid until the thread's next call of this function.
@@ -291,6 +289,9 @@ const char * bf16n_last_kernel(void) {
     return g_kernel_text.c_str();
 }
 
+// The number of BF16 token columns up to which bf16n_mmv is the faster dense path; beyond it dequant + a stock GEMM is.
+// 8 is the reference's fixed rule (core/torch/torch_bindings.cpp:195); matrices whose products run on the matrix cores
+// stay ahead for far longer (every pass of up to 128 columns decodes the matrix once).
 int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
     return guarded([&] {
         ensure_init();
@@ -363,6 +364,31 @@ int bf16n_mmv_glu2(const bf16n_weight * gate, const bf16n_weight * up, const bf1
             dev::launch_compat_mmv(*gate, up, 2, make_cols(*a), a->ncols, a->x_bf16 != 0, g_cus, (hipStream_t) stream);
         }
         launch_check("mmv_glu");
+    });
+}
+
+// No counterpart in the reference (whose engines run the router's top-k as a launch of their own): bf16n_mmv_glu2 over
+// routed experts that selects the experts in its own prologue.
+int bf16n_mmv_glu2_topk(const bf16n_weight * gate, const bf16n_weight * up, const bf16n_mmv_args * a, const float * logits,
+                        int64_t logits_stride, int n_experts, int k, int renorm, float * weights, int64_t weights_stride, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*gate);
+        check_weight(*up);
+        require(dev::is_tile_layout(*gate) && dev::is_tile_layout(*up) && gate->K == up->K && gate->rows == up->rows,
+                "mmv_glu2_topk: gate / up must be expert stacks of the same shape in the tile layout");
+        require(logits && weights && a->ids, "mmv_glu2_topk: null pointer");
+        require(n_experts > 0 && n_experts <= 256 && k > 0 && k <= n_experts && k <= 64 && k <= a->n_used,
+                "mmv_glu2_topk: need 0 < k <= min(n_experts, slots, 64) and at most 256 experts");
+        require(a->ids_s0 == 4 && a->x_bf16, "mmv_glu2_topk: int32 id rows and BF16 activations");
+        require(a->ncols > 0 && a->ncols <= 65535 && a->ncols % a->n_used == 0, "ncols must be tokens x slots");
+        require(a->nrows > 0 && a->nrows % gate->R == 0 && a->row0 % gate->R == 0 && a->rows_per_matrix % gate->R == 0,
+                "rows of a product must be whole units");
+        require(a->row0 >= 0 && a->row0 + a->nrows <= a->rows_per_matrix && (int64_t) n_experts * a->rows_per_matrix <= gate->rows,
+                "mmv_glu2_topk: product rows out of range");
+        const dev::topk_args ta = {logits, logits_stride, n_experts, k, renorm != 0, weights, weights_stride};
+        dev::launch_tile_mmv(*gate, up, make_cols(*a), a->ncols, true, (hipStream_t) stream, &ta);
+        launch_check("mmv_glu2_topk");
     });
 }
 

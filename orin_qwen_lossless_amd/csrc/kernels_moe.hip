@@ -2,6 +2,7 @@
 // and the router's softmax + top-k (on the device so that a decode step has no host round trip and can be captured
 // into a HIP graph).  All reductions run in a fixed order: results are bitwise reproducible.
 #include "dev_common.h"
+#include "dev_topk.h"
 #include "launchers.h"
 
 namespace bf16n {
@@ -158,65 +159,6 @@ __global__ void __launch_bounds__(ROUTE_THREADS) k_route(const char * __restrict
         if (e == (int) gridDim.x - 1) {
             bounds[gridDim.x] = base + done;
         }
-    }
-}
-
-// softmax over the experts, k largest (ties: lower index), weights renormalised to sum 1 if asked; one wave per token.
-// The logits of a token sit in registers (NQ per lane, expert = lane + 64 q); every selection is two wave reductions
-// on the VALU: the maximum, then the smallest index that holds it.  NaN logits count as -inf, and a selection only
-// ever returns an index below n_experts that was not taken before, whatever the values are: the ids feed address
-// arithmetic in the kernels that follow.
-template <int NQ>
-__device__ __forceinline__ void topk_token(const float * __restrict__ lg, int n_experts, int k, bool renorm, int32_t * ids_row,
-                                           float * weights_row, int lane, int * ids_copy = nullptr) {
-    float val[NQ];
-    bool open[NQ]; // a real expert that has not been taken yet
-    float mx = -INFINITY;
-#pragma unroll
-    for (int q = 0; q < NQ; q++) {
-        const int i = lane + 64 * q;
-        open[q] = i < n_experts;
-        const float v = open[q] ? lg[i] : -INFINITY;
-        val[q] = v != v ? -INFINITY : v;
-        mx = fmaxf(mx, val[q]);
-    }
-    mx = lane63(wave_max_dpp(mx));
-    float sum = 0.f;
-#pragma unroll
-    for (int q = 0; q < NQ; q++) {
-        sum += open[q] ? expf(val[q] - mx) : 0.f;
-    }
-    sum = lane63(wave_sum_dpp(sum));
-    float top = 0.f, mine = 0.f; // lane j keeps the j-th weight
-    for (int j = 0; j < k; j++) {
-        float bv = -INFINITY;
-#pragma unroll
-        for (int q = 0; q < NQ; q++) {
-            bv = open[q] ? fmaxf(bv, val[q]) : bv;
-        }
-        bv = lane63(wave_max_dpp(bv));
-        uint32_t bi = 0xFFFFFFFFu;
-#pragma unroll
-        for (int q = NQ - 1; q >= 0; q--) {
-            bi = open[q] && val[q] == bv ? (uint32_t) (lane + 64 * q) : bi; // descending q: the lane's lowest index stays
-        }
-        bi = lane63(wave_min_dpp(bi)); // k <= n_experts: an open expert holds the maximum of the open ones
-        const float pj = expf(bv - mx) / sum;
-        top += pj;
-        if (lane == (j & 63)) {
-            mine = pj; // k <= 64
-            ids_row[j] = (int32_t) bi;
-            if (ids_copy) {
-                ids_copy[j] = (int) bi;
-            }
-        }
-#pragma unroll
-        for (int q = 0; q < NQ; q++) {
-            open[q] = open[q] && (uint32_t) (lane + 64 * q) != bi;
-        }
-    }
-    if (lane < k) {
-        weights_row[lane] = renorm ? mine / top : mine;
     }
 }
 

@@ -12,6 +12,7 @@
 //   * k_tile_dequant, k_tile_get_rows: exact BF16 rows (launch.cu:367-443).
 #include "dev_common.h"
 #include "dev_compat.h"
+#include "dev_topk.h"
 #include "dev_w64.h"
 #include "launchers.h"
 
@@ -953,31 +954,75 @@ constexpr int tv_max_waves() { return GLU && sizeof(TX) == 2 ? TV_WAVES : TV_WAV
 // wavefront, many wavefronts) — and the partial sums (one per lane and row) of a group's `wpg` wavefronts per matrix
 // are added in tile order.  GLU: the group has wpg wavefronts on the gate matrix and wpg on the up matrix, and the
 // block writes silu(gate x) * (up x).
-template <typename TX, bool GLU, bool ONCE>
-__global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw) {
+// TOPK: the launch selects the experts itself (the router's softmax + top-k would otherwise be a launch of one
+// wavefront between the router's GEMV and this one).  Wavefront 0 of every block selects for the block's token from the
+// logits while the block stages its tables, and leaves the k ids in LDS; slots from k on (experts every token uses)
+// come from the id rows as before.  The first block of every token also writes the ids and weights to the rows that
+// the following launches read.  Every block of a token computes the same selection: the same function on the same
+// logits as k_router_topk.
+template <typename TX, bool GLU, bool ONCE, bool TOPK = false>
+__global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(const bf16n_weight w, const bf16n_weight w_up, const cols p, int wpg, int upw,
+                                                                             const topk_args ta = {}) {
     constexpr int NM = GLU ? 2 : 1;
+    constexpr int NQ = 4; // the fused selection takes up to 256 experts
     __shared__ __align__(16) uint32_t lut[NM * LUT_WORDS];
     __shared__ float part[TV_WAVES][32];
+    __shared__ int32_t sel_id[64];
+    __shared__ float sel_w[64];
     extern __shared__ __align__(16) uint32_t rings[];
     const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
     const int slabs = (int) (w.K / TILE_K), wpgm = NM * wpg, gpb = (int) (blockDim.x >> 6) / wpgm;
     const int gi = wave / wpgm, m = (wave % wpgm) / wpg, wi = wave % wpg; // group in the block, matrix, position in K
-    const col_view cv = col_setup(p, blockIdx.y);
+    col_view cv;
+    if constexpr (TOPK) {
+        const int t = (int) blockIdx.y / p.n_used, slot = (int) blockIdx.y % p.n_used;
+        float val[NQ];
+        bool open[NQ];
+        int32_t given = 0;
+        if (wave == 0) {
+            topk_load<NQ>(ta.logits + (int64_t) t * ta.stride, ta.n_experts, lane, val, open); // in flight beside the tables
+        }
+        if (slot >= ta.k) {
+            given = *(const int32_t *) (p.ids + t * p.ids_s1 + slot * p.ids_s0);
+        }
+        stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
+        if (GLU) {
+            stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
+        }
+        if (wave == 0) {
+            topk_select<NQ>(val, open, ta.k, ta.renorm, sel_id, sel_w, lane);
+        }
+        __syncthreads();
+        if (blockIdx.x == 0 && slot == 0 && tid < ta.k) { // the rows the next launches read
+            *(int32_t *) (const_cast<char *>(p.ids) + t * p.ids_s1 + tid * p.ids_s0) = sel_id[tid];
+            ta.weights[(int64_t) t * ta.out_stride + tid] = sel_w[tid];
+        }
+        const int e = slot < ta.k ? sel_id[slot] : given;
+        cv.x = p.x + t * p.x_tok + (slot % p.x_per_slot) * p.x_slot;
+        cv.y = p.y + t * p.y_tok + slot * p.y_slot;
+        cv.rbase = p.row0 + (int64_t) e * p.rows_per_matrix;
+    } else {
+        cv = col_setup(p, blockIdx.y);
+    }
     const int64_t groups = p.nrows / TILE_R, g = (int64_t) blockIdx.x * gpb + gi;
     const bool live = gi < gpb && g < groups;
     const w64_ptrs q = w64p(GLU && m ? w_up : w);
     const int64_t unit0 = live ? (cv.rbase / TILE_R + g) * slabs + wi * upw : 0;
     // the unit bases first: the stream loads that depend on them can start as soon as the tables are requested
     const uint32_t first = q.ubase[unit0], end = q.ubase[unit0 + upw];
-    stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
-    if (GLU) {
-        stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
+    if constexpr (!TOPK) {
+        stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
+        if (GLU) {
+            stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
+        }
     }
     tchain_t<4, ONCE> ch[1];
     if (live) {
         ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end, ONCE);
     }
-    __syncthreads();
+    if constexpr (!TOPK) {
+        __syncthreads();
+    }
     if (live) {
         const uint32_t * my_lut = lut + m * LUT_WORDS;
         float acc = 0.f;
@@ -1280,7 +1325,12 @@ void launch_tile_mm_dense(const bf16n_weight & w, int64_t row0, int64_t nrows, c
 }
 
 // y = W x (up == nullptr) or silu(gate x) * (up x), one column per launch row
-void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols & p, int ncols, bool x_bf16, hipStream_t stream) {
+void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols & p, int ncols, bool x_bf16, hipStream_t stream,
+                     const topk_args * topk) {
+    if (topk && !(up && x_bf16 && p.ids && p.ids_s0 == 4 && topk->n_experts <= 256 && topk->k <= p.n_used && topk->k <= 64)) {
+        throw std::invalid_argument("bf16n: the GEMV that selects its experts takes gate / up tiles, BF16 activations, int32 id rows, "
+                                    "at most 256 experts and k <= min(slots, 64)");
+    }
     const int slabs = (int) (w.K / TILE_K);
     // wavefronts per row group and matrix: one per tile where the block has room for them, else the fewest tiles per
     // wavefront that fit
@@ -1302,11 +1352,13 @@ void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols
     const dim3 nt(waves * 64);
 #define TILE_MMV(TX, GLU, UP)                                                                                   \
     if (once) {                                                                                                 \
-        hipLaunchKernelGGL((k_tile_mmv<TX, GLU, true>), grid, nt, shm, stream, w, UP, p, wpg, upw);             \
+        hipLaunchKernelGGL((k_tile_mmv<TX, GLU, true>), grid, nt, shm, stream, w, UP, p, wpg, upw, topk_args{});  \
     } else {                                                                                                    \
-        hipLaunchKernelGGL((k_tile_mmv<TX, GLU, false>), grid, nt, shm, stream, w, UP, p, wpg, upw);            \
+        hipLaunchKernelGGL((k_tile_mmv<TX, GLU, false>), grid, nt, shm, stream, w, UP, p, wpg, upw, topk_args{}); \
     }
-    if (up) {
+    if (topk) { // (every expert of a token is read once: the non-temporal loads)
+        hipLaunchKernelGGL((k_tile_mmv<bf16_t, true, true, true>), grid, nt, shm, stream, w, *up, p, wpg, upw, *topk);
+    } else if (up) {
         if (x_bf16) {
             TILE_MMV(bf16_t, true, *up)
         } else {

@@ -46,7 +46,9 @@ bool nib_mm_ids_ok(const bf16n_weight & w, const bf16n_weight * up);
 void launch_nib_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
                        const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
                        int64_t n_pairs, int cus, hipStream_t stream);
-void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols & p, int ncols, bool x_bf16, hipStream_t stream);
+struct topk_args;
+void launch_tile_mmv(const bf16n_weight & w, const bf16n_weight * up, const cols & p, int ncols, bool x_bf16, hipStream_t stream,
+                     const topk_args * topk = nullptr);
 void launch_tile_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, hipStream_t stream);
 void launch_tile_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_s0, int64_t n, void * dst, bool dst_bf16,
                           int64_t dst_s1, int64_t row0, hipStream_t stream);

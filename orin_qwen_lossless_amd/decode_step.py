@@ -90,7 +90,13 @@ class Bf16nStep:
         """(ys [T, 9, K] FP32 per-slot outputs, wts [T, 9], ids [T, 9])."""
         ops = self.ops
         logits, routes = ops.mmv(x2, w["router"]), None
-        if ops.moe_experts_batched(x2.shape[0], TOPK + 1, w["gate"], w["up"], w["down"], EA):
+        batched = ops.moe_experts_batched(x2.shape[0], TOPK + 1, w["gate"], w["up"], w["down"], EA)
+        if not batched and ops.topk_in_gemv_supported(w["gate"], w["up"], E, TOPK):
+            # the gate / up GEMV selects the experts itself: no top-k launch
+            wts, ids = self.routing
+            hidden = ops.mmv_glu2_topk(x2, w["gate"], w["up"], logits, TOPK, N_MID, self.routing)
+            return ops.mmv(hidden, w["down"], ids, K_MODEL), wts, ids
+        if batched:
             wts, ids, routes = ops.router_topk_routes(logits, TOPK, EA, out=self.routing)  # one launch up to 16 tokens
         else:
             wts, ids = ops.router_topk(logits, TOPK, out=self.routing)

@@ -273,7 +273,7 @@ def roundtrip_equal(w: Weight, src: torch.Tensor, chunk_bytes: int = 64 << 20) -
 
 
 def _mmv_common(x: torch.Tensor, w: Weight, ids: torch.Tensor | None, rows_per_matrix: int, out_bf16: bool, glu: bool,
-                multi_col: bool = True, up: Weight | None = None) -> torch.Tensor:
+                multi_col: bool = True, up: Weight | None = None, topk=None) -> torch.Tensor:
     """glu: w holds [gate; up] per matrix.  up given: w is the gate matrix and up a separate matrix of the same shape
     (the product is silu(gate x) * (up x) with as many rows as either)."""
     cw = _cweight(w)
@@ -336,7 +336,11 @@ def _mmv_common(x: torch.Tensor, w: Weight, ids: torch.Tensor | None, rows_per_m
         a.nrows = n_out
     L = _lib.lib()
     with torch.cuda.device(x.device):
-        if cu is not None:
+        if topk is not None:
+            logits, k, renorm, wts = topk
+            _lib.check(L.bf16n_mmv_glu2_topk(C.byref(cw), C.byref(cu), C.byref(a), logits.data_ptr(), logits.stride(0), logits.shape[1],
+                                             k, int(renorm), wts.data_ptr(), wts.stride(0), _stream()))
+        elif cu is not None:
             _lib.check(L.bf16n_mmv_glu2(C.byref(cw), C.byref(cu), C.byref(a), _stream()))
         elif glu:
             _lib.check(L.bf16n_mmv_glu(C.byref(cw), C.byref(a), _stream()))
@@ -363,6 +367,34 @@ def mmv_glu2(x: torch.Tensor, gate: Weight, up: Weight, ids: torch.Tensor | None
     if (gate.meta.K, gate.meta.rows) != (up.meta.K, up.meta.rows):
         raise ValueError("bf16n.mmv_glu: gate/up shapes must match")
     return _mmv_common(x, gate, ids, rows_per_matrix, out_dtype == torch.bfloat16, False, True, up)
+
+
+# the routed gate / up GEMV can select the experts itself (bf16n_mmv_glu2_topk): one launch fewer in a decode step
+TOPK_IN_EXPERT_GEMV = True
+
+
+def topk_in_gemv_supported(gate: Weight, up: Weight, n_experts: int, k: int) -> bool:
+    """Whether mmv_glu2_topk takes these expert stacks: the tile layout, at most 256 experts to select from."""
+    tiles = all(m.meta.wave64 and m.meta.R == 32 and m.meta.format == FMT_HUFPAIR for m in (gate, up))
+    return TOPK_IN_EXPERT_GEMV and tiles and n_experts <= 256 and 0 < k <= 64 and (gate.meta.K, gate.meta.rows) == (up.meta.K, up.meta.rows)
+
+
+def mmv_glu2_topk(x: torch.Tensor, gate: Weight, up: Weight, logits: torch.Tensor, k: int, rows_per_matrix: int,
+                  out: tuple[torch.Tensor, torch.Tensor], renorm: bool = True, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """router_topk(logits, k, renorm, out) and mmv_glu2(x, gate, up, ids, rows_per_matrix) in one launch
+    (bf16n_mmv_glu2_topk): every block of the GEMV selects its token's experts from the logits in its prologue.
+    out = (weights f32, ids int32) [tokens, m >= k]: columns 0..k-1 are written, the columns from k on are read as
+    further slots of every token (experts that all tokens use).  x: BF16 [tokens, K].  Returns [tokens, m, rows]."""
+    wts, ids = out
+    if not (logits.is_cuda and logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1):
+        raise ValueError("bf16n.mmv_glu2_topk: logits must be f32 [tokens, n_experts], contiguous along experts")
+    if not (wts.dtype == torch.float32 and ids.dtype == torch.int32 and wts.shape == ids.shape and wts.dim() == 2
+            and wts.shape[0] == logits.shape[0] and wts.shape[1] >= k and wts.is_contiguous() and ids.is_contiguous()
+            and wts.device == logits.device and ids.device == logits.device):
+        raise ValueError("bf16n.mmv_glu2_topk: out must be contiguous (f32, int32) [tokens, m >= k] tensors on the logits' device")
+    if x.dtype != torch.bfloat16 or x.dim() != 2:
+        raise ValueError("bf16n.mmv_glu2_topk: x must be bf16 [tokens, K]")
+    return _mmv_common(x, gate, ids, rows_per_matrix, out_dtype == torch.bfloat16, False, True, up, (logits, k, renorm, wts))
 
 
 def gemv_max_tokens(w: Weight) -> int:

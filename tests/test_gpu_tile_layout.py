@@ -351,3 +351,52 @@ def test_router_topk_and_routing_lists_in_one_launch(ops, oracle, T, E, k, extra
     s5, d5, b5 = ops.mm_ids_route(i4, n_listed, False)
     at = listed(i4, b5)
     assert torch.equal(b4, b5) and torch.equal(d4[at], d5[at]) and torch.equal(s4[at], s5[at])
+
+
+@pytest.mark.parametrize("T,E,k,extra,N,K", [(1, 256, 8, 1, 512, 2048), (3, 256, 8, 1, 512, 2048), (2, 40, 4, 0, 64, 512),
+                                              (1, 64, 6, 2, 96, 1024)])
+def test_gate_up_gemv_that_selects_its_experts(ops, T, E, k, extra, N, K):
+    """bf16n_mmv_glu2_topk: the routed gate / up GEMV with the router's softmax + top-k in its prologue writes the ids
+    and weights that bf16n_router_topk_strided writes and the products that bf16n_mmv_glu2 writes with those ids, bit
+    for bit; the columns of the id rows from k on (experts every token uses) are read and left alone; ties and NaN
+    logits select as the stand-alone kernel does."""
+    EA = E + extra
+    gate = enc(ops, synth.weights(EA * N, K, 801), HP, 32, False, True)
+    up = enc(ops, synth.weights(EA * N, K, 802), HP, 32, False, True)
+    assert ops.topk_in_gemv_supported(gate, up, E, k)
+    x = tbf16(synth.activations(T, K, 803))
+    lg = torch.randn((T, E), generator=torch.Generator().manual_seed(4)).cuda()
+    lg[0, 5] = lg[0, 9] = lg[0].max() + 1.0     # a tie at the top: the lower index first
+    lg[T - 1, 3] = float("nan")                  # NaN counts as -inf
+    n = k + extra
+
+    def rows():
+        wts = torch.full((T, n), 1.0, device="cuda")
+        ids = torch.full((T, n), -7, dtype=torch.int32, device="cuda")
+        for j in range(extra):
+            ids[:, k + j] = E + j
+        return wts, ids
+
+    w_ref, i_ref = ops.router_topk(lg, k, out=rows())
+    y_ref = ops.mmv_glu2(x, gate, up, i_ref, N)
+    w_f, i_f = rows()
+    y_f = ops.mmv_glu2_topk(x, gate, up, lg, k, N, (w_f, i_f))
+    assert torch.equal(i_f, i_ref) and torch.equal(w_f, w_ref)
+    assert int(i_f[0, 0]) == 5 and int(i_f[0, 1]) == 9 and 3 not in i_f[T - 1, :k].tolist()
+    assert torch.equal(y_f, y_ref)
+    y16 = ops.mmv_glu2_topk(x, gate, up, lg, k, N, rows(), out_dtype=torch.bfloat16)
+    assert torch.equal(y16, ops.mmv_glu2(x, gate, up, i_ref, N, out_dtype=torch.bfloat16))
+    # without renormalisation the weights are the softmax values themselves
+    w_n, i_n = rows()
+    ops.mmv_glu2_topk(x, gate, up, lg, k, N, (w_n, i_n), renorm=False)
+    w_s, _ = ops.router_topk(lg, k, renorm=False, out=rows())
+    assert torch.equal(w_n, w_s) and torch.equal(i_n, i_ref)
+    # the contract: int32 id rows of the logits' token count, tile-layout stacks, at most 256 experts
+    with pytest.raises(ValueError):
+        ops.mmv_glu2_topk(x, gate, up, lg, k, N, (w_f, i_f.long()))
+    with pytest.raises(ValueError):
+        ops.mmv_glu2_topk(x, gate, up, lg, n + 1, N, (w_f, i_f))
+    units = enc(ops, synth.weights(EA * N, K, 804), HP, 4, False, True)
+    assert not ops.topk_in_gemv_supported(units, units, E, k)
+    with pytest.raises(ValueError, match="tile layout"):
+        ops.mmv_glu2_topk(x, units, units, lg, k, N, rows())

@@ -41,7 +41,7 @@ def static_call(ops, x, ids, w, n_experts, up=None, out_dtype=torch.float32):
 def test_static_routing_lists_match_the_allocating_path(ops, layout):
     E, k, K, N = 24, 4, 2048, 512
     if layout == "nibble":  # expert stacks in the 4-bit code: the third dispatch branch of the entry point
-        gate, up, down = (enc(ops, synth.weights(r, c, 201 + i), 1, 1, False) for i, (r, c) in enumerate(((E * N, K), (E * N, K), (E * K, N))))
+        gate, up, down = (enc(ops, synth.weights(r, c, 201 + i), 1, 0, False) for i, (r, c) in enumerate(((E * N, K), (E * N, K), (E * K, N))))
     else:
         r_gu, r_dn = (32, 32) if layout == "tiles" else (4, 16)
         gate = enc(ops, synth.weights(E * N, K, 201), HP, r_gu, False, True)
