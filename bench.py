@@ -435,7 +435,7 @@ def suite(ops, w_head, head_copies, K: int) -> dict:
     return {"lm_head_batches": {"tiles": tdesc, "tiles_bytes": tbytes, "by_batch": batches}}
 
 
-def prefill_only(T: int, steps: int, mode: str = "hybrid") -> None:
+def prefill_only(T: int, steps: int, mode: str = "hybrid", two_phase_mib: int = 0) -> None:
     """Only the batched MoE kernels of one 35B-A3B-shaped layer (256 experts x (gate, up 512 x 2048; down 2048 x 512),
     top-8, experts in the mi355x policy's layout) on T tokens: routing lists once, then fused gate/up + SwiGLU (BF16)
     and down, `steps` times.  For profiling these kernels alone; prints its own JSON line."""
@@ -452,15 +452,20 @@ def prefill_only(T: int, steps: int, mode: str = "hybrid") -> None:
     x = synth.activations_torch(T, K, 34, "cuda")
     _, ids = ops.router_topk(synth.normal_torch(T * E, 35, "cuda").view(T, E), topk)
     src1, dst, bounds = ops.mm_ids_route(ids, E, False)
+    scratch = None
+    if two_phase_mib > 0:  # the two-phase form (expand a group of experts into scratch, multiply from there) for every call
+        ops.MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT = 1
+        scratch = torch.empty(two_phase_mib << 20, dtype=torch.uint8, device="cuda")
 
     def gate_up(i):
-        return ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds))
+        return ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=(src1, dst, bounds), scratch=scratch)
 
     a = gate_up(0)
     t_gu = med_us(gate_up, steps, 2)
-    t_dn = med_us(lambda i: ops.moe_mm_ids(a, ids, down, E, routes=(dst, dst, bounds)), steps, 2)
+    t_dn = med_us(lambda i: ops.moe_mm_ids(a, ids, down, E, routes=(dst, dst, bounds), scratch=scratch), steps, 2)
     flops_gu, flops_dn = 2.0 * T * topk * 2 * N * K, 2.0 * T * topk * K * N
     print(json.dumps({"workload": f"MoE prefill, {T} tokens, top-{topk} of {E} experts", "gate_up": gdesc, "down": ddesc,
+                      "form": f"two phases through {two_phase_mib} MiB of scratch" if two_phase_mib else "fused decode + matrix cores",
                       "gate_up_us": round(t_gu, 1), "down_us": round(t_dn, 1), "gate_up_bytes": gb + ub, "down_bytes": db,
                       "gate_up_TFLOPs": round(flops_gu / t_gu / 1e6, 1), "down_TFLOPs": round(flops_dn / t_dn / 1e6, 1),
                       "frac_of_bf16_mfma_peak": round((flops_gu + flops_dn) / (t_gu + t_dn) / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}))
@@ -514,6 +519,8 @@ def main() -> None:
     ap.add_argument("--suite", action="store_true", help="also sweep the output projection over batch sizes in both layouts")
     ap.add_argument("--prefill", type=int, default=0, metavar="T",
                     help="run only the batched MoE kernels of one layer on T tokens (for profiling) and exit")
+    ap.add_argument("--two-phase-mib", type=int, default=0, metavar="M",
+                    help="with --prefill: the two-phase form of the batched product (bf16n_mm_ids_scratch) through M MiB of scratch")
     ap.add_argument("--experts-4bit", action="store_true", help="with --prefill / --decode-step: the expert stacks in the 4-bit code (policy mode nibble)")
     ap.add_argument("--decode-step", type=int, default=0, metavar="T",
                     help="run only the 40-layer decode step at batch T (for profiling) and exit")
@@ -521,7 +528,7 @@ def main() -> None:
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path has no collective); run with --gpus 1")
     if args.prefill > 0:
-        prefill_only(args.prefill, min(args.steps, 20), "nibble" if args.experts_4bit else "hybrid")
+        prefill_only(args.prefill, min(args.steps, 20), "nibble" if args.experts_4bit else "hybrid", args.two_phase_mib)
         return
     if args.decode_step > 0:
         decode_only(args.decode_step, min(args.steps, 20), args.weight_sets, "nibble" if args.experts_4bit else "hybrid")

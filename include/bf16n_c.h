@@ -112,6 +112,16 @@ int bf16n_mm_ids_route(const void * ids, int ids_i64, int64_t ids_row_stride, in
 int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row,
                  const int32_t * ids_src1, const int32_t * ids_dst, const int32_t * bounds, void * dst, int dst_bf16,
                  int64_t dst_col, int n_experts, int n_tok, int n_used, void * stream);          /* launch.h:77-79, launch.cu:473-535 */
+/* No counterpart in the reference.  bf16n_mm_ids for calls with many tokens per expert (prefill), in two phases through
+ * a scratch buffer of the caller's: groups of experts are decoded once into the scratch (BF16, matrix-core operand
+ * order) by a kernel with the GEMV's decode rate and multiplied from there by a kernel without a decoder; the fused
+ * kernel of bf16n_mm_ids decodes an expert once per pass of 128 of its tokens.  Tile layout only.  scratch: 16-byte
+ * aligned device memory of at least *per_expert bytes (bf16n_mm_ids_scratch_bytes; *advised is the size whose groups
+ * stay in the last-level cache between the two kernels).  Same arguments and results as bf16n_mm_ids otherwise. */
+int bf16n_mm_ids_scratch_bytes(const bf16n_weight * w, const bf16n_weight * up, int n_experts, uint64_t * per_expert, uint64_t * advised);
+int bf16n_mm_ids_scratch(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row,
+                         const int32_t * ids_src1, const int32_t * ids_dst, const int32_t * bounds, void * dst, int dst_bf16,
+                         int64_t dst_col, int n_experts, void * scratch, uint64_t scratch_bytes, void * stream);
 /* No counterpart in the reference.  bf16n_mm_ids_route + bf16n_mm_ids in one call that allocates nothing, for callers
  * that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid it): the
  * routing lists are kept in a device array that belongs to the library (about 516 KiB per GPU, held until the process

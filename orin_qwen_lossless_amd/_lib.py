@@ -53,6 +53,8 @@ SYMBOLS = {
     "bf16n_mm_ids_supported": (_i, [_WP, _WP]),
     "bf16n_mm_ids_route": (_i, [_vp, _i, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "bf16n_mm_ids": (_i, [_WP, _WP, _vp, _i64, _vp, _vp, _vp, _vp, _i, _i64, _i, _i, _i, _vp]),
+    "bf16n_mm_ids_scratch_bytes": (_i, [_WP, _WP, _i, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "bf16n_mm_ids_scratch": (_i, [_WP, _WP, _vp, _i64, _vp, _vp, _vp, _vp, _i, _i64, _i, _vp, C.c_uint64, _vp]),
     "bf16n_moe_mm_ids_static": (_i, [_WP, _WP, _vp, _i64, _vp, _i, _i64, _i, _vp, _i, _i64, _i, _i, _i, _vp]),
     "bf16n_moe_combine": (_i, [_vp, _vp, _i, _vp, _i, _i, _i, _i64, _vp]),
     "bf16n_add_rmsnorm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i64, C.c_float, _vp]),

@@ -484,6 +484,47 @@ int bf16n_mm_ids(const bf16n_weight * w, const bf16n_weight * up, const void * x
     });
 }
 
+// No counterpart in the reference.  bf16n_mm_ids for calls with many tokens per expert, in two phases through a scratch
+// buffer of the caller's: groups of experts are decoded once into the scratch (as BF16, in matrix-core operand order)
+// and multiplied from there.  The result is the one of bf16n_mm_ids up to the order of the FP32 sums, which is the same
+// here (the same instruction sequence per output element).
+int bf16n_mm_ids_scratch_bytes(const bf16n_weight * w, const bf16n_weight * up, int n_experts, uint64_t * per_expert, uint64_t * advised) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        require(per_expert && advised, "null output");
+        require(dev::is_tile_layout(*w) && (!up || dev::is_tile_layout(*up)), "the two-phase batched product takes the tile layout only");
+        require(n_experts > 0 && w->rows % n_experts == 0, "rows must split evenly into experts");
+        *per_expert = dev::tile_mm_ids_scratch_per_expert(*w, up, n_experts);
+        // a group of experts should stay in the 256 MB last-level cache between its two kernels: about half of it
+        const uint64_t want = (uint64_t) 128 << 20;
+        uint64_t g = want / *per_expert;
+        g = g < 1 ? 1 : g > (uint64_t) n_experts ? (uint64_t) n_experts : g;
+        *advised = g * *per_expert;
+    });
+}
+
+int bf16n_mm_ids_scratch(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row,
+                         const int32_t * ids_src1, const int32_t * ids_dst, const int32_t * bounds, void * dst, int dst_bf16,
+                         int64_t dst_col, int n_experts, void * scratch, uint64_t scratch_bytes, void * stream) {
+    return guarded([&] {
+        ensure_init();
+        check_weight(*w);
+        if (up) {
+            check_weight(*up);
+        }
+        require(dev::is_tile_layout(*w) && (!up || (dev::is_tile_layout(*up) && up->rows == w->rows && up->K == w->K)),
+                "the two-phase batched product takes the tile layout only");
+        require(n_experts > 0 && w->rows % n_experts == 0, "rows must split evenly into experts");
+        require(x_bf16 && dst && ids_dst && bounds && scratch, "null pointer");
+        require(((uintptr_t) x_bf16 & 15) == 0 && x_row % 8 == 0, "activations must be 16-byte aligned with 16-byte row strides");
+        require(((uintptr_t) dst & 15) == 0 && dst_col % 4 == 0, "dst must be 16-byte aligned with a column stride that is a multiple of 4");
+        dev::launch_tile_mm_ids_expand(*w, up, x_bf16, x_row, ids_src1, ids_dst, bounds, dst, dst_bf16 != 0, dst_col, n_experts, scratch,
+                                       scratch_bytes, g_cus, (hipStream_t) stream);
+        launch_check("mm_ids_scratch");
+    });
+}
+
 // Routing lists + batched product in one call that allocates nothing: the lists live in the library's own device array
 // (see `scratch` above).  No counterpart in the reference, whose callers allocate the lists per call.
 int bf16n_moe_mm_ids_static(const bf16n_weight * w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const void * ids,

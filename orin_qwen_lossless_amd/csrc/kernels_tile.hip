@@ -468,6 +468,226 @@ __global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_tile(const bf
     }
 }
 
+// ---------------------------------------------------------------- batched MoE prefill in two phases (many tokens per expert)
+//
+// With a few hundred tokens per expert the fused kernel above decodes every expert once per pass of 128 tokens, at
+// half the decode chains per CU of the GEMV (its accumulators take the registers), and the decode is what it waits
+// for.  The two-phase form decodes a group of experts once, at the GEMV's chain count, into a scratch buffer of the
+// caller's (k_tile_expand), and multiplies from there with a kernel that has no decoder in its registers (k_mm_raw).
+// The scratch keeps the tiles in the decoder's own order, the A-operand order of the matrix instruction: tile u of
+// the group, step s, 16-column block kb, lane l -> 16 bytes at ((u * 8 + s) * 2 + kb) * 1024 + 16 l, so that both
+// kernels move whole 1 KiB rows per wavefront and instruction.  A group is sized to stay in the last-level cache
+// between the two kernels.
+constexpr int TILE_RAW_BYTES = TILE_R * TILE_K * 2;   // one tile as BF16
+constexpr int EXPAND_WAVES = 16;
+
+// chain c of the launch decodes tiles [c * tpc, (c + 1) * tpc) of matrix blockIdx.y (0: w, 1: w_up) from unit
+// unit_first on; two chains per wavefront.  Experts without tokens are skipped (bounds, tiles_per_expert).
+__global__ void __launch_bounds__(EXPAND_WAVES * 64) k_tile_expand(const bf16n_weight w, const bf16n_weight w_up, int64_t unit_first, int n_units,
+                                                                   int tpc, int tiles_per_expert, const int32_t * __restrict__ bounds,
+                                                                   uint4 * __restrict__ out) {
+    __shared__ __align__(16) uint32_t lut[LUT_WORDS];
+    extern __shared__ __align__(16) uint32_t rings[];
+    const int lane = threadIdx.x & 63, wave = (int) uniform(threadIdx.x >> 6);
+    const bool second = blockIdx.y != 0;
+    const w64_ptrs q = w64p(second ? w_up : w);
+    stage_lut(lut, q.lut);
+    const int n_chains = (n_units + tpc - 1) / tpc;
+    const int c0 = ((int) blockIdx.x * EXPAND_WAVES + wave) * 2;
+    __syncthreads();
+    if (c0 >= n_chains) {
+        return;
+    }
+    const bool two = c0 + 1 < n_chains;
+    int u0[2], n[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int c = two || k == 0 ? c0 + k : c0;  // a missing second chain repeats the first and stores nothing
+        u0[k] = c * tpc;
+        n[k] = n_units - u0[k] < tpc ? n_units - u0[k] : tpc;
+        if (bounds) {
+            const int e = (int) ((unit_first + u0[k]) / tiles_per_expert);
+            if (bounds[e + 1] == bounds[e]) {
+                n[k] = 0;
+            }
+        }
+    }
+    if (n[0] == 0 && (!two || n[1] == 0)) {
+        return;
+    }
+    // (a chain of an expert without tokens rides along with its neighbour and stores nothing)
+    const bool st0 = n[0] > 0, st1 = two && n[1] > 0;
+    if (!st0) { u0[0] = u0[1]; n[0] = n[1]; }
+    if (!st1) { u0[1] = u0[0]; n[1] = n[0]; }
+    const int steps = n[0] < n[1] ? n[1] : n[0];
+    tchain_t<4, true> ch[2];
+    uint32_t * ring = rings + wave * (2 * WAVE_LDS_WORDS);
+    ch[0].start(ring, q, unit_first + u0[0], n[0], lane, true);
+    ch[1].start(ring + WAVE_LDS_WORDS, q, unit_first + u0[1], n[1], lane, true);
+    uint4 * o0 = out + ((int64_t) (second ? n_units : 0) + u0[0]) * (TILE_RAW_BYTES / 16) + lane;
+    uint4 * o1 = out + ((int64_t) (second ? n_units : 0) + u0[1]) * (TILE_RAW_BYTES / 16) + lane;
+    for (int u = 0; u < steps; u++) { // (n[0] == n[1] except for the last chain of the launch, whose partner runs past its own end harmlessly: see below)
+        ch[0].begin_tile();
+        ch[1].begin_tile();
+#pragma unroll 1
+        for (int hh = 0; hh < 2; hh++) {
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                uint32_t wp[2][8];
+                tile_step<2, 4, true>(ch, lut, 0, s, wp);
+                ch[0].reload(s, lane);
+                ch[1].reload(s, lane);
+                const int so = ((4 * hh + s) * 2) * 64;
+                if (st0 && u < n[0]) {
+                    o0[so] = make_uint4(wp[0][0], wp[0][1], wp[0][2], wp[0][3]);
+                    o0[so + 64] = make_uint4(wp[0][4], wp[0][5], wp[0][6], wp[0][7]);
+                }
+                if (st1 && u < n[1]) {
+                    o1[so] = make_uint4(wp[1][0], wp[1][1], wp[1][2], wp[1][3]);
+                    o1[so + 64] = make_uint4(wp[1][4], wp[1][5], wp[1][6], wp[1][7]);
+                }
+            }
+        }
+        o0 += TILE_RAW_BYTES / 16;
+        o1 += TILE_RAW_BYTES / 16;
+    }
+}
+
+// The product from expanded tiles.  Work items, passes, staging of the activations and the stores are those of
+// k_mm_tile's 128-token shape; the A operands are loaded, two steps ahead, from the scratch (t0: tiles of w for the
+// experts [e0, e0 + n_e), t1: of w_up, or t0 again).
+template <bool GLU, int NT, int W>
+__global__ void __launch_bounds__((mt_shape<NT, W>::THREADS)) k_mm_raw(const uint4 * __restrict__ t0, const uint4 * __restrict__ t1, const mm_args a,
+                                                                       int e0, int n_e, int slabs) {
+    using S = mt_shape<NT, W>;
+    constexpr int D = 2; // steps of A operands in flight (four take 64 registers and spill)
+    extern __shared__ __align__(16) uint32_t shm[];
+    uint16_t * bbuf = (uint16_t *) shm; // two buffers of TOK x MT_BSTRIDE
+    const int tid = threadIdx.x, lane = tid & 63, l32 = tid & 31, half = lane >> 5, wave = (int) uniform(tid >> 6);
+    const int halves = 2 * slabs;
+    const int groups = (int) (a.rows / TILE_R);
+    constexpr int GPI = GLU ? S::WAVES : 2 * S::WAVES;
+    const int slabs_per_expert = (groups + GPI - 1) / GPI;
+    const bool stager = S::STAGERS == S::THREADS || wave < S::STAGERS / 64;
+    const int b_tok = stager ? tid / S::TPT : 0, b_part = tid % S::TPT;
+    constexpr int TU = TILE_RAW_BYTES / 16; // uint4 per tile
+    for (int item = blockIdx.x; item < n_e * slabs_per_expert; item += gridDim.x) {
+        const int el = item / slabs_per_expert, e = e0 + el, sl = item % slabs_per_expert;
+        const int j0 = a.bounds[e], n = a.bounds[e + 1] - j0;
+        const int g0 = GLU ? sl * GPI + wave : sl * GPI + 2 * wave;
+        const bool live = g0 < groups, has1 = GLU || g0 + 1 < groups;
+        const int g1 = GLU ? g0 : (has1 ? g0 + 1 : g0);
+        const uint4 * pa0 = t0 + ((int64_t) el * groups + (live ? g0 : 0)) * slabs * TU + lane;
+        const uint4 * pa1 = t1 + ((int64_t) el * groups + (live ? g1 : 0)) * slabs * TU + lane;
+        const int n_steps = T_STEPS * slabs;
+        for (int tp = 0; tp < n; tp += S::TOK) {
+            const int left = n - tp, nt = left >= S::TOK ? NT : (left + 31) >> 5;
+            const int btk = tp + b_tok;
+            const int bj = j0 + (btk < n ? btk : 0);
+            const uint16_t * xsrc = a.x + ((int64_t) (a.ids_src1 ? a.ids_src1[bj] : bj) * a.x_row + S::CPT * b_part);
+            uint16_t * bdst = bbuf + b_tok * MT_BSTRIDE + S::CPT * b_part;
+            uint4 f0, f1, f2, f3;
+            if (stager) {
+                MT_STAGE_LOAD(S::VPT, f0, f1, f2, f3, (const uint4 *) xsrc);
+            }
+            // A operands of the first D steps: [step][chain][16-column block]
+            uint4 av[D][2][2];
+#pragma unroll
+            for (int s = 0; s < D; s++) {
+                av[s][0][0] = pa0[(s * 2) * 64];
+                av[s][0][1] = pa0[(s * 2 + 1) * 64];
+                av[s][1][0] = pa1[(s * 2) * 64];
+                av[s][1][1] = pa1[(s * 2 + 1) * 64];
+            }
+            f32x16_t acc[2][NT];
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        acc[c][t][i] = 0.f;
+                    }
+                }
+            }
+            if (stager) {
+                MT_STAGE_STORE(S::VPT, f0, f1, f2, f3, (uint4 *) bdst);
+            }
+            __syncthreads();
+#pragma unroll 1
+            for (int hs = 0; hs < halves; hs++) {
+                const uint16_t * bcur = bbuf + (hs & 1) * (S::TOK * MT_BSTRIDE);
+                const int nxt = hs + 1 < halves ? hs + 1 : hs;
+                uint4 b0, b1, b2, b3;
+                if (stager) {
+                    MT_STAGE_LOAD(S::VPT, b0, b1, b2, b3, (const uint4 *) (xsrc + nxt * MT_HK));
+                }
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    const uint16_t * bp = bcur + l32 * MT_BSTRIDE + 32 * s + 8 * half;
+                    const int sd = s % D;
+                    const bf16x8_t a00 = __builtin_bit_cast(bf16x8_t, av[sd][0][0]), a01 = __builtin_bit_cast(bf16x8_t, av[sd][0][1]);
+                    const bf16x8_t a10 = __builtin_bit_cast(bf16x8_t, av[sd][1][0]), a11 = __builtin_bit_cast(bf16x8_t, av[sd][1][1]);
+                    // the same slot's operands D steps on (the last steps of a pass ask for the pass's last step again)
+                    const int st = 4 * hs + s + D, sn = st < n_steps ? st : n_steps - 1;
+                    av[sd][0][0] = pa0[(sn * 2) * 64];
+                    av[sd][0][1] = pa0[(sn * 2 + 1) * 64];
+                    av[sd][1][0] = pa1[(sn * 2) * 64];
+                    av[sd][1][1] = pa1[(sn * 2 + 1) * 64];
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        if (t == 0 || t < nt) {
+                            const bf16x8_t bv0 = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE);
+                            const bf16x8_t bv1 = *(const bf16x8_t *) (bp + t * 32 * MT_BSTRIDE + 16);
+                            acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a00, bv0, acc[0][t], 0, 0, 0);
+                            acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a10, bv0, acc[1][t], 0, 0, 0);
+                            acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a01, bv1, acc[0][t], 0, 0, 0);
+                            acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a11, bv1, acc[1][t], 0, 0, 0);
+                        }
+                    }
+                }
+                if (stager) {
+                    MT_STAGE_STORE(S::VPT, b0, b1, b2, b3, (uint4 *) (bdst + ((hs + 1) & 1) * (S::TOK * MT_BSTRIDE)));
+                }
+                __syncthreads();
+            }
+            if (live) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int tk = tp + 32 * t + l32;
+                    if (t < nt && tk < n) {
+                        const int64_t col = (int64_t) (a.ids_dst ? a.ids_dst[j0 + tk] : tk) * a.dst_col;
+#pragma unroll
+                        for (int c = 0; c < (GLU ? 1 : 2); c++) {
+                            if (c == 1 && !has1) {
+                                continue;
+                            }
+                            const int64_t row0 = (int64_t) (c ? g1 : g0) * TILE_R + 4 * half;
+#pragma unroll
+                            for (int g = 0; g < 4; g++) {
+                                float v[4];
+#pragma unroll
+                                for (int i = 0; i < 4; i++) {
+                                    const float p = acc[c][t][4 * g + i];
+                                    v[i] = GLU ? acc[1][t][4 * g + i] * silu(p) : p;
+                                }
+                                const int64_t o = col + row0 + 8 * g;
+                                if (a.dst_bf16) {
+                                    *(uint2 *) ((uint16_t *) a.dst + o) =
+                                        make_uint2(f32_to_bf16_rne(v[0]) | ((uint32_t) f32_to_bf16_rne(v[1]) << 16),
+                                                   f32_to_bf16_rne(v[2]) | ((uint32_t) f32_to_bf16_rne(v[3]) << 16));
+                                } else {
+                                    *(float4 *) ((float *) a.dst + o) = make_float4(v[0], v[1], v[2], v[3]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 // Few active experts (decode at small batch): a pass over an expert is one decode chain per wavefront, K / 32 steps
 // long, and nothing runs beside it, so the chain is cut instead: WPI wavefronts share a work item (expert, pair of row
 // groups, or gate and up of one group), each decodes K / 256 / WPI tiles per chain against its columns of the
@@ -1175,6 +1395,9 @@ void tile_init() {
     mt_attr<false, 1, 16>();
     lds_attr((const void *) k_mm_tile<false, 1, 16, true>, mt_shm<1, 16>(false));
     ks_attr<true>(); ks_attr<false>();
+    (void) hipFuncSetAttribute((const void *) k_tile_expand, hipFuncAttributeMaxDynamicSharedMemorySize, EXPAND_WAVES * 2 * WAVE_LDS_WORDS * 4);
+    (void) hipFuncSetAttribute((const void *) k_mm_raw<true, 4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 128 * MT_BSTRIDE * 2);
+    (void) hipFuncSetAttribute((const void *) k_mm_raw<false, 4, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 128 * MT_BSTRIDE * 2);
 }
 
 template <int W> int64_t mt_items(const mm_args & a, bool glu) {
@@ -1239,6 +1462,57 @@ void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const v
         mt_launch_small(w, up, a, n_pairs, cus, stream);
     } else {
         mt_launch<4, 8>(w, up, a, cus, stream);
+    }
+}
+
+// The two-phase form of launch_tile_mm_ids for calls with many tokens per expert: groups of experts are expanded into
+// `scratch` (bytes: at least one expert's tiles of w and up) and multiplied from there, group after group.
+uint64_t tile_mm_ids_scratch_per_expert(const bf16n_weight & w, const bf16n_weight * up, int n_experts) {
+    return (uint64_t) (w.rows / n_experts) * w.K * 2 * (up ? 2 : 1);
+}
+void launch_tile_mm_ids_expand(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
+                               const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
+                               void * scratch, uint64_t scratch_bytes, int cus, hipStream_t stream) {
+    mm_args a;
+    a.x = (const uint16_t *) x_bf16; a.x_row = x_row;
+    a.ids_src1 = ids_src1; a.ids_dst = ids_dst; a.bounds = bounds;
+    a.dst = (char *) dst; a.dst_col = dst_col; a.dst_bf16 = dst_bf16;
+    a.rows = w.rows / n_experts; a.n_experts = n_experts; a.n_tok = 0;
+    const uint64_t per_expert = tile_mm_ids_scratch_per_expert(w, up, n_experts);
+    if (a.rows % TILE_R != 0 || !scratch || ((uintptr_t) scratch & 15) != 0 || scratch_bytes < per_expert) {
+        throw std::invalid_argument("bf16n: the two-phase batched product needs rows per expert in multiples of 32 and a 16-byte "
+                                    "aligned scratch buffer for at least one expert's tiles as BF16");
+    }
+    const int slabs = (int) (w.K / TILE_K), groups = (int) (a.rows / TILE_R), tpe = groups * slabs;
+    int64_t G = (int64_t) (scratch_bytes / per_expert);
+    G = G < n_experts ? G : n_experts;
+    // groups of equal size (the last one is not a small remainder)
+    const int64_t n_groups = (n_experts + G - 1) / G;
+    G = (n_experts + n_groups - 1) / n_groups;
+    using S = mt_shape<4, 8>;
+    const size_t shm = (size_t) 2 * S::TOK * MT_BSTRIDE * 2;
+    for (int64_t e0 = 0; e0 < n_experts; e0 += G) {
+        const int n_e = (int) (n_experts - e0 < G ? n_experts - e0 : G);
+        const int n_units = n_e * tpe;
+        // chains enough for every CU's 32 slots where the group has them; a chain stays inside one expert
+        int tpc = 1;
+        const int64_t all_tiles = (int64_t) n_units * (up ? 2 : 1), slots = (int64_t) cus * 2 * EXPAND_WAVES;
+        while (all_tiles / (tpc * 2) >= slots && tpe % (tpc * 2) == 0) {
+            tpc *= 2;
+        }
+        const int n_chains = (n_units + tpc - 1) / tpc;
+        const dim3 grid((unsigned) ((n_chains + 2 * EXPAND_WAVES - 1) / (2 * EXPAND_WAVES)), up ? 2 : 1);
+        hipLaunchKernelGGL(k_tile_expand, grid, dim3(EXPAND_WAVES * 64), (size_t) EXPAND_WAVES * 2 * WAVE_LDS_WORDS * 4, stream, w, up ? *up : w,
+                           (int64_t) e0 * tpe, n_units, tpc, tpe, bounds, (uint4 *) scratch);
+        const uint4 * t0 = (const uint4 *) scratch;
+        const uint4 * t1 = up ? t0 + (int64_t) n_units * (TILE_RAW_BYTES / 16) : t0;
+        const int64_t items = (int64_t) n_e * ((groups + (up ? 8 : 16) - 1) / (up ? 8 : 16));
+        const dim3 g2((unsigned) (items < cus ? items : cus));
+        if (up) {
+            hipLaunchKernelGGL((k_mm_raw<true, 4, 8>), g2, dim3(S::THREADS), shm, stream, t0, t1, a, (int) e0, n_e, slabs);
+        } else {
+            hipLaunchKernelGGL((k_mm_raw<false, 4, 8>), g2, dim3(S::THREADS), shm, stream, t0, t1, a, (int) e0, n_e, slabs);
+        }
     }
 }
 

@@ -55,6 +55,10 @@ void launch_tile_get_rows(const bf16n_weight & w, const void * ids, int64_t ids_
 void launch_tile_mm_ids(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
                         const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
                         int64_t n_pairs, int cus, hipStream_t stream);
+uint64_t tile_mm_ids_scratch_per_expert(const bf16n_weight & w, const bf16n_weight * up, int n_experts);
+void launch_tile_mm_ids_expand(const bf16n_weight & w, const bf16n_weight * up, const void * x_bf16, int64_t x_row, const int32_t * ids_src1,
+                               const int32_t * ids_dst, const int32_t * bounds, void * dst, bool dst_bf16, int64_t dst_col, int n_experts,
+                               void * scratch, uint64_t scratch_bytes, int cus, hipStream_t stream);
 
 bool tile_mm_dense_pays(const bf16n_weight & w, int64_t nrows, int cus);
 constexpr int TILE_DENSE_F32_COLS = 10; // FP32 columns per dense tile product: three BF16 components each, 32 per pass

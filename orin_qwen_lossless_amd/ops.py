@@ -513,11 +513,34 @@ def mm_ids_route(topk_ids: torch.Tensor, n_experts: int, per_slot: bool):
     return src1, dst, bounds
 
 
+# moe_mm_ids: routed pairs per expert from which the tile layout's two-phase form (decode a group of experts into
+# scratch once, multiply from there) replaces the fused kernel, which decodes an expert once per 128 of its tokens.
+# Off by default: measured on a 256-expert layer it is behind the fused kernel at every token count (1.86 against 1.09
+# ms at 8192 tokens, 1.03 against 0.40 ms at 2048): writing and re-reading the experts as BF16 (1.6 GB a layer) costs
+# more than the second decode it saves.  Callers that pass `scratch` and lower this value get it.
+MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT = 1 << 30
+_mm_scratch: dict = {}
+
+
+def mm_ids_scratch(w: Weight, up: Weight | None, n_experts: int) -> torch.Tensor:
+    """The scratch buffer of the two-phase batched product for these expert stacks (the size the library advises: groups
+    of experts that stay in the last-level cache), one per device and size, kept for later calls."""
+    per, adv = C.c_uint64(0), C.c_uint64(0)
+    cw, cu = _cweight(w), _cweight(up) if up is not None else None
+    _lib.check(_lib.lib().bf16n_mm_ids_scratch_bytes(C.byref(cw), C.byref(cu) if cu is not None else None, n_experts, C.byref(per), C.byref(adv)))
+    key = (w.plane.device, adv.value)
+    if key not in _mm_scratch:
+        _mm_scratch[key] = torch.empty(adv.value, dtype=torch.uint8, device=w.plane.device)
+    return _mm_scratch[key]
+
+
 def moe_mm_ids(x: torch.Tensor, topk_ids: torch.Tensor, w: Weight, n_experts: int, up: Weight | None = None,
-               out_dtype: torch.dtype = torch.float32, routes=None) -> torch.Tensor:
+               out_dtype: torch.dtype = torch.float32, routes=None, scratch: torch.Tensor | None = None) -> torch.Tensor:
     """Batched MUL_MAT_ID over routed tokens (core/torch/torch_bindings.cpp:307-345): x [T, K] (gate / up) or
     [T, n_used, K] (down), BF16; out [T, n_used, N]; up given: fused gate/up + SwiGLU.  routes: the lists of
-    mm_ids_route(topk_ids, n_experts, x.dim() == 3) if the caller already has them (they are computed otherwise)."""
+    mm_ids_route(topk_ids, n_experts, x.dim() == 3) if the caller already has them (they are computed otherwise).
+    scratch: a uint8 device buffer for the two-phase form (tile layout, from MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT routed
+    pairs per expert on); None: the operator keeps one of the advised size per device (mm_ids_scratch)."""
     cw = _cweight(w)
     cu = _cweight(up) if up is not None else None
     _check_ids(topk_ids)
@@ -538,6 +561,14 @@ def moe_mm_ids(x: torch.Tensor, topk_ids: torch.Tensor, w: Weight, n_experts: in
     if not L.bf16n_mm_ids_supported(C.byref(cw), C.byref(cu) if cu is not None else None):
         raise ValueError("bf16n.moe_mm_ids: no batched kernel for this matrix (format/K/R/layout)")
     src1, dst, bounds = routes if routes is not None else mm_ids_route(topk_ids, n_experts, per_slot)
+    tiles = w.meta.wave64 and w.meta.R == 32 and w.meta.format == FMT_HUFPAIR and (up is None or (up.meta.wave64 and up.meta.R == 32))
+    if tiles and T * n_used >= MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT * n_experts:
+        buf = scratch if scratch is not None else mm_ids_scratch(w, up, n_experts)
+        with torch.cuda.device(x.device):
+            _lib.check(L.bf16n_mm_ids_scratch(C.byref(cw), C.byref(cu) if cu is not None else None, x.data_ptr(), w.meta.K,
+                                              src1.data_ptr(), dst.data_ptr(), bounds.data_ptr(), y.data_ptr(),
+                                              int(out_dtype == torch.bfloat16), N, n_experts, buf.data_ptr(), buf.numel(), _stream()))
+        return y
     with torch.cuda.device(x.device):
         _lib.check(L.bf16n_mm_ids(C.byref(cw), C.byref(cu) if cu is not None else None, x.data_ptr(), w.meta.K,
                                   src1.data_ptr(), dst.data_ptr(), bounds.data_ptr(), y.data_ptr(),

@@ -400,3 +400,40 @@ def test_gate_up_gemv_that_selects_its_experts(ops, T, E, k, extra, N, K):
     assert not ops.topk_in_gemv_supported(units, units, E, k)
     with pytest.raises(ValueError, match="tile layout"):
         ops.mmv_glu2_topk(x, units, units, lg, k, N, rows())
+
+
+@pytest.mark.parametrize("E,N,K,T,k,scratch_experts", [(8, 512, 2048, 300, 4, 8), (8, 512, 2048, 300, 4, 3), (6, 96, 512, 700, 2, 1),
+                                                        (16, 64, 1024, 2100, 1, 5)])
+def test_two_phase_batched_product_equals_the_fused_kernel(ops, E, N, K, T, k, scratch_experts, monkeypatch):
+    """bf16n_mm_ids_scratch (experts decoded once into a scratch buffer in matrix-core operand order, multiplied from
+    there) writes the bits of bf16n_mm_ids (the same matrix instructions in the same order per output element): fused
+    gate / up + SwiGLU, BF16 and FP32 out, the plain product and the down product, with scratch for all experts, for
+    some (several groups, the last smaller) and for one; an expert without tokens is skipped."""
+    gate = enc(ops, synth.weights(E * N, K, 811), HP, 32, False, True)
+    up = enc(ops, synth.weights(E * N, K, 812), HP, 32, False, True)
+    down = enc(ops, synth.weights(E * K, N, 813), HP, 32, False, True) if N % 512 == 0 else None
+    x = tbf16(synth.activations(T, K, 814))
+    rng = np.random.default_rng(11)
+    ids_np = np.stack([rng.permutation(E - 1)[:k] for _ in range(T)]).astype(np.int32)  # the last expert has no tokens
+    ids = torch.from_numpy(ids_np).cuda()
+    routes = ops.mm_ids_route(ids, E, False)
+    monkeypatch.setattr(ops, "MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT", 10 ** 9)
+    want16 = ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=routes)
+    want32 = ops.moe_mm_ids(x, ids, gate, E, up=up, routes=routes)
+    want_g = ops.moe_mm_ids(x, ids, gate, E, routes=routes)
+    monkeypatch.setattr(ops, "MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT", 1)
+    per = 2 * N * K * 2
+    buf = torch.empty(scratch_experts * per + 4096, dtype=torch.uint8, device="cuda")
+    got16 = ops.moe_mm_ids(x, ids, gate, E, up=up, out_dtype=torch.bfloat16, routes=routes, scratch=buf)
+    assert torch.equal(got16.view(torch.int16), want16.view(torch.int16))
+    assert torch.equal(ops.moe_mm_ids(x, ids, gate, E, up=up, routes=routes, scratch=buf), want32)
+    assert torch.equal(ops.moe_mm_ids(x, ids, gate, E, routes=routes, scratch=buf), want_g)
+    assert torch.equal(ops.moe_mm_ids(x, ids, gate, E, up=up, routes=routes), want32)   # the operator's own scratch
+    if down is not None:
+        r3 = (routes[1], routes[1], routes[2])
+        monkeypatch.setattr(ops, "MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT", 10 ** 9)
+        want_d = ops.moe_mm_ids(want16, ids, down, E, routes=r3)
+        monkeypatch.setattr(ops, "MM_IDS_TWO_PHASE_PAIRS_PER_EXPERT", 1)
+        assert torch.equal(ops.moe_mm_ids(want16, ids, down, E, routes=r3, scratch=buf), want_d)
+    with pytest.raises(ValueError, match="scratch"):
+        ops.moe_mm_ids(x, ids, gate, E, up=up, routes=routes, scratch=buf[: per // 2])
