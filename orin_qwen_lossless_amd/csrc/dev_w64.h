@@ -95,6 +95,7 @@ struct w64_dec_t {
     uint32_t * ring;
     range_t src;            // the blocks that hold words of this wave (starts on a 128-byte line)
     uint4 pend;             // the block that starts at `filled`, in flight
+    uint4 first_blk;        // the first block between start and start_finish
     int lane;
     bool once;              // stream blocks with the non-temporal hint (same in every lane)
 
@@ -116,7 +117,8 @@ struct w64_dec_t {
         }
     }
     // stream words [first, end) of the aux stream belong to this wave
-    __device__ __forceinline__ void start(uint32_t * ring_, const uint32_t * stream, uint32_t first, uint32_t end, int lane_, bool once_ = false) {
+    __device__ __forceinline__ void start(uint32_t * ring_, const uint32_t * stream, uint32_t first, uint32_t end, int lane_, bool once_ = false,
+                                          bool split = false) {
         ring = ring_;
         lane = lane_;
         once = once_;
@@ -129,9 +131,16 @@ struct w64_dec_t {
         // whole blocks up to the one that holds the last word (the stream is padded: a block may run past `end`)
         const uint32_t blocks = (uint32_t) ((int32_t) end - a - 1) / BLK + 1;
         src = make_range(stream + (int32_t) uniform((uint32_t) a), uniform(blocks * BLK * 4));
-        const uint4 b0 = load_block(0);
+        first_blk = load_block(0);
         pend = load_block(BLK);
-        store_block(0, b0);
+        if (!split) {
+            start_finish();
+        }
+    }
+    // the second half of start(..., split = true): callers put other loads between the request of a chain's first
+    // blocks and the wait for them
+    __device__ __forceinline__ void start_finish() {
+        store_block(0, first_blk);
         filled = BLK;
     }
     // at least AHEAD words in the ring beyond the consumer; the block after them in flight.  At most one block per
@@ -207,9 +216,13 @@ struct w64_dec_t {
 };
 typedef w64_dec_t<-1> w64_dec;
 
+// Every block of a launch stages the same 16 KiB; the blocks start at different 1 KiB pieces of it so that they do not
+// all ask for the same cache lines at the same moment.
 __device__ __forceinline__ void stage_lut(uint32_t * lut, const uint32_t * lut_g) {
+    const int rot = (int) ((blockIdx.x + 5 * blockIdx.y) * 64) & (LUT_WORDS / 4 - 1);
     for (int i = threadIdx.x; i < LUT_WORDS / 4; i += blockDim.x) {
-        ((uint4 *) lut)[i] = ((const uint4 *) lut_g)[i];
+        const int k = (i + rot) & (LUT_WORDS / 4 - 1);
+        ((uint4 *) lut)[k] = ((const uint4 *) lut_g)[k];
     }
 }
 

@@ -54,7 +54,7 @@ template <int D, bool ONCE = false> struct tchain_t {
     }
     // first / end: the stream words of the units (their unit bases, read by the caller ahead of time)
     __device__ __forceinline__ void start(uint32_t * ring, const w64_ptrs & q, int64_t unit0, int n_units, int lane, uint32_t first,
-                                          uint32_t end, bool stream_once = false) {
+                                          uint32_t end, bool stream_once = false, bool split = false) {
         plane = make_range(q.plane + uniform64(unit0 * T_BYTES), uniform((uint32_t) (n_units * T_BYTES)));
         off = 16 * (uint32_t) lane;
 #pragma unroll
@@ -62,7 +62,7 @@ template <int D, bool ONCE = false> struct tchain_t {
             sm[s] = load_step(lane);
             off += STEP_BYTES;
         }
-        dec.start(ring, q.stream, uniform(first), uniform(end), lane, stream_once);
+        dec.start(ring, q.stream, uniform(first), uniform(end), lane, stream_once, split);
     }
     // s: the step just consumed (a compile-time value at every call)
     __device__ __forceinline__ void reload(int s, int lane) {
@@ -1230,17 +1230,19 @@ __global__ void __launch_bounds__((tv_max_waves<TX, GLU>()) * 64) k_tile_mmv(con
     const int64_t unit0 = live ? (cv.rbase / TILE_R + g) * slabs + wi * upw : 0;
     // the unit bases first: the stream loads that depend on them can start as soon as the tables are requested
     const uint32_t first = q.ubase[unit0], end = q.ubase[unit0 + upw];
+    tchain_t<4, ONCE> ch[1];
+    if (live) {
+        ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end, ONCE, !TOPK);
+    }
     if constexpr (!TOPK) {
+        // the chain's first stream and plane loads travel while the tables are staged
         stage_lut(lut, (const uint32_t *) (w.aux + w.off_a));
         if (GLU) {
             stage_lut(lut + LUT_WORDS, (const uint32_t *) (w_up.aux + w_up.off_a));
         }
-    }
-    tchain_t<4, ONCE> ch[1];
-    if (live) {
-        ch[0].start(rings + wave * WAVE_LDS_WORDS, q, unit0, upw, lane, first, end, ONCE);
-    }
-    if constexpr (!TOPK) {
+        if (live) {
+            ch[0].dec.start_finish();
+        }
         __syncthreads();
     }
     if (live) {
