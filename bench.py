@@ -392,7 +392,9 @@ def configs(ops, w_head, head_copies, comp_bytes: int, K: int, n_sets: int = 40)
     t_steady = med_us(lambda i: graph8.replay(), 32, 4) / 8
     del graph8
     touched = nbytes["router"] + (nbytes["gate"] + nbytes["up"] + nbytes["down"]) * (D.TOPK + 1) // D.EA
-    out["moe_layer_batch1_graph"] = {"us": round(t_layer, 2), "us_per_layer_of_8_in_one_graph": round(t_steady, 2), "launches": 5,
+    fused_topk = ops.topk_in_gemv_supported(sets[0]["gate"], sets[0]["up"], D.E, D.TOPK)
+    out["moe_layer_batch1_graph"] = {"us": round(t_layer, 2), "us_per_layer_of_8_in_one_graph": round(t_steady, 2),
+                                     "launches": 4 if fused_topk else 5,  # router, (top-8,) gate/up, down, weighted sum + norm
                                      "compressed_bytes_touched": int(touched),
                                      "GBps": round(touched / t_layer / 1e3, 1), "frac_of_hbm_peak": round(touched / t_layer / 1e3 / HBM_PEAK_GBS, 4),
                                      "experts": "256 routed (top-8, softmax weights renormalised) + 1 shared, 32x256 tiles"}
