@@ -22,7 +22,7 @@ def test_more_than_one_gpu_is_refused():
 def test_one_json_line_with_roofline_and_cpu_baseline():
     # a reduced matrix (the same kernel instance: K = 2048, 16-row units) so that the test takes seconds
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--rows", "65536", "--steps", "10", "--warmup", "2",
-                        "--cpu-rows", "2048", "--cpu-seconds", "3"], capture_output=True, text=True, timeout=900)
+                        "--cpu-rows", "2048", "--cpu-seconds", "3", "--weight-sets", "8"], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
     assert len(lines) == 1
@@ -55,9 +55,17 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     for key in ("lm_head_batch4", "gemv_512x2048", "gemv_2048x512", "moe_layer_batch1_graph", "moe_prefill_T2048", "moe_prefill_T8192",
                 "decode_step"):
         assert key in cf, key
+    assert cf["decode_step"]["weight_sets"] == 8
     for b in ("batch1", "batch4", "batch16"):
         e = cf["decode_step"][b]
         assert e["us"] > 0 and e["bf16_us"] > 0 and e["eager_equals_graph"] and 0 < e["frac_of_hbm_peak"] < 1
+        # both stock-kernel comparators up to four tokens, the speed-up against the faster of them
+        best = min(e["bf16_us"], e["bf16_static_ids_us"]) if b != "batch16" else e["bf16_us"]
+        assert abs(e["speedup_vs_bf16"] - best / e["us"]) < 0.02
+    # the kernel name comes from the library's dispatch, the stock GEMV is timed like the headline kernel
+    assert rf["kernel"].startswith("k_w64_mmv<bf16_t, 4, 1, ") and "blas_timing" in d["extra"]
+    b4 = cf["lm_head_batch4"]
+    assert b4["units_of_16_rows"]["kernel"].startswith("k_w64_mmv<bf16_t, 4, 4, ") and b4["matrix_core_tiles"]["us"] > 0
         assert abs(e["speedup_vs_bf16"] - e["bf16_us"] / e["us"]) < 0.02
     e4 = cf["decode_step"]["experts_4bit_code"]
     assert e4["batch1"]["us"] > 0 and e4["batch4"]["us"] > 0 and 1.0 < e4["expert_bytes_vs_tiles"] < 1.2
