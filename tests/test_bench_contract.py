@@ -66,7 +66,6 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert rf["kernel"].startswith("k_w64_mmv<bf16_t, 4, 1, ") and "blas_timing" in d["extra"]
     b4 = cf["lm_head_batch4"]
     assert b4["units_of_16_rows"]["kernel"].startswith("k_w64_mmv<bf16_t, 4, 4, ") and b4["matrix_core_tiles"]["us"] > 0
-        assert abs(e["speedup_vs_bf16"] - e["bf16_us"] / e["us"]) < 0.02
     e4 = cf["decode_step"]["experts_4bit_code"]
     assert e4["batch1"]["us"] > 0 and e4["batch4"]["us"] > 0 and 1.0 < e4["expert_bytes_vs_tiles"] < 1.2
     for T in (2048, 8192):
