@@ -360,8 +360,11 @@ typedef float nm_f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t nm_u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int NM_WAVES = 8; // per block: K / 256 half chunks in one turn each, K > 2048 in two
 
-// TURNS: half chunks per wavefront (wavefront v takes v TURNS + [0, TURNS)).  Every load of a wavefront is issued before
-// the first is used: a launch is a few serial latencies long, and eight wavefronts per block leave the registers for it.
+// TURNS: half chunks per wavefront (wavefront v takes v TURNS + [0, TURNS)).  The loads of a wavefront are written
+// ahead of their uses; with one turn the compiler issues them in batches of about nine (68 registers, three blocks per
+// CU).  All 28 pinned ahead of the first use (a scheduling barrier; 148 registers) measured 2 to 6 % faster for
+// 5120 x 2048 up to 32 columns, 30 % slower at 64 (one block per CU), and with two turns 5 to 7 % slower (256
+// registers and spills): left to the compiler.
 template <int TURNS>
 __global__ void __launch_bounds__(NM_WAVES * 64) k_nib_mm(const bf16n_weight w, const cols p, const int ncols) {
     extern __shared__ __align__(16) float nm_part[]; // [wavefront][accumulator register][lane]
