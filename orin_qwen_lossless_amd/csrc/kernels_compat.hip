@@ -359,6 +359,12 @@ typedef __bf16 nm_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float nm_f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t nm_u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int NM_WAVES = 8; // per block: K / 256 half chunks in one turn each, K > 2048 in two
+// Words per (wavefront, accumulator register) row of the partial sums in LDS: lane l at l + l / 32.  The threads that add
+// the partial sums of one token's 32 rows read 16 registers x 2 half-waves of one lane position: 64 words apart they
+// all met one bank (32-way conflicts: 7,900 conflict cycles per block, 3 of a launch's 14 us), 66 apart with the
+// upper half-wave shifted by one they spread over all banks, two to a bank.
+constexpr int NM_PSTRIDE = 66;
+__device__ __forceinline__ int nm_part_at(int wave, int i, int lane) { return (wave * 16 + i) * NM_PSTRIDE + lane + (lane >> 5); }
 
 // TURNS: half chunks per wavefront (wavefront v takes v TURNS + [0, TURNS)).  The loads of a wavefront are written
 // ahead of their uses; with one turn the compiler issues them in batches of about nine (68 registers, three blocks per
@@ -425,7 +431,7 @@ __global__ void __launch_bounds__(NM_WAVES * 64) k_nib_mm(const bf16n_weight w, 
     }
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-        nm_part[(wave * 16 + i) * 64 + lane] = acc[i];
+        nm_part[nm_part_at(wave, i, lane)] = acc[i];
     }
     __syncthreads();
     // accumulator register i of lane l: row 8 (i / 4) + 4 (l / 32) + i % 4 of the group, token l % 32.  A thread per
@@ -433,11 +439,11 @@ __global__ void __launch_bounds__(NM_WAVES * 64) k_nib_mm(const bf16n_weight w, 
     for (int e = (int) threadIdx.x; e < 1024; e += (int) blockDim.x) {
         const int tok = e >> 5, rr = e & 31;
         const int i = 4 * (rr >> 3) + (rr & 3), l = tok + 32 * ((rr >> 2) & 1);
-        float v = 0.f;
-        for (int k = 0; k < n_waves; k++) {
-            v += nm_part[(k * 16 + i) * 64 + l];
-        }
         if (g0 + rr < p.nrows && t0 + tok < ncols) {
+            float v = 0.f;
+            for (int k = 0; k < n_waves; k++) {
+                v += nm_part[nm_part_at(k, i, l)];
+            }
             const char * xt = p.x + (int64_t) (t0 + tok) * p.x_tok;
             for (uint32_t k = esc0; k < esc1; k++) {
                 const uint32_t rec = q.esc[k];
@@ -529,7 +535,7 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
         p.x_tok % 16 == 0) {
         const int halves = (int) (w.K / 256), turns = halves > NM_WAVES ? 2 : 1, waves = (halves + turns - 1) / turns;
         const dim3 grid((unsigned) nm_blocks, (unsigned) ((ncols + 31) / 32));
-        const size_t shm = (size_t) waves * 16 * 64 * sizeof(float);
+        const size_t shm = (size_t) waves * 16 * NM_PSTRIDE * sizeof(float);
         if (turns == 2) {
             hipLaunchKernelGGL(k_nib_mm<2>, grid, dim3(waves * 64), shm, stream, w, p, ncols);
         } else {
