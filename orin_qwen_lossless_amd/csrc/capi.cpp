@@ -310,8 +310,13 @@ int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out) {
             // 2048 x 4096: 17-21 us against 22-28 us), where the dispatch takes that kernel for every count from 9 to
             // 64; matrices of up to 256 rows run their GEMV columns side by side on idle CUs (4.9-9.5 us for 9-64
             // columns); between the two the GEMV columns lose to dequant + GEMM beyond the reference's 8
-            const bool all_counts = dev::nib_mm_pays(*w, w->rows, 9, g_cus) && dev::nib_mm_pays(*w, w->rows, 64, g_cus);
-            *out = all_counts || w->rows <= 256 ? 64 : 8;
+            // (the 16-row kernel takes over where its launch is at most two blocks per CU: 1024 x 2048 6.5-6.8 us up to
+            // 64 columns against 15.4 us for dequant + GEMM)
+            bool all_counts = true;
+            for (int n = 9; n <= 64 && all_counts; n++) {
+                all_counts = dev::nib_mm_pays(*w, w->rows, n, g_cus) || dev::nib_mm16_pays(*w, w->rows, n, g_cus);
+            }
+            *out = all_counts || w->rows <= 256 ? 64 : dev::nib_mm16_pays(*w, w->rows, 16, g_cus) ? 16 : 8;
         } else {
             *out = 8;
         }

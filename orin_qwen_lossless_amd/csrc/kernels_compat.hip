@@ -454,6 +454,83 @@ __global__ void __launch_bounds__(NM_WAVES * 64) k_nib_mm(const bf16n_weight w, 
     }
 }
 
+// The same product for at most 16 token columns per block on 16-row groups (v_mfma_f32_16x16x32_bf16): twice the blocks
+// of k_nib_mm, which matters while its groups of 32 rows leave CUs idle (2048 rows: 64 blocks on 256 CUs).  Lane
+// (row r of 16, k part q of 4) decodes two adjacent slots of its row per step, 8 n + 2 q and the next: eight adjacent
+// columns 128 j + 32 n + 8 q + [0, 8) in each of the chunk's four column blocks j, the A operands of four matrix
+// instructions (k positions 8 q + [0, 8) of instruction j); lane (token t of 16, q) supplies the same columns of its
+// token as B operands.  A wavefront takes STEPS consecutive steps of a row (a chunk is four steps); the partial sums of
+// the wavefronts are added in K order through LDS (rows of 68 words: the 64 threads that add for four tokens meet every
+// bank twice), the products of escaped weights last.
+typedef float nm_f32x4_t __attribute__((ext_vector_type(4)));
+constexpr int NM16_PSTRIDE = 68;
+template <int STEPS>
+__global__ void __launch_bounds__(NM_WAVES * 64) k_nib_mm16(const bf16n_weight w, const cols p, const int ncols) {
+    extern __shared__ __align__(16) float nm_part[]; // [wavefront][accumulator register][lane]
+    const nib_ptrs q = nibp(w, 0);
+    const int K = (int) w.K;
+    const int lane = threadIdx.x & 63, r = lane & 15, kq = lane >> 4, wave = (int) (threadIdx.x >> 6), n_waves = (int) (blockDim.x >> 6);
+    const int64_t g0 = (int64_t) blockIdx.x * 16;
+    const int64_t row = p.row0 + (g0 + r < p.nrows ? g0 + r : p.nrows - 1);
+    const int t0 = (int) blockIdx.y * 16;
+    const char * x = p.x + (int64_t) (t0 + r < ncols ? t0 + r : ncols - 1) * p.x_tok;
+    const uint4 T = *(const uint4 *) (q.table + row * 16);
+    // the sums this thread finishes at the end are (token, row) = (e / 16, e % 16) for e = thread, thread + block size
+    const int64_t my_row = g0 + (threadIdx.x & 15);
+    const int64_t my_gr = p.row0 + (my_row < p.nrows ? my_row : p.nrows - 1);
+    const uint32_t esc0 = q.esc_off[my_gr], esc1 = q.esc_off[my_gr + 1];
+    const int first = wave * STEPS, c = first >> 2, s0 = 8 * (first & 3) + 2 * kq; // this lane's first slot
+    const uint8_t * pl = q.plane + row * K + c * CHUNK + 16 * s0;
+    const uint8_t * cd = q.codes + row * (K / 2) + c * (CHUNK / 2) + 8 * s0;
+    const char * xb = x + 2 * (c * CHUNK + 4 * s0);
+    uint4 sm0[STEPS], sm1[STEPS], cdv[STEPS], b[STEPS][4];
+#pragma unroll
+    for (int n = 0; n < STEPS; n++) {
+        sm0[n] = *(const uint4 *) (pl + 128 * n);
+        sm1[n] = *(const uint4 *) (pl + 128 * n + 16);
+        cdv[n] = *(const uint4 *) (cd + 64 * n);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            b[n][j] = *(const uint4 *) (xb + 64 * n + 256 * j);
+        }
+    }
+    nm_f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int n = 0; n < STEPS; n++) {
+        uint32_t w0[8], w1[8];
+        nib_chunk(sm0[n], make_uint2(cdv[n].x, cdv[n].y), T, w0);
+        nib_chunk(sm1[n], make_uint2(cdv[n].z, cdv[n].w), T, w1);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const nm_u32x4_t a = {w0[2 * j], w0[2 * j + 1], w1[2 * j], w1[2 * j + 1]};
+            const nm_u32x4_t bv = {b[n][j].x, b[n][j].y, b[n][j].z, b[n][j].w};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(nm_bf16x8_t, a), __builtin_bit_cast(nm_bf16x8_t, bv), acc, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        nm_part[(wave * 4 + i) * NM16_PSTRIDE + lane] = acc[i];
+    }
+    __syncthreads();
+    // accumulator register i of lane l: row 4 (l / 16) + i of the group, token l % 16
+    for (int e = (int) threadIdx.x; e < 256; e += (int) blockDim.x) {
+        const int tok = e >> 4, rr = e & 15;
+        const int i = rr & 3, l = tok + 16 * (rr >> 2);
+        if (g0 + rr < p.nrows && t0 + tok < ncols) {
+            float v = 0.f;
+            for (int k = 0; k < n_waves; k++) {
+                v += nm_part[(k * 4 + i) * NM16_PSTRIDE + l];
+            }
+            const char * xt = p.x + (int64_t) (t0 + tok) * p.x_tok;
+            for (uint32_t k = esc0; k < esc1; k++) {
+                const uint32_t rec = q.esc[k];
+                v = fmaf(bf16_bits_to_f32(esc_bits(rec)), x_at<bf16_t>(xt, (int) (rec & 0xFFFu)), v);
+            }
+            store_y(p.y + (int64_t) (t0 + tok) * p.y_tok, p.y_bf16, g0 + rr, v);
+        }
+    }
+}
+
 // exact rows of a NIBBLE matrix: FP32 or BF16, to out + i * stride (bytes); row index from ids (gather) or row0 + i
 template <bool BF>
 __global__ void __launch_bounds__(NT) k_nib_rows(const bf16n_weight w, const char * __restrict__ ids, int64_t ids_s0, int64_t n,
@@ -509,6 +586,30 @@ int grid_for(int64_t work, int ncols, int cus) {
 
 } // namespace
 
+// Steps per wavefront of k_nib_mm16 (a row has K / 128): the fewest for which a block has at most eight wavefronts, or
+// four (fewer, longer wavefronts) when the row groups outnumber the CUs anyway; 0: K does not fit the kernel.
+int nib_mm16_steps(const bf16n_weight & w, int64_t nrows, int cus) {
+    if (w.format != FMT_NIBBLE || w.K % CHUNK != 0 || w.K / 128 > 4 * NM_WAVES) {
+        return 0;
+    }
+    const int steps_all = (int) (w.K / 128);
+    const int fewest = steps_all <= NM_WAVES ? 1 : steps_all <= 2 * NM_WAVES ? 2 : 4;
+    return fewest == 2 && (nrows + 15) / 16 > cus ? 4 : fewest;
+}
+// Whether a dense batch of BF16 columns takes the 16-row matrix-core kernel (k_nib_mm16): by the CUs its row groups
+// fill, from two columns (a group per CU), three (half of them) or five (a quarter) on; smaller matrices stay with the
+// GEMV columns, which run side by side on idle CUs (256 x 2048: 3.2-4.6 us at 2-16 columns against 4.7-5.9; 512 x 4096:
+// 4.6-9.3 against 7.4-10.0).  Beyond 16 columns every block of 16 tokens decodes the matrix again, which still wins
+// while the launch is at most two blocks per CU (2048 x 4096: 10.5-10.7 us at 17-32 columns and 15.7-17.3 at 40-64
+// against 16.5-19.9 in 32-row groups; 1024 x 2048: 6.5-6.8 us up to 64 against 10.7-12.8; 5120 x 2048, 640 blocks at
+// 17 columns: 12.4 against 11.2, left to the 32-row groups).  The dispatch below and bf16n_gemv_max_tokens share this
+// rule.
+bool nib_mm16_pays(const bf16n_weight & w, int64_t nrows, int ncols, int cus) {
+    const int64_t groups = (nrows + 15) / 16, token_blocks = (ncols + 15) / 16;
+    const bool enough = (ncols >= 2 && groups >= cus) || (ncols >= 3 && groups * 2 >= cus) || (ncols >= 5 && groups * 4 >= cus);
+    return enough && (token_blocks == 1 || groups * token_blocks <= 2 * (int64_t) cus) && nib_mm16_steps(w, nrows, cus) != 0;
+}
+
 // Whether a dense batch of `ncols` BF16 columns over `nrows` rows of a 4-bit-code matrix goes through the matrix cores
 // (k_nib_mm): the row groups of 32 must give enough CUs a block, by column count.  The dispatch below and
 // bf16n_gemv_max_tokens share this rule.
@@ -531,9 +632,25 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
     // GEMV columns at 9 / 16 / 32 / 64).  Smaller matrices stay with the GEMV columns, which run side by side on idle CUs
     // (256 x 2048: 4.9-9.5 us for 9-64 columns against 10.5-12.6 us here).
     const int64_t nm_blocks = (p.nrows + 31) / 32;
+    if (matrix_cores && !p.ids && glu == 0 && x_bf16 && nib_mm16_pays(w, p.nrows, ncols, cus) && ((uintptr_t) p.x & 15) == 0 &&
+        p.x_tok % 16 == 0) {
+        // 16-row groups (5120 x 2048: 7.7 / 8.2 / 8.8 / 10.5 us at 2 / 4 / 8 / 16 columns against 8.3 / 11.4
+        // in GEMV columns and 9.7 / 10.8 in 32-row groups; 2048 x 4096: 8.0 / 8.2 / 9.0 / 10.3 us at 3 / 4 / 8 / 16
+        // against 9.4 / 9.3 / 15.3 / 15.5; 1024 x 2048: 5.6 / 6.5 us at 5 / 16 against 6.8 / 9.1; 2048 x 512: 3.3 / 3.6
+        // us at 2 / 16 against 3.5 / 5.5)
+        const int steps = nib_mm16_steps(w, p.nrows, cus), waves = (int) (w.K / 128) / steps;
+        note_kernel("k_nib_mm16", nullptr, 1, steps);
+        const dim3 grid((unsigned) ((p.nrows + 15) / 16), (unsigned) ((ncols + 15) / 16));
+        const size_t shm = (size_t) waves * 4 * NM16_PSTRIDE * sizeof(float);
+        if (steps == 1)      hipLaunchKernelGGL(k_nib_mm16<1>, grid, dim3(waves * 64), shm, stream, w, p, ncols);
+        else if (steps == 2) hipLaunchKernelGGL(k_nib_mm16<2>, grid, dim3(waves * 64), shm, stream, w, p, ncols);
+        else                 hipLaunchKernelGGL(k_nib_mm16<4>, grid, dim3(waves * 64), shm, stream, w, p, ncols);
+        return;
+    }
     if (matrix_cores && !p.ids && glu == 0 && x_bf16 && nib_mm_pays(w, p.nrows, ncols, cus) && ((uintptr_t) p.x & 15) == 0 &&
         p.x_tok % 16 == 0) {
         const int halves = (int) (w.K / 256), turns = halves > NM_WAVES ? 2 : 1, waves = (halves + turns - 1) / turns;
+        note_kernel("k_nib_mm", nullptr, 1, turns);
         const dim3 grid((unsigned) nm_blocks, (unsigned) ((ncols + 31) / 32));
         const size_t shm = (size_t) waves * 16 * NM_PSTRIDE * sizeof(float);
         if (turns == 2) {
@@ -552,6 +669,7 @@ void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu,
         const int nc = p.ids ? 1 : fills ? (ncols >= 3 ? 4 : ncols == 2 ? 2 : 1) : ncols >= 16 ? 4 : ncols >= 8 ? 2 : 1;
         const int ngroups = (ncols + nc - 1) / nc;
         const dim3 grid(grid_for((p.nrows + rpb - 1) / rpb * HALVES, ngroups, cus), ngroups);
+        note_kernel("k_nib_mmv", x_bf16 ? "bf16_t" : "float", 2, glu, nc);
 #define NIBC(TX, G, N) hipLaunchKernelGGL((k_nib_mmv<TX, G, N>), grid, dim3(NT), 0, stream, w, wu, p, ncols)
 #define NIB(TX, G) do { if (nc == 4) NIBC(TX, G, 4); else if (nc == 2) NIBC(TX, G, 2); else NIBC(TX, G, 1); } while (0)
         if (x_bf16) { if (glu == 0) NIB(bf16_t, 0); else if (glu == 1) NIB(bf16_t, 1); else NIB(bf16_t, 2); }

@@ -22,6 +22,7 @@ template <typename TX> constexpr const char * tx_name() { return sizeof(TX) == 2
 
 // 32-lane layouts (kernels_compat.hip). glu: 0 plain, 1 merged [gate; up] NIBBLE matrix, 2 separate gate / up matrices
 bool nib_mm_pays(const bf16n_weight & w, int64_t nrows, int ncols, int cus);
+bool nib_mm16_pays(const bf16n_weight & w, int64_t nrows, int ncols, int cus);
 void launch_compat_mmv(const bf16n_weight & w, const bf16n_weight * up, int glu, const cols & p, int ncols, bool x_bf16,
                        int cus, hipStream_t stream, bool matrix_cores = true);
 void launch_compat_dequant(const bf16n_weight & w, int64_t row0, int64_t nrows, uint16_t * out, int cus, hipStream_t stream);

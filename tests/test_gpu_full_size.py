@@ -455,27 +455,34 @@ def test_dense_matrices_of_the_decode_step(ops, oracle, name, rows, k, mode, wan
     xb = synth.activations(4, k, 77)
     x = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16).cuda()
     y4 = ops.mmv(x, enc).cpu().numpy()
+    on_matrix_cores = ops.last_kernel().startswith("k_nib_mm16<")   # the 4-bit code: four columns in 16-row groups
+    assert on_matrix_cores == (fmt == 1)
+    y4_cols = ops.mmv(x, enc, multi_col=False).cpu().numpy()         # per-column launches
     for t in range(4):
         xf = synth.bf16_bits_to_f32(xb[t])
         ref32 = oracle.gemv_f32(wb, xf)
         y64, bound = oracle.gemv_f64(wb, xf)
         y1 = ops.mmv(x[t: t + 1], enc).cpu().numpy()[0]
-        assert np.array_equal(y1, y4[t])                       # batch 4 = four batch-1 products, bit for bit
-        assert np.all(np.abs(y1 - ref32) <= 1e-3 * np.abs(ref32) + 1e-5)
-        assert np.all(np.abs(y1 - y64) <= 1e-5 * bound)
+        assert np.array_equal(y1, y4_cols[t])                  # four batch-1 products, bit for bit
+        if not on_matrix_cores:
+            assert np.array_equal(y1, y4[t])                   # the column groups of the wave64 GEMV keep those bits
+        for y in (y1, y4[t]):
+            assert np.all(np.abs(y - ref32) <= 1e-3 * np.abs(ref32) + 1e-5)
+            assert np.all(np.abs(y - y64) <= 1e-5 * bound)
     y16 = ops.linear(x, enc)
     assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y4))
 
 
 @pytest.mark.parametrize("rows,k", [(5120, 2048), (2048, 4096), (1000, 512)])
 def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, oracle, rows, k):
-    """Dense batches on a 4-bit matrix, escapes included.  Few BF16 columns (and FP32 columns) share decodes on the VALU
-    and have the bits of their single-column products.  From nine BF16 columns on — from five where the matrix has row
-    groups for half of the CUs, from 25 where for an eighth only, never with fewer — the product runs on the matrix
-    cores, 32 tokens per decode: there a column has the same
-    bits at every batch size and at every position (a token's sum never meets another token's), within the FP64 bound
-    of the GEMV.  Rows that are no multiple of 32 and batches that are no multiple of 32 tokens leave a ragged last
-    block."""
+    """Dense batches on a 4-bit matrix, escapes included.  FP32 columns, and BF16 columns on a matrix too small for the
+    matrix cores, share decodes on the VALU and have the bits of their single-column products.  Up to 16 BF16 columns
+    run on the matrix cores in 16-row groups where these fill the CUs (from two columns), half of them (from three) or
+    a quarter (from five), also in several blocks of 16 tokens while the launch is at most two blocks per CU; larger
+    batches in 32-row groups, 32 tokens per decode (with groups for a quarter of the CUs, from 25 columns with an
+    eighth).  On either kernel a column has the same bits at every batch size and at every
+    position (a token's sum never meets another token's), within the FP64 bound of the GEMV.  Rows that are no multiple
+    of the group and batches that are no multiple of the token block leave a ragged last block."""
     from orin_qwen_lossless_amd import synth
 
     wb = synth.weights(rows, k, 900 + rows % 89)
@@ -487,22 +494,46 @@ def test_nibble_projection_columns_share_a_decode_bit_for_bit(ops, oracle, rows,
     xb = synth.activations(70, k, 78)
     x = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16).cuda()
     single = torch.cat([ops.mmv(x[t: t + 1], enc) for t in range(9)])
-    blocks, cus = (rows + 31) // 32, torch.cuda.get_device_properties(0).multi_processor_count
-    first = 5 if blocks * 2 >= cus else 9 if blocks * 4 >= cus else 25 if blocks * 8 >= cus else 10 ** 9
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    g16, g32 = (rows + 15) // 16, (rows + 31) // 32
+    first16 = 2 if g16 >= cus else 3 if g16 * 2 >= cus else 5 if g16 * 4 >= cus else 10 ** 9
+    first32 = 5 if g32 * 2 >= cus else 9 if g32 * 4 >= cus else 25 if g32 * 8 >= cus else 10 ** 9
+
+    def on_16_row_groups(T):  # several blocks of 16 tokens while the launch stays within two blocks per CU
+        return T >= first16 and (T <= 16 or g16 * ((T + 15) // 16) <= 2 * cus)
+
     y70 = ops.mmv(x, enc)
-    for T in (2, 3, 4, 5, 8, 9, 31, 32, 33, 64):
-        assert torch.equal(ops.mmv(x[:T], enc), single[:T] if T < first else y70[:T]), T
-    assert torch.equal(ops.mmv(x[37:65], enc), y70[37:65])  # other positions in the block of 32
-    assert not torch.equal(y70[:9], single)                 # (the two paths do differ: another order of summation)
-    y70n = y70.cpu().numpy()
+    assert not on_16_row_groups(70) or first32 > 70
+    by16 = torch.cat([ops.mmv(x[i: i + 16], enc) for i in range(0, 64, 16)])  # (on 16-row groups wherever a batch is)
+    y16 = by16[:16]
+    for T in (2, 3, 4, 5, 8, 9, 16, 17, 24, 25, 31, 32, 33, 64):
+        y = ops.mmv(x[:T], enc)
+        kernel = ops.last_kernel()
+        if on_16_row_groups(T):
+            assert kernel.startswith("k_nib_mm16<") and torch.equal(y, by16[:T]), (T, kernel)
+        elif T >= first32:
+            assert kernel.startswith("k_nib_mm<") and torch.equal(y, y70[:T]), (T, kernel)
+        else:
+            assert kernel.startswith("k_nib_mmv<") and torch.equal(y[:9], single[:T]), (T, kernel)
+    if first32 <= 28 and not on_16_row_groups(28):
+        assert torch.equal(ops.mmv(x[37:65], enc), y70[37:65])  # other positions in the block of 32
+        assert not torch.equal(y70[:9], single)                 # (the two paths do differ: another order of summation)
+    if first16 <= 9:
+        assert torch.equal(ops.mmv(x[5:14], enc), y16[5:14])    # other positions in the block of 16
+        assert not torch.equal(y16[:9], single)
+    y70n, y16n = y70.cpu().numpy(), y16.cpu().numpy()
     for t in (0, 2, 31, 32, 69):
         y64, bound = oracle.gemv_f64(wb, synth.bf16_bits_to_f32(xb[t]))
         assert np.all(np.abs(y70n[t] - y64) <= 1e-5 * bound), t
         if t < 9:
             assert np.all(np.abs(single[t].cpu().numpy() - y64) <= 1e-5 * bound), t
+            assert np.all(np.abs(y16n[t] - y64) <= 1e-5 * bound), t
     # BF16 out: the one rounding of the FP32 sums
-    y16 = ops.mmv(x[:30], enc, out_dtype=torch.bfloat16)
-    assert np.array_equal(y16.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(y70n[:30]))
+    for n, ref in ((70, y70n), (12, y16n)):
+        yb = ops.mmv(x[:n], enc, out_dtype=torch.bfloat16)
+        assert np.array_equal(yb.cpu().view(torch.int16).numpy().view(np.uint16), synth.f32_to_bf16_bits(ref[:n]))
+    # a caller that asks for per-column launches gets the single-column bits at any count
+    assert torch.equal(ops.mmv(x[:9], enc, multi_col=False), single)
     xf = x[:4].float()
     single_f = torch.cat([ops.mmv(xf[t: t + 1], enc) for t in range(4)])
     assert torch.equal(ops.mmv(xf, enc), single_f)

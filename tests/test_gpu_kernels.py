@@ -106,6 +106,49 @@ def test_nibble_column_groups_equal_single_columns(ops, oracle, K):
             assert torch.equal(ops.mmv_glu(x[:T], w), g1[:T]), (T, x.dtype)
 
 
+@pytest.mark.parametrize("rows,K,first", [(4104, 512, 2), (4104, 1024, 2), (1030, 2048, 5), (4360, 2048, 2), (2056, 4096, 3), (2048, 1536, 3)])
+def test_nibble_few_columns_on_16_row_groups(ops, oracle, rows, K, first):
+    """Dense NIBBLE batches of up to 16 BF16 columns over matrices whose 16-row groups fill the CUs (from two columns),
+    half of them (from three) or a quarter (from five) run on the matrix cores in 16-row groups (k_nib_mm16): every step
+    count per wavefront (K = 512 .. 4096), a last group of fewer than 16 rows, escaped weights there and elsewhere,
+    strided activation rows, several blocks of 16 tokens; within the oracle's bounds, the BF16 output the rounding of
+    the FP32 one, and a token's bits the same at every batch size and position the kernel takes.  FP32 activations keep
+    the GEMV columns."""
+    assert ops.cu_count() == 256, "the thresholds of this test are those of 256 CUs"
+    wb = synth.weights(rows, K, rows + K)
+    for r, col in ((0, 3), (17, K - 1), (rows - 1, 7), (rows - 3, K // 2)):
+        wb[r, col] = 0x4500 if r % 2 else 0xC4FF                     # exponents outside the rows' tables: escapes
+    w = enc(ops, wb, NIB, 0, False, False)
+    xb = synth.activations(16, K, K + rows)
+    xf = synth.bf16_bits_to_f32(xb)
+    x = tbf16(xb)
+    y16 = ops.mmv(x, w)
+    assert ops.last_kernel().startswith("k_nib_mm16<")
+    check_gemv(oracle, y16[[0, 9, 15]].cpu().numpy(), wb, xf[[0, 9, 15]])
+    assert np.array_equal(bits(ops.mmv(x, w, out_dtype=torch.bfloat16)), rne_bf16(y16.cpu().numpy()))
+    for T in range(1, 16):
+        yT = ops.mmv(x[:T], w)
+        took = ops.last_kernel().startswith("k_nib_mm16<")
+        assert took == (T >= first), (T, ops.last_kernel())
+        if took:
+            assert torch.equal(yT, y16[:T]), T
+        else:
+            check_gemv(oracle, yT[T - 1:].cpu().numpy(), wb, xf[T - 1: T])
+    wide = torch.zeros((16, K + 64), dtype=x.dtype, device="cuda")
+    wide[:, :K] = x
+    assert torch.equal(ops.mmv(wide[:, :K], w), y16)
+    # more than 16 columns: blocks of 16 tokens, each column as in a batch of its own (two blocks per CU at most)
+    x40 = torch.cat([x, x.flip(0), x[:8]])
+    groups = (rows + 15) // 16
+    y40 = ops.mmv(x40, w)
+    assert ops.last_kernel().startswith("k_nib_mm16<") == (groups * 3 <= 512), ops.last_kernel()
+    if groups * 3 <= 512:
+        assert torch.equal(y40, torch.cat([y16, y16.flip(0), y16[:8]]))
+    y_f32 = ops.mmv(torch.from_numpy(xf[:5]).cuda(), w)
+    assert ops.last_kernel().startswith("k_nib_mmv<float")
+    check_gemv(oracle, y_f32[[0, 4]].cpu().numpy(), wb, xf[[0, 4]])
+
+
 @pytest.mark.parametrize("fmt,R,cm,w64", LAYOUTS)
 def test_one_hot_activations_give_exact_weights(ops, fmt, R, cm, w64):
     K, rows = 2048, 64
