@@ -78,9 +78,14 @@ typedef struct bf16n_mmv_args {
 int bf16n_init(void);                 /* init(), launch.h:47, launch.cu:270-306: once per process, before graph capture */
 int bf16n_cu_count(int * out);        /* sm_count(), launch.h:48 */
 int bf16n_mmv(const bf16n_weight * w, const bf16n_mmv_args * a, void * stream, int multi_col); /* mmv, launch.h:52, launch.cu:313-325 */
+/* (multi_col, launch.h:52: columns of a dense batch may share decodes.  0: every column has the bits of its own
+ * single-column launch.  Non-zero: the same, except where a dense batch of BF16 columns runs on the matrix cores (tile
+ * layout; the 4-bit code from two columns on for matrices that fill the GPU): there a column has the same bits at every
+ * batch size and position, another summation order than the single-column GEMV, the same error bound.) */
 /* the dense dispatch rule: BF16 token columns up to which bf16n_mmv beats dequant + GEMM for this matrix (8, the
  * reference's fixed rule, core/torch/torch_bindings.cpp:195 and ops.py:25-27; 16 for matrices of 128 Mi weights and more
- * in wave64 units; 64 for the 4-bit code, whose batches run on the matrix cores; 512 for tile-layout matrices there) */
+ * in wave64 units; 64 for the 4-bit code where its batches run on the matrix cores at every count, 16 where up to 16
+ * columns; 512 for tile-layout matrices there) */
 int bf16n_gemv_max_tokens(const bf16n_weight * w, int * out);
 /* The dense path beyond bf16n_gemv_max_tokens: y (n_tok x rows, BF16) = x (n_tok x K, BF16) W^T through exact dequant of
  * the matrix, in pieces of at most 64 MiB, into `scratch`, and a stock BF16 GEMM with FP32 accumulation (hipBLASLt) on
