@@ -14,7 +14,9 @@ Per layer (pre-norm, residual stream h in BF16):
 256 experts x (gate 512 x 2048, up 512 x 2048, down 2048 x 512) and one shared expert of the same shape.  The shared
 expert is stacked behind the routed ones as expert 256 and runs as a ninth slot of every token with weight 1: its two
 products ride in the routed experts' launches instead of two launches of their own (run on a second stream beside the
-routed ones they cost more than in line: the fork and join of the graph outweighed them).  8 launches per layer."""
+routed ones they cost more than in line: the fork and join of the graph outweighed them).  7 launches per layer while
+the experts run as GEMV columns (the gate / up launch selects them itself), 8 with the batched kernels up to 8 tokens
+(selection and routing lists in one launch), 9 beyond."""
 from __future__ import annotations
 
 import numpy as np
