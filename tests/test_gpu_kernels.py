@@ -149,6 +149,37 @@ def test_nibble_few_columns_on_16_row_groups(ops, oracle, rows, K, first):
     check_gemv(oracle, y_f32[[0, 4]].cpu().numpy(), wb, xf[[0, 4]])
 
 
+@pytest.mark.parametrize("T", [6, 70])
+def test_nibble_batches_over_a_row_range_through_the_c_abi(ops, T):
+    """bf16n_mmv with row0 / nrows (a view of some rows of a tensor, as the engine adapter hands them over) on the
+    matrix-core kernels of the 4-bit code: the product over rows [row0, row0 + nrows) is that slice of the whole
+    product, bit for bit, with a first row that is no multiple of the row groups and a ragged last group."""
+    import ctypes as C
+
+    from orin_qwen_lossless_amd import _lib
+
+    rows, K, row0, nrows = 4400, 1024, 1030, 2213
+    wb = synth.weights(rows, K, 991)
+    wb[row0 + 5, 9] = wb[row0 + nrows - 1, K - 3] = 0x4500        # escapes inside the range
+    w = enc(ops, wb, NIB, 0, False, False)
+    x = tbf16(synth.activations(T, K, 992))
+    whole = ops.mmv(x, w)
+    assert ops.last_kernel().startswith("k_nib_mm16<" if T <= 16 else "k_nib_mm<")
+    y = torch.full((T, nrows), float("nan"), dtype=torch.float32, device="cuda")
+    a = _lib.MmvArgs()
+    a.x, a.y, a.ids = x.data_ptr(), y.data_ptr(), None
+    a.x_tok, a.y_tok = K * 2, nrows * 4
+    a.rows_per_matrix, a.row0, a.nrows, a.ncols = rows, row0, nrows, T
+    a.x_bf16, a.y_bf16 = 1, 0
+    _lib.check(_lib.lib().bf16n_mmv(C.byref(ops._cweight(w)), C.byref(a), C.c_void_p(torch.cuda.current_stream().cuda_stream), 1))
+    torch.cuda.synchronize()
+    took = ops.last_kernel()
+    # (six tokens: 16-row groups for the tensor and for the range; 70 tokens, five blocks of 16, are more than two
+    # blocks per CU for either: 32-row groups)
+    assert took.startswith("k_nib_mm16<" if T <= 16 else "k_nib_mm<"), took
+    assert torch.equal(y, whole[:, row0: row0 + nrows])
+
+
 @pytest.mark.parametrize("fmt,R,cm,w64", LAYOUTS)
 def test_one_hot_activations_give_exact_weights(ops, fmt, R, cm, w64):
     K, rows = 2048, 64
